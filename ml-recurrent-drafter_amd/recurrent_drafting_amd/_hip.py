@@ -1,0 +1,81 @@
+"""ctypes binding of libredrafter_hip.so (the C ABI declared in include/redrafter_hip.h).
+
+PyTorch is used only for device memory and streams: tensors are handed over as raw device pointers
+plus sizes/strides, and every launch goes to torch's current HIP stream.  There is no fallback: if
+the library is missing, or a tensor is not on the GPU, the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libredrafter_hip.so")
+_lib = None
+
+RD_BF16, RD_F16, RD_F32 = 0, 1, 2
+_DTYPES = {torch.bfloat16: RD_BF16, torch.float16: RD_F16, torch.float32: RD_F32}
+
+_P, _I, _L, _Z, _F = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
+
+_PROTOTYPES = {
+    "rd_version": (C.c_int, []),
+    "rd_last_error": (C.c_char_p, []),
+    "rd_tree_workspace_bytes": (_Z, [_I, _I, _I]),
+    "rd_tree_build": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "rd_tree_mask": (_I, [_P, _P, _P, _P, _I, _L, _L, _I, _I, _I, _P, _P]),
+}
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def lib():
+    """Loads the shared library on first use."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build it with "
+                "`python ml-recurrent-drafter_amd/build_hip.py` (needs hipcc); "
+                "there is no CPU or PyTorch fallback for the HIP kernels"
+            )
+        handle = C.CDLL(_LIB_PATH)
+        for name, (res, args) in _PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = lib().rd_last_error().decode()
+        raise RuntimeError(f"libredrafter_hip error {rc}: {msg}")
+
+
+def ptr(t: torch.Tensor | None):
+    """Device pointer of a tensor (None -> NULL).  Refuses host tensors: the kernels would fault."""
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise RuntimeError(
+            "the HIP hot path needs tensors on the GPU (got a CPU tensor); "
+            "there is no CPU fallback in this package"
+        )
+    return t.data_ptr()
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPES[dt]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dt}; expected bfloat16, float16 or float32") from None

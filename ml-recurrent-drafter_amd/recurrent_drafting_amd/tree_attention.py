@@ -1,0 +1,112 @@
+"""Tree attention on the GPU: draft beams -> prefix tree -> packed tokens, mask and unpacker.
+
+Same call surface as the reference's recurrent_drafting/tree_attention.py (`pack`, `unpack` and the
+underscore helpers its tests use); the work is done by the HIP kernels behind rd_tree_build,
+rd_tree_mask and rd_unpack_rows.  One device-to-host read (the packed length) per `pack`, where the
+reference has two (tree_attention.py:78 and :99).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import _hip
+
+
+@dataclass
+class PackedTree:
+    """Everything one `pack` produces; `pack()` returns the reference's 4-tuple view of it."""
+
+    packed_beams: torch.Tensor  # (B, n) int64
+    unpacker: torch.Tensor  # (B, W, L) int64
+    packed_token_indices: torch.Tensor  # (B, n) int64, flat index beam*L+pos of each packed slot
+    position_offsets: torch.Tensor  # (B, n) int64
+    prefix_tree: torch.Tensor  # (B, W, L) int64
+    counts: torch.Tensor  # (B+2,) int32 on device: per-row count, max, total
+    n: int  # packed length (max over rows), host value
+
+
+def _check_beams(beams: torch.Tensor) -> Tuple[int, int, int]:
+    assert beams.dim() == 3, f"beams must be (batch, beam_width, beam_length), got {tuple(beams.shape)}"
+    assert beams.dtype == torch.long, f"beams.dtype {beams.dtype} is not long"
+    return tuple(beams.shape)  # type: ignore[return-value]
+
+
+def build_tree(beams: torch.Tensor) -> PackedTree:
+    """Dedup + unpacker + pack + position offsets in two launches (tree_attention.py:331-335)."""
+    B, W, L = _check_beams(beams)
+    beams = beams.contiguous()
+    dev = beams.device
+    n_tok = B * W * L
+    slab = torch.empty((5, n_tok), dtype=torch.long, device=dev)
+    counts = torch.empty(B + 2, dtype=torch.int32, device=dev)
+    lib = _hip.lib()
+    ws_bytes = lib.rd_tree_workspace_bytes(B, W, L)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    _hip.check(
+        lib.rd_tree_build(
+            _hip.ptr(beams), B, W, L,
+            _hip.ptr(slab[0]), _hip.ptr(slab[1]), _hip.ptr(slab[2]), _hip.ptr(slab[3]),
+            _hip.ptr(slab[4]), _hip.ptr(counts), _hip.ptr(ws), ws_bytes, _hip.stream(),
+        )
+    )
+    n = int(counts[B].item())  # the one host read; shapes below depend on it
+    return PackedTree(
+        packed_beams=slab[2, : B * n].view(B, n),
+        unpacker=slab[1].view(B, W, L),
+        packed_token_indices=slab[3, : B * n].view(B, n),
+        position_offsets=slab[4, : B * n].view(B, n),
+        prefix_tree=slab[0].view(B, W, L),
+        counts=counts,
+        n=n,
+    )
+
+
+def build_mask(tree: PackedTree, padding_mask: torch.Tensor) -> torch.Tensor:
+    """(B, n, prev+n) bool mask of the packed rows (tree_attention.py:336-337)."""
+    B, W, L = tree.unpacker.shape
+    assert padding_mask.dim() == 2 and padding_mask.shape[0] == B
+    assert padding_mask.dtype in (torch.int32, torch.int64, torch.bool, torch.uint8)
+    prev = padding_mask.shape[1]
+    if prev > 0 and padding_mask.stride(1) != 1:
+        padding_mask = padding_mask.contiguous()
+    n = tree.n
+    out = torch.empty((B, n, prev + n), dtype=torch.bool, device=tree.unpacker.device)
+    _hip.check(
+        _hip.lib().rd_tree_mask(
+            _hip.ptr(tree.unpacker), _hip.ptr(tree.packed_token_indices), _hip.ptr(tree.counts),
+            _hip.ptr(padding_mask) if prev > 0 else None, padding_mask.element_size(),
+            padding_mask.stride(0) if prev > 0 else 0, prev, B, W, L, _hip.ptr(out), _hip.stream(),
+        )
+    )
+    return out
+
+
+def pack(
+    beams: torch.Tensor, padding_mask: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(packed_beams (B,n), unpacker (B,W,L), causal_mask (B,n,prev+n) bool, position_offsets (B,n)).
+
+    Drop-in for tree_attention.pack (tree_attention.py:301-338)."""
+    tree = build_tree(beams)
+    mask = build_mask(tree, padding_mask)
+    return tree.packed_beams, tree.unpacker, mask, tree.position_offsets
+
+
+# The reference's tests call these helpers directly; they are thin views of the fused kernels.
+def _dedup_prefix(beams: torch.Tensor) -> torch.Tensor:
+    return build_tree(beams).prefix_tree
+
+
+def _get_unpacker(beams: torch.Tensor, prefix_tree: Optional[torch.Tensor] = None) -> torch.Tensor:
+    return build_tree(beams).unpacker
+
+
+def _pack_beams(
+    beams: torch.Tensor, prefix_tree: Optional[torch.Tensor] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    t = build_tree(beams)
+    return t.packed_beams, t.packed_token_indices

@@ -1,0 +1,110 @@
+"""GPU parity: rd_tree_build / rd_tree_mask through the C ABI vs the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import tree_oracle as T
+
+pytestmark = pytest.mark.gpu
+
+A = lambda x: np.asarray(x, dtype=np.int64)  # noqa: E731
+
+
+def _dev(x, dtype=torch.long):
+    return torch.tensor(np.asarray(x), dtype=dtype, device="cuda")
+
+
+def _check_against_oracle(beams, padding_mask):
+    from recurrent_drafting_amd import tree_attention
+
+    tok, unp, mask, off, idx = T.pack(beams, padding_mask)
+    tree = tree_attention.build_tree(_dev(beams))
+    assert np.array_equal(tree.prefix_tree.cpu().numpy(), T.dedup_prefix(beams))
+    assert tree.n == tok.shape[1]
+    assert np.array_equal(tree.packed_beams.cpu().numpy(), tok)
+    assert np.array_equal(tree.packed_token_indices.cpu().numpy(), idx)
+    assert np.array_equal(tree.unpacker.cpu().numpy(), unp)
+    assert np.array_equal(tree.position_offsets.cpu().numpy(), off)
+    for dt in (torch.long, torch.int32, torch.bool):
+        g_tok, g_unp, g_mask, g_off = tree_attention.pack(_dev(beams), _dev(padding_mask, dt))
+        assert g_mask.dtype == torch.bool and g_mask.shape == mask.shape
+        assert np.array_equal(g_mask.cpu().numpy(), mask)
+        assert np.array_equal(g_tok.cpu().numpy(), tok) and np.array_equal(g_off.cpu().numpy(), off)
+
+
+def test_reference_literals(literals):
+    t = literals["tree"]
+    for case in literals["pack_masks"]["cases"]:
+        _check_against_oracle(A(t["beams"]), A(case["padding_mask"]))
+    c = literals["no_common_prefix"]
+    for case in c["cases"]:
+        _check_against_oracle(A(c["beams"]), np.ones((1, case["prompt_len"]), dtype=np.int64))
+
+
+def test_reference_literal_values_directly(literals):
+    """Reads like the reference's test_pack: outputs equal the literals, no oracle in between."""
+    from recurrent_drafting_amd import tree_attention
+
+    t = literals["tree"]
+    for case in literals["pack_masks"]["cases"]:
+        tok, unp, mask, off = tree_attention.pack(_dev(t["beams"]), _dev(case["padding_mask"]))
+        assert tok.cpu().tolist() == t["packed_beams"]
+        assert unp.cpu().tolist() == t["unpacker"]
+        assert mask.cpu().to(torch.long).tolist() == case["mask"]
+        assert off.cpu().tolist() == t["position_offsets"]
+    p, i = tree_attention._pack_beams(_dev(t["beams"]))
+    assert p.cpu().tolist() == t["packed_beams"] and i.cpu().tolist() == t["packed_token_indices"]
+    assert tree_attention._dedup_prefix(_dev(t["beams"])).cpu().tolist() == t["prefix_tree"]
+
+
+def test_reference_vectors(ref_vectors):
+    for c in ref_vectors["pack"]:
+        beams = A(c["beams"])
+        _check_against_oracle(beams, A(c["padding_mask"]).reshape(beams.shape[0], -1))
+
+
+@pytest.mark.parametrize("B,W,L,vocab,prev", [
+    (1, 1, 2, 3, 0), (2, 3, 4, 2, 5), (4, 7, 5, 3, 17), (8, 45, 5, 4, 33), (3, 64, 5, 5, 100),
+    (5, 13, 13, 2, 1), (16, 64, 5, 6, 64), (2, 128, 32, 2, 7),
+])
+def test_random_shapes(B, W, L, vocab, prev):
+    rng = np.random.default_rng(B * 1000 + W * 10 + L)
+    beams = rng.integers(0, vocab, size=(B, W, L))
+    pm = (rng.random((B, prev)) > 0.2).astype(np.int64)
+    _check_against_oracle(beams, pm)
+
+
+def test_benchmark_config_full_size():
+    """Config 2: (8,45,5) beams with shared prefixes, prev 0 and prev 2548."""
+    beams = T.synthetic_beams(8, 45, 5, seed=123)
+    _check_against_oracle(beams, np.zeros((8, 0), dtype=np.int64))
+    rng = np.random.default_rng(1)
+    pm = np.ones((8, 2548), dtype=np.int64)
+    for b in range(8):
+        pm[b, : rng.integers(0, 2048)] = 0
+    pm[rng.random(pm.shape) < 0.001] = 0  # a few pad-valued tokens inside the live region
+    _check_against_oracle(beams, pm)
+
+
+def test_replicated_batch_invariants():
+    """x64 replicated batch (512 rows): packed[unpacker] == beams, counts == distinct prefixes."""
+    from recurrent_drafting_amd import tree_attention
+
+    beams = np.concatenate([T.synthetic_beams(8, 45, 5, seed=s) for s in range(64)], axis=0)
+    tree = tree_attention.build_tree(_dev(beams))
+    packed = tree.packed_beams.cpu().numpy()
+    unp = tree.unpacker.cpu().numpy()
+    assert np.array_equal(np.take_along_axis(packed, unp.reshape(512, -1), axis=1).reshape(beams.shape), beams)
+    counts = tree.counts.cpu().numpy()
+    tok, _, n_sel = T.pack_beams(beams, T.dedup_prefix(beams))
+    assert np.array_equal(counts[:512], n_sel) and counts[512] == n_sel.max() and counts[513] == n_sel.sum()
+    assert np.array_equal(packed, tok)
+
+
+def test_limits_raise():
+    from recurrent_drafting_amd import tree_attention
+
+    with pytest.raises(RuntimeError, match="width"):
+        tree_attention.build_tree(torch.zeros((1, 2048, 2), dtype=torch.long, device="cuda"))
+    with pytest.raises(AssertionError):
+        tree_attention.build_tree(torch.zeros((1, 4, 2), dtype=torch.int32, device="cuda"))
