@@ -81,6 +81,83 @@ RD_API int rd_tree_mask(const int64_t* unpacker, const int64_t* packed_token_ind
                  int64_t pm_row_stride, int64_t prev, int batch, int width, int length,
                  uint8_t* mask, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Row gather: out[b, t, :] = packed[b, index[b, t], :], t in [0, n_out).
+ * Replaces tree_attention.unpack (tree_attention.py:341-387) for hidden states and logits, and
+ * _select_one_per_row gathers (recurrent_drafting.py:37-40) when n_out == 1.
+ * Rows are row_bytes long; batch strides are in bytes (packed) / elements (index).  An index
+ * outside [0, n_src) leaves its output row untouched.
+ * ------------------------------------------------------------------------------------------ */
+RD_API int rd_unpack_rows(const void* packed, int64_t packed_batch_stride_bytes, int64_t row_bytes,
+                          const int64_t* index, int64_t index_batch_stride, int batch, int n_out,
+                          int n_src, void* out, int64_t out_batch_stride_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * First maximal index of every row of a (rows, vocab) matrix; NaN counts as the largest value.
+ * Replaces torch.argmax(logits_by_llm, dim=-1) (recurrent_drafting.py:52, :425).
+ * row_stride in elements.
+ * ------------------------------------------------------------------------------------------ */
+RD_API int rd_argmax_rows(const void* x, int dtype, int64_t rows, int64_t vocab, int64_t row_stride,
+                          int64_t* out, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Greedy acceptance.  Replaces _greedy_choose_from_candidates (recurrent_drafting.py:468-496) and
+ * the token half of _greedy_prepare_next_input (:261-263).
+ *
+ * beams (batch,width,length): drafted tokens, position 0 is the LLM's own token.
+ * llm_tokens: the LLM's argmax per candidate position.  With unpacker == NULL it is laid out
+ * (batch,width,length) with row stride llm_row_stride; otherwise it is indexed per PACKED slot,
+ * llm_tokens[b*llm_row_stride + unpacker[b,i,k]], which skips the unpack of the logits.
+ * Outputs (batch,): n_tokens_in_seq, seq_in_beam (first beam with the longest match), and
+ * optionally next_token = llm[b, seq, n] and last_slot = the index of that position (packed slot
+ * when unpacker is given, else seq*length+n) for gathering the drafter context.
+ * ------------------------------------------------------------------------------------------ */
+RD_API int rd_accept_greedy(const int64_t* beams, const int64_t* llm_tokens, int64_t llm_row_stride,
+                            const int64_t* unpacker, int batch, int width, int length,
+                            int64_t* n_tokens_in_seq, int64_t* seq_in_beam, int64_t* next_token,
+                            int64_t* last_slot, void* stream);
+
+/* Leading pad run per row.  Replaces _count_left_paddings (recurrent_drafting.py:387-388). */
+RD_API int rd_count_left_paddings(const int64_t* input_ids, int64_t ids_row_stride, int64_t prev,
+                                  int batch, int64_t pad_token_id, int32_t* pads, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Token ids after acceptance, right-aligned and left-padded, plus the per-row plan that
+ * rd_kv_compact follows.  Replaces the integer half of _update_kv_cache_and_input_ids
+ * (recurrent_drafting.py:163-171, :211-226).
+ *
+ * plan: rd_realign_plan_ints(batch, length) int32: [0] = new length M (max over rows), [1] = prev,
+ * [2] = length, [3] = 0, then per row {old_pads, new_pads, n_new, live_len, src_row[length]} where
+ * src_row[j] is the cache row holding accepted token j: prev + seq*length + j when unpacker is
+ * NULL (cache already unpacked by rd_kv_unpack), prev + unpacker[b,seq,j] otherwise.
+ * new_ids: capacity batch*(prev+length), written as a contiguous (batch, M) array.
+ * ------------------------------------------------------------------------------------------ */
+RD_API size_t rd_realign_plan_ints(int batch, int length);
+RD_API int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride, int64_t prev,
+                           const int64_t* n_tokens_in_seq, const int64_t* seq_in_beam,
+                           const int64_t* beams, const int64_t* unpacker, int batch, int width,
+                           int length, int64_t pad_token_id, int32_t* plan, int64_t* new_ids,
+                           void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * KV cache, shape (n_layers, 2, batch, n_heads, max_len, head_dim), rows of row_bytes bytes.
+ *
+ * rd_kv_unpack: cache[..., prev+t, :] = cache[..., prev+index[b,t], :] for t in [0, n_out), all
+ * reads before any write.  Replaces Cache.unpack (kv_cache.py:58-98).  n_src = number of packed
+ * rows present at [prev, prev+n_src).
+ *
+ * rd_kv_compact: in place, per (layer, k|v, row, head): live rows [old_pads, prev) move to
+ * [new_pads, ...) and the accepted rows src_row[0..n_new) follow them.  Replaces the cache half of
+ * _update_kv_cache_and_input_ids (recurrent_drafting.py:174-209).  Rows outside [new_pads, M) keep
+ * stale data (the reference leaves other stale data there).
+ * ------------------------------------------------------------------------------------------ */
+RD_API int rd_kv_unpack(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
+                        int64_t row_bytes, int64_t prev, const int64_t* index, int n_out, int n_src,
+                        void* stream);
+RD_API int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
+                         int64_t row_bytes, int64_t prev, int length, const int32_t* plan,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

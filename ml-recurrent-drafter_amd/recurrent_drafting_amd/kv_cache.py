@@ -1,0 +1,105 @@
+"""Pre-allocated KV cache with the reference's View/Cache objects (recurrent_drafting/kv_cache.py).
+
+One dense tensor (n_layers, 2, batch, n_heads, max_length, head_dim) lives in HBM for the whole
+generation; `View.cat` appends in place and hands back a strided view, `Cache.unpack` and
+`Cache.compact` move rows with the HIP kernels rd_kv_unpack / rd_kv_compact (in place, no clone).
+"""
+
+from __future__ import annotations
+
+from typing import Tuple
+
+import torch
+
+from . import _hip
+
+
+class View:
+    """Key or value rows of one layer: cache[layer, kv, :, :, 0:length, :] (kv_cache.py:10-35)."""
+
+    def __init__(self, cache: torch.Tensor, layer: int, kv: int):
+        self._cache = cache
+        self._layer = layer
+        self._kv = kv  # 0 = key, 1 = value
+        self.length = 0
+
+    @property
+    def shape(self) -> Tuple[int, int, int, int]:
+        _, _, batch_size, n_heads, _, head_dim = self._cache.shape
+        return (batch_size, n_heads, self.length, head_dim)
+
+    def cat(self, new_kv: torch.Tensor) -> torch.Tensor:
+        """Appends (batch, n_heads, n_new, head_dim) rows in place and returns rows [0, length)."""
+        _, _, batch_size, n_heads, max_length, head_dim = self._cache.shape
+        n_new = new_kv.shape[2]
+        assert new_kv.shape == (batch_size, n_heads, n_new, head_dim)
+        assert self.length + n_new <= max_length
+        slab = self._cache[self._layer, self._kv]
+        slab[:, :, self.length : self.length + n_new, :] = new_kv
+        self.length += n_new
+        return slab[:, :, : self.length, :]
+
+    def slice(self, prev: int) -> torch.Tensor:
+        """Rows [prev, length)."""
+        return self._cache[self._layer, self._kv, :, :, prev : self.length, :]
+
+
+class Cache:
+    def __init__(
+        self,
+        batch_size: int,
+        max_length: int,
+        n_layers: int,
+        n_heads: int,
+        head_dim: int,
+        dtype: torch.dtype,
+        device: torch.device,
+    ) -> None:
+        self._cache = torch.zeros(
+            [n_layers, 2, batch_size, n_heads, max_length, head_dim], dtype=dtype, device=device
+        )
+        self.sliced = tuple(
+            (View(self._cache, layer, 0), View(self._cache, layer, 1)) for layer in range(n_layers)
+        )
+
+    # -- geometry handed to the C ABI ---------------------------------------------------------
+    def _geometry(self):
+        n_layers, _, batch, n_heads, max_len, head_dim = self._cache.shape
+        return n_layers, batch, n_heads, max_len, head_dim * self._cache.element_size()
+
+    def set_length(self, length: int) -> None:
+        for key, value in self.sliced:
+            key.length = value.length = length
+
+    def unpack(self, prompt_length: int, tree_attn_index: torch.Tensor) -> None:
+        """Every candidate position (beam, k) gets its own cache row behind the prompt:
+        row prompt_length + beam*L + k takes the packed row prompt_length + tree_attn_index[b,beam,k]
+        (kv_cache.py:58-98)."""
+        batch, width, length = tree_attn_index.shape
+        n_layers, cb, n_heads, max_len, row_bytes = self._geometry()
+        assert cb == batch
+        n_out = width * length
+        n_src = self.sliced[0][0].length - prompt_length
+        assert n_src > 0, "no packed rows behind the prompt"
+        assert prompt_length + n_out <= max_len
+        index = tree_attn_index.contiguous()
+        assert index.dtype == torch.long
+        _hip.check(
+            _hip.lib().rd_kv_unpack(
+                _hip.ptr(self._cache), n_layers, batch, n_heads, max_len, row_bytes, prompt_length,
+                _hip.ptr(index), n_out, n_src, _hip.stream(),
+            )
+        )
+        self.set_length(prompt_length + n_out)
+
+    def compact(self, prev: int, beam_length: int, plan: torch.Tensor, new_length: int) -> None:
+        """Follows a plan written by rd_realign_plan: accepted rows kept, rows re-right-aligned."""
+        n_layers, batch, n_heads, max_len, row_bytes = self._geometry()
+        assert plan.dtype == torch.int32
+        _hip.check(
+            _hip.lib().rd_kv_compact(
+                _hip.ptr(self._cache), n_layers, batch, n_heads, max_len, row_bytes, prev,
+                beam_length, _hip.ptr(plan), _hip.stream(),
+            )
+        )
+        self.set_length(new_length)

@@ -110,3 +110,33 @@ def _pack_beams(
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     t = build_tree(beams)
     return t.packed_beams, t.packed_token_indices
+
+
+def gather_rows(packed: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """out[b, t, :] = packed[b, index[b, t], :] for packed (B, n, F) and index (B, T) int64."""
+    assert packed.dim() == 3 and index.dim() == 2 and index.dtype == torch.long
+    B, n_src, F = packed.shape
+    T = index.shape[1]
+    assert index.shape[0] == B
+    if packed.stride(2) != 1 or packed.stride(1) != F:
+        packed = packed.contiguous()
+    index = index.contiguous()
+    out = torch.empty((B, T, F), dtype=packed.dtype, device=packed.device)
+    es = packed.element_size()
+    _hip.check(
+        _hip.lib().rd_unpack_rows(
+            _hip.ptr(packed), packed.stride(0) * es, F * es, _hip.ptr(index), T, B, T, n_src,
+            _hip.ptr(out), T * F * es, _hip.stream(),
+        )
+    )
+    return out
+
+
+def unpack(packed_tensor: torch.Tensor, unpacker: torch.Tensor) -> torch.Tensor:
+    """(B, n, F) packed rows -> (B, W, L, F) as if every beam had been verified on its own.
+
+    Drop-in for tree_attention.unpack (tree_attention.py:341-387)."""
+    assert len(packed_tensor.shape) == 3
+    B, W, L = unpacker.shape
+    out = gather_rows(packed_tensor, unpacker.reshape(B, W * L))
+    return out.view(B, W, L, packed_tensor.shape[2])
