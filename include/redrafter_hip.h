@@ -158,6 +158,75 @@ RD_API int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, int6
                          int64_t row_bytes, int64_t prev, int length, const int32_t* plan,
                          void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Verification attention.
+ *
+ * rd_attn_prepare: once per LLM forward (where the reference builds the additive bias,
+ * modeling_llama.py:228 / attention.py:75-88).  Compresses the bool mask (batch, n_q, kv_len),
+ * given as 0/1 bytes with element strides mask_stride_b / mask_stride_q (keys contiguous), into
+ * bits: rd_attn_bits_words() uint64, one word per (row, 64 keys); and writes the work plan
+ * (rd_attn_plan_ints() int32): per batch row the first key any query attends to and the split of
+ * its keys into work items.  fix_empty_rows != 0 turns a row that attends to nothing into a row
+ * that attends to everything, which is what attention.set_sdpa_fully_masked_rows
+ * (attention.py:58-72) does and what a finite-minimum additive bias amounts to.
+ *
+ * rd_verify_attention: out = softmax(q k^T * scale, masked) v per (batch row, head).  Replaces
+ * repeat_interleave + F.scaled_dot_product_attention(attn_mask=bias) (modeling_llama.py:161-169).
+ * q (batch, n_heads, n_q, head_dim), k/v (batch, n_kv_heads, kv_len, head_dim) and out
+ * (batch, n_heads, n_q, head_dim) are addressed through HOST arrays of three element strides
+ * {batch, head, sequence}; the last dimension is contiguous.  k and v are normally the strided
+ * views View.cat returns (kv_cache.py:24-31).  bf16 with head_dim 128 runs on the MFMA kernel
+ * (needs 16-byte aligned q/k/v, strides that are multiples of 8 elements, and the workspace);
+ * everything else, or force_generic != 0, runs on the generic kernel (head_dim <= 256).
+ * ------------------------------------------------------------------------------------------ */
+RD_API size_t rd_attn_plan_ints(int batch, int n_q, int kv_len);
+RD_API size_t rd_attn_bits_words(int batch, int n_q, int kv_len);
+RD_API int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64_t mask_stride_q,
+                           int batch, int n_q, int kv_len, int fix_empty_rows, uint64_t* bits,
+                           int32_t* plan, void* stream);
+RD_API size_t rd_attention_workspace_bytes(int batch, int n_heads, int n_q, int kv_len,
+                                           int head_dim);
+RD_API int rd_verify_attention(const void* q, const int64_t* q_strides, const void* k,
+                               const int64_t* k_strides, const void* v, const int64_t* v_strides,
+                               void* out, const int64_t* o_strides, int dtype, int batch,
+                               int n_heads, int n_kv_heads, int n_q, int kv_len, int head_dim,
+                               float scale, const uint64_t* bits, const int32_t* plan,
+                               void* workspace, size_t workspace_bytes, int force_generic,
+                               void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Causal mask from a padding mask: mask[b,i,j] = (j <= kv_len - query_len + i) && padding[b,j].
+ * Replaces attention.causal_mask (attention.py:12-55) without the (kv_len, kv_len) temporary.
+ * padding_mask as in rd_tree_mask; mask is (batch, query_len, kv_len) 0/1 bytes, contiguous.
+ * ------------------------------------------------------------------------------------------ */
+RD_API int rd_causal_mask(const void* padding_mask, int pm_elem_bytes, int64_t pm_row_stride,
+                          int batch, int64_t kv_len, int64_t query_len, uint8_t* mask,
+                          void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * One beam-search iteration after the drafter's lm_head GEMM.
+ * Replaces maintain_logits (modeling_drafter.py:63-77), warp_logits (:80-99), log_softmax,
+ * the beam-score add, torch.topk over width*vocab, % and // (:201-215), and the beams gather +
+ * cat (:218-220).  Equal scores are ordered by the lower flat index beam*vocab + token
+ * (torch.topk leaves that order unspecified).
+ *
+ * logits (batch*width, vocab) of `dtype`, row stride in elements, rows 16-byte aligned.
+ * log_p_beam (batch,width) f32: running beam scores.  top_k / mask_value: 50 / -50000 upstream.
+ * Outputs: new_log_p_beam (batch,width) f32 sorted descending, tokens and parents (batch,width).
+ * beams_out (batch,width,t_len+1), optional: beams_in (batch,width,t_len) gathered by parent with
+ * the new token appended.  logp_out, optional: (batch*width, vocab) f32 log-probabilities of the
+ * new token under each INPUT beam (rounded through `dtype` as upstream), row stride in elements.
+ * Limits: width <= 64, vocab <= 65536, top_k <= 512.  force_fallback != 0 runs the slow exact
+ * path that otherwise only serves rows with very many tied logits.
+ * ------------------------------------------------------------------------------------------ */
+RD_API size_t rd_beam_topk_workspace_bytes(int batch, int width);
+RD_API int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, int batch, int width,
+                        int vocab, const float* log_p_beam, int top_k, float mask_value,
+                        const int64_t* beams_in, int t_len, float* new_log_p_beam, int64_t* tokens,
+                        int64_t* parents, int64_t* beams_out, float* logp_out,
+                        int64_t logp_row_stride, void* workspace, size_t workspace_bytes,
+                        int force_fallback, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

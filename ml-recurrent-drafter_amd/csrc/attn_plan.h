@@ -1,0 +1,21 @@
+// Layout of the attention plan shared by the planning and the attention kernels.
+//
+// plan (int32):
+//   [0] n_items  [1] n_q  [2] kv_len  [3] words per mask row  [4] max_splits  [5] chunk  [6..7] 0
+//   per batch row b, 4 ints at RD_PLAN_HDR + 4*b:  {kv_begin, n_splits, first_item, 0}
+//   items, 4 ints each at RD_PLAN_HDR + 4*batch:   {b, kv_lo, kv_hi, split}  (longest first)
+//   scratch: first attended key of every (b, q) row
+#pragma once
+
+#include "rd_common.h"
+
+#define RD_PLAN_HDR 8
+
+namespace rd {
+
+constexpr int kAttnChunk = 512;       // target keys per work item
+constexpr int kAttnSortLimit = 2048;  // more items than this are dispatched unsorted
+
+inline int attn_max_splits(int kv_len) { return (kv_len + kAttnChunk - 1) / kAttnChunk; }
+
+}  // namespace rd

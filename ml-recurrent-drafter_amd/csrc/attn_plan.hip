@@ -1,0 +1,159 @@
+// Mask compression and work planning for the verification attention (gfx950).
+//   mask_bits_kernel   bool mask (batch, n_q, kv) -> one uint64 per (row, 64 keys); a wave reads 64
+//                      mask bytes coalesced and a ballot turns them into the word
+//   attn_plan_kernel   per batch row: first key any query attends to (whole 64-key tiles of left
+//                      padding are never loaded), split of the remaining keys into near-equal
+//                      chunks, and the chunk list sorted longest-first for dispatch
+#include "attn_plan.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+
+__global__ __launch_bounds__(kThreads) void mask_bits_kernel(
+    const uint8_t* __restrict__ mask, int64_t stride_b, int64_t stride_q, int n_q, int kv_len,
+    int words, int fix_empty_rows, uint64_t* __restrict__ bits, int32_t* __restrict__ row_first) {
+  const int q = blockIdx.x, b = blockIdx.y;
+  const uint8_t* row = mask + (int64_t)b * stride_b + (int64_t)q * stride_q;
+  uint64_t* out = bits + ((int64_t)b * n_q + q) * words;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int first = kv_len;
+  for (int w = wave; w < words; w += kWaves) {
+    const int j = w * 64 + lane;
+    const bool on = j < kv_len && row[j] != 0;
+    const uint64_t word = __ballot(on);
+    if (lane == 0) out[w] = word;
+    if (word != 0) {
+      const int f = w * 64 + __builtin_ctzll(word);
+      first = f < first ? f : first;
+    }
+  }
+  __shared__ int s_first[kWaves];
+  if (lane == 0) s_first[wave] = first;
+  __syncthreads();
+  first = kv_len;
+  for (int w = 0; w < kWaves; ++w) first = s_first[w] < first ? s_first[w] : first;
+  if (first == kv_len && fix_empty_rows) {
+    // a query that attends to nothing attends to everything (finite-minimum bias semantics)
+    for (int w = threadIdx.x; w < words; w += kThreads) {
+      const int rem = kv_len - w * 64;
+      out[w] = rem >= 64 ? ~0ull : ((1ull << rem) - 1ull);
+    }
+    first = 0;
+  }
+  if (threadIdx.x == 0) row_first[(int64_t)b * n_q + q] = first;
+}
+
+__global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __restrict__ row_first,
+                                                             int B, int n_q, int kv_len, int words,
+                                                             int chunk, int max_splits,
+                                                             int32_t* __restrict__ plan) {
+  __shared__ int s_n_items;
+  int32_t* per_row = plan + RD_PLAN_HDR;
+  int32_t* items = plan + RD_PLAN_HDR + 4 * B;
+  // pass 1: per batch row, first attended key and number of splits
+  for (int b = threadIdx.x; b < B; b += kThreads) {
+    int first = kv_len;
+    for (int q = 0; q < n_q; ++q) {
+      const int f = row_first[(int64_t)b * n_q + q];
+      first = f < first ? f : first;
+    }
+    const int begin = (first / 64) * 64;
+    const int live = kv_len - begin;
+    int splits = (live + chunk - 1) / chunk;
+    splits = splits < 1 ? 1 : (splits > max_splits ? max_splits : splits);
+    per_row[4 * b + 0] = begin;
+    per_row[4 * b + 1] = splits;
+    per_row[4 * b + 3] = 0;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int n = 0;
+    for (int b = 0; b < B; ++b) {
+      per_row[4 * b + 2] = n;  // first item of this row (before sorting)
+      n += per_row[4 * b + 1];
+    }
+    s_n_items = n;
+    plan[0] = n; plan[1] = n_q; plan[2] = kv_len; plan[3] = words;
+    plan[4] = max_splits; plan[5] = chunk; plan[6] = 0; plan[7] = 0;
+  }
+  __syncthreads();
+  const int n_items = s_n_items;
+  // pass 2: every item computes its own extent and its rank (longest first, ties by index)
+  auto extent = [&](int it, int& b, int& s, int& lo, int& hi) {
+    b = 0;
+    while (b + 1 < B && per_row[4 * (b + 1) + 2] <= it) ++b;
+    s = it - per_row[4 * b + 2];
+    const int begin = per_row[4 * b + 0], splits = per_row[4 * b + 1];
+    const int live = kv_len - begin;
+    int per = (live + splits - 1) / splits;
+    per = (per + 63) / 64 * 64;
+    lo = begin + s * per;
+    hi = lo + per;
+    lo = lo < kv_len ? lo : kv_len;
+    hi = hi < kv_len ? hi : kv_len;
+  };
+  __shared__ int s_len[rd::kAttnSortLimit];
+  const bool sorted = n_items <= rd::kAttnSortLimit;
+  if (sorted) {
+    for (int it = threadIdx.x; it < n_items; it += kThreads) {
+      int b, s, lo, hi;
+      extent(it, b, s, lo, hi);
+      s_len[it] = hi - lo;
+    }
+  }
+  __syncthreads();
+  for (int it = threadIdx.x; it < n_items; it += kThreads) {
+    int b, s, lo, hi;
+    extent(it, b, s, lo, hi);
+    int rank = it;
+    if (sorted) {
+      const int len = hi - lo;
+      rank = 0;
+      for (int o = 0; o < n_items; ++o) {
+        const int olen = s_len[o];
+        rank += (olen > len) || (olen == len && o < it);
+      }
+    }
+    items[4 * rank + 0] = b;
+    items[4 * rank + 1] = lo;
+    items[4 * rank + 2] = hi;
+    items[4 * rank + 3] = s;
+  }
+}
+
+}  // namespace
+
+extern "C" size_t rd_attn_plan_ints(int batch, int n_q, int kv_len) {
+  if (batch <= 0 || n_q <= 0 || kv_len <= 0) return 0;
+  const int max_splits = rd::attn_max_splits(kv_len);
+  return RD_PLAN_HDR + 4 * (size_t)batch + 4 * (size_t)batch * max_splits + (size_t)batch * n_q;
+}
+
+extern "C" size_t rd_attn_bits_words(int batch, int n_q, int kv_len) {
+  if (batch <= 0 || n_q <= 0 || kv_len <= 0) return 0;
+  return (size_t)batch * n_q * ((kv_len + 63) / 64);
+}
+
+extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64_t mask_stride_q,
+                               int batch, int n_q, int kv_len, int fix_empty_rows, uint64_t* bits,
+                               int32_t* plan, void* stream) {
+  RD_REQUIRE(batch > 0 && n_q > 0 && kv_len > 0, RD_EINVAL,
+             "rd_attn_prepare: bad sizes (batch %d n_q %d kv_len %d)", batch, n_q, kv_len);
+  RD_REQUIRE(batch <= 65535 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
+             "rd_attn_prepare: batch %d too large for kv_len %d", batch, kv_len);
+  RD_REQUIRE(mask && bits && plan, RD_EINVAL, "rd_attn_prepare: null pointer");
+  RD_REQUIRE(mask_stride_q >= kv_len && mask_stride_b >= 0, RD_EINVAL,
+             "rd_attn_prepare: mask_stride_q %lld < kv_len %d", (long long)mask_stride_q, kv_len);
+  const int words = (kv_len + 63) / 64;
+  const int max_splits = rd::attn_max_splits(kv_len);
+  int32_t* row_first = plan + RD_PLAN_HDR + 4 * (size_t)batch + 4 * (size_t)batch * max_splits;
+  hipStream_t s = rd::as_stream(stream);
+  hipLaunchKernelGGL(mask_bits_kernel, dim3(n_q, batch), dim3(kThreads), 0, s, mask, mask_stride_b,
+                     mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first);
+  if (int e = rd::check_launch("rd_attn_prepare(bits)")) return e;
+  hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 0, s, row_first, batch, n_q, kv_len,
+                     words, rd::kAttnChunk, max_splits, plan);
+  return rd::check_launch("rd_attn_prepare(plan)");
+}

@@ -177,7 +177,43 @@ __global__ __launch_bounds__(kThreads) void tree_mask_kernel(
   for (int64_t c = head + (nvec << 4) + threadIdx.x; c < row_len; c += kThreads) out[c] = value(c);
 }
 
+template <typename PM>
+__global__ __launch_bounds__(kThreads) void causal_mask_kernel(const PM* __restrict__ padding_mask,
+                                                              int64_t pm_row_stride, int64_t kv_len,
+                                                              int64_t query_len,
+                                                              uint8_t* __restrict__ mask) {
+  const int64_t i = blockIdx.x;
+  const int b = blockIdx.y;
+  const PM* pm = padding_mask + (int64_t)b * pm_row_stride;
+  uint8_t* out = mask + ((int64_t)b * query_len + i) * kv_len;
+  const int64_t last = kv_len - query_len + i;  // last key this query may attend to
+  for (int64_t j = threadIdx.x; j < kv_len; j += kThreads) out[j] = (j <= last) && (pm[j] != 0);
+}
+
 }  // namespace
+
+extern "C" int rd_causal_mask(const void* padding_mask, int pm_elem_bytes, int64_t pm_row_stride,
+                              int batch, int64_t kv_len, int64_t query_len, uint8_t* mask,
+                              void* stream) {
+  RD_REQUIRE(batch > 0 && kv_len > 0 && query_len > 0 && query_len <= kv_len, RD_EINVAL,
+             "rd_causal_mask: bad sizes (batch %d kv_len %lld query_len %lld)", batch,
+             (long long)kv_len, (long long)query_len);
+  RD_REQUIRE(batch <= 65535 && query_len <= 2147483647LL, RD_ELIMIT, "rd_causal_mask: too large");
+  RD_REQUIRE(padding_mask && mask, RD_EINVAL, "rd_causal_mask: null pointer");
+  RD_REQUIRE(pm_row_stride >= kv_len, RD_EINVAL, "rd_causal_mask: pm_row_stride < kv_len");
+  RD_REQUIRE(pm_elem_bytes == 1 || pm_elem_bytes == 4 || pm_elem_bytes == 8, RD_EINVAL,
+             "rd_causal_mask: pm_elem_bytes must be 1, 4 or 8 (got %d)", pm_elem_bytes);
+  hipStream_t s = rd::as_stream(stream);
+  const dim3 grid((unsigned)query_len, batch);
+#define RD_LAUNCH_CM(T)                                                                     \
+  hipLaunchKernelGGL(causal_mask_kernel<T>, grid, dim3(kThreads), 0, s,                      \
+                     reinterpret_cast<const T*>(padding_mask), pm_row_stride, kv_len, query_len, mask)
+  if (pm_elem_bytes == 1) RD_LAUNCH_CM(uint8_t);
+  else if (pm_elem_bytes == 4) RD_LAUNCH_CM(int32_t);
+  else RD_LAUNCH_CM(int64_t);
+#undef RD_LAUNCH_CM
+  return rd::check_launch("rd_causal_mask");
+}
 
 extern "C" size_t rd_tree_workspace_bytes(int batch, int width, int length) {
   if (batch <= 0 || width <= 0 || length <= 0) return 0;

@@ -34,6 +34,20 @@ _PROTOTYPES = {
     "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P]),
     "rd_kv_unpack": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _I, _I, _P]),
     "rd_kv_compact": (_I, [_P, _I, _I, _I, _L, _L, _L, _I, _P, _P]),
+    "rd_attn_plan_ints": (_Z, [_I, _I, _I]),
+    "rd_attn_bits_words": (_Z, [_I, _I, _I]),
+    "rd_attn_prepare": (_I, [_P, _L, _L, _I, _I, _I, _I, _P, _P, _P]),
+    "rd_attention_workspace_bytes": (_Z, [_I, _I, _I, _I, _I]),
+    "rd_verify_attention": (
+        _I,
+        [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P, _Z, _I, _P],
+    ),
+    "rd_causal_mask": (_I, [_P, _I, _L, _I, _L, _L, _P, _P]),
+    "rd_beam_topk_workspace_bytes": (_Z, [_I, _I]),
+    "rd_beam_topk": (
+        _I,
+        [_P, _I, _L, _I, _I, _I, _P, _I, _F, _P, _I, _P, _P, _P, _P, _P, _L, _P, _Z, _I, _P],
+    ),
 }
 
 

@@ -1,0 +1,124 @@
+"""Attention masks and the masked attention itself.
+
+`causal_mask`, `set_sdpa_fully_masked_rows` and `bias` keep the reference's signatures
+(recurrent_drafting/attention.py).  The model forward does not build an additive bias: it calls
+`prepare` once per forward (where the reference calls `bias`) and `masked_attention` per layer
+(where the reference calls F.scaled_dot_product_attention).
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import math
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _hip
+
+
+def causal_mask(padding_mask: torch.Tensor, query_len: int, device: torch.device) -> torch.Tensor:
+    """(batch, kv) padding mask -> (batch, query_len, kv) bool (attention.py:12-55)."""
+    assert padding_mask.dtype in [torch.int32, torch.int64, torch.bool]
+    assert query_len > 0
+    batch, kv_len = padding_mask.shape
+    if padding_mask.stride(1) != 1:
+        padding_mask = padding_mask.contiguous()
+    out = torch.empty((batch, query_len, kv_len), dtype=torch.bool, device=padding_mask.device)
+    _hip.check(
+        _hip.lib().rd_causal_mask(
+            _hip.ptr(padding_mask), padding_mask.element_size(), padding_mask.stride(0), batch,
+            kv_len, query_len, _hip.ptr(out), _hip.stream(),
+        )
+    )
+    return out
+
+
+def set_sdpa_fully_masked_rows(causal_mask: torch.Tensor) -> torch.Tensor:
+    """A row that attends to nothing attends to everything (attention.py:58-72)."""
+    assert causal_mask.dtype in [torch.int32, torch.int64, torch.bool]
+    dead = causal_mask.eq(0).all(dim=-1, keepdim=True)
+    return causal_mask.masked_fill(dead, True)
+
+
+def bias(causal_mask: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """0 where attended, finfo(dtype).min elsewhere (attention.py:75-88).  Kept for callers that
+    want the additive form; the HIP attention consumes the mask itself."""
+    out = torch.zeros(causal_mask.shape, dtype=dtype, device=causal_mask.device)
+    return out.masked_fill_(causal_mask.logical_not(), torch.finfo(dtype).min)
+
+
+@dataclass
+class PreparedMask:
+    """Bit-packed mask and work plan shared by every layer of one forward."""
+
+    bits: torch.Tensor  # (B, n_q, words) int64 holding uint64 words
+    plan: torch.Tensor  # int32
+    batch: int
+    n_q: int
+    kv_len: int
+    workspace: Optional[torch.Tensor] = None
+
+
+def prepare(mask: torch.Tensor, fix_empty_rows: bool = True) -> PreparedMask:
+    """mask: (B, n_q, kv_len) bool/uint8, keys contiguous."""
+    assert mask.dim() == 3 and mask.dtype in (torch.bool, torch.uint8)
+    if mask.stride(2) != 1:
+        mask = mask.contiguous()
+    B, n_q, kv_len = mask.shape
+    lib = _hip.lib()
+    dev = mask.device
+    bits = torch.empty(lib.rd_attn_bits_words(B, n_q, kv_len), dtype=torch.int64, device=dev)
+    plan = torch.empty(lib.rd_attn_plan_ints(B, n_q, kv_len), dtype=torch.int32, device=dev)
+    _hip.check(
+        lib.rd_attn_prepare(
+            _hip.ptr(mask), mask.stride(0), mask.stride(1), B, n_q, kv_len, int(fix_empty_rows),
+            _hip.ptr(bits), _hip.ptr(plan), _hip.stream(),
+        )
+    )
+    return PreparedMask(bits.view(B, n_q, -1), plan, B, n_q, kv_len)
+
+
+def _strides3(t: torch.Tensor):
+    assert t.dim() == 4 and t.stride(3) == 1, "last dimension must be contiguous"
+    return (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+
+
+def masked_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    prepared: PreparedMask,
+    scale: Optional[float] = None,
+    force_generic: bool = False,
+) -> torch.Tensor:
+    """q (B, H, n_q, D) [any strides with D contiguous], k/v (B, Hkv, kv_len, D) strided views.
+
+    Returns (B, n_q, H*D), i.e. already in the layout o_proj consumes."""
+    B, H, n_q, D = q.shape
+    Bk, Hkv, kv_len, Dk = k.shape
+    assert (Bk, Dk) == (B, D) and v.shape == k.shape and q.dtype == k.dtype == v.dtype
+    assert (prepared.batch, prepared.n_q, prepared.kv_len) == (B, n_q, kv_len), "mask/plan mismatch"
+    if q.stride(3) != 1:
+        q = q.contiguous()
+    if k.stride(3) != 1:
+        k = k.contiguous()
+    if v.stride(3) != 1:
+        v = v.contiguous()
+    out = torch.empty((B, n_q, H, D), dtype=q.dtype, device=q.device)
+    o_view = out.permute(0, 2, 1, 3)  # (B, H, n_q, D) strides
+    lib = _hip.lib()
+    ws_bytes = lib.rd_attention_workspace_bytes(B, H, n_q, kv_len, D)
+    if prepared.workspace is None or prepared.workspace.numel() < ws_bytes:
+        prepared.workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
+    _hip.check(
+        lib.rd_verify_attention(
+            _hip.ptr(q), _strides3(q), _hip.ptr(k), _strides3(k), _hip.ptr(v), _strides3(v),
+            _hip.ptr(out), _strides3(o_view), _hip.dtype_code(q.dtype), B, H, Hkv, n_q, kv_len, D,
+            float(scale if scale is not None else 1.0 / math.sqrt(D)), _hip.ptr(prepared.bits),
+            _hip.ptr(prepared.plan), _hip.ptr(prepared.workspace), prepared.workspace.numel(),
+            int(force_generic), _hip.stream(),
+        )
+    )
+    return out.view(B, n_q, H * D)

@@ -41,7 +41,10 @@ def masked_attention(q, k, v, mask) -> np.ndarray:
     """q (B,H,nq,D), k/v (B,Hkv,kv,D), mask (B,nq,kv) bool -> (B,H,nq,D) float64.
 
     Masked scores get the most negative finite value of the compute type rather than -inf, as the
-    additive bias of attention.py:87-88 does; a row with no attended key therefore averages V."""
+    additive bias of attention.py:87-88 does; a row with no attended key therefore averages V.
+    That is the reference's CPU behaviour.  On a GPU the reference rewrites such rows to all-True
+    before building the bias (modeling_llama.py:264-265, attention.py:58-72): callers that model
+    the GPU path pass tree_oracle.fully_masked_rows_to_true(mask) instead."""
     q = np.asarray(q, dtype=np.float64)
     k = np.asarray(k, dtype=np.float64)
     v = np.asarray(v, dtype=np.float64)

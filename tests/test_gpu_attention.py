@@ -1,0 +1,215 @@
+"""GPU parity: mask compression, causal mask and the verification attention (MFMA + generic)
+against the float64 oracle.  Tolerances: bf16 2e-2 of the output scale, fp32 1e-5."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp_oracle as O
+from oracle import tree_oracle as T
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(x, dtype):
+    return torch.tensor(np.asarray(x), dtype=dtype, device="cuda")
+
+
+def test_causal_mask_literals(literals):
+    from recurrent_drafting_amd import attention
+
+    for case in literals["causal_mask"]["cases"]:
+        for dt in (torch.long, torch.int32, torch.bool):
+            m = attention.causal_mask(_dev(case["padding_mask"], dt), case["query_len"], torch.device("cuda"))
+            assert m.dtype == torch.bool and m.cpu().to(torch.long).tolist() == case["mask"]
+    for case in literals["fully_masked_rows"]["cases"]:
+        got = attention.set_sdpa_fully_masked_rows(_dev(case["mask"], torch.long))
+        assert got.cpu().tolist() == case["expected"]
+    nf = torch.finfo(torch.float32).min
+    for case in literals["bias"]["cases"]:
+        m = _dev(case["mask"], torch.long)
+        b = attention.bias(m, torch.float32)
+        assert torch.equal(b, torch.where(m != 0, 0.0, nf).to(torch.float32))
+
+
+def test_causal_mask_random():
+    from recurrent_drafting_amd import attention
+
+    rng = np.random.default_rng(0)
+    pm = (rng.random((5, 300)) > 0.3).astype(np.int64)
+    for ql in (1, 7, 300):
+        got = attention.causal_mask(_dev(pm, torch.long), ql, torch.device("cuda"))
+        assert np.array_equal(got.cpu().numpy(), T.causal_mask(pm, ql))
+
+
+def test_mask_bits_and_plan():
+    from recurrent_drafting_amd import attention
+
+    rng = np.random.default_rng(1)
+    B, nq, kv = 3, 10, 1500
+    mask = rng.random((B, nq, kv)) > 0.5
+    mask[0, :, :700] = False  # row 0: first attended key >= 700 -> begin 640
+    mask[1, 3, :] = False  # an empty row gets all keys
+    mask[2, :, :64] = False
+    mask[2, 5, 70] = True
+    prep = attention.prepare(_dev(mask, torch.bool))
+    words = prep.bits.cpu().numpy().view(np.uint64)
+    fixed = T.fully_masked_rows_to_true(mask)
+    for b in range(B):
+        for q in range(nq):
+            bits = np.unpackbits(words[b, q].view(np.uint8), bitorder="little")[:kv].astype(bool)
+            assert np.array_equal(bits, fixed[b, q]), (b, q)
+            assert not np.unpackbits(words[b, q].view(np.uint8), bitorder="little")[kv:].any()
+    plan = prep.plan.cpu().numpy()
+    n_items, max_splits = plan[0], plan[4]
+    assert plan[1] == nq and plan[2] == kv and plan[3] == (kv + 63) // 64
+    per_row = plan[8 : 8 + 4 * B].reshape(B, 4)
+    firsts = [int(np.argmax(fixed[b].any(axis=0))) // 64 * 64 for b in range(B)]
+    assert per_row[:, 0].tolist() == firsts
+    items = plan[8 + 4 * B : 8 + 4 * B + 4 * n_items].reshape(n_items, 4)
+    assert n_items == per_row[:, 1].sum() and per_row[:, 1].max() <= max_splits
+    lens = items[:, 2] - items[:, 1]
+    assert (np.diff(lens) <= 0).all()  # longest first
+    for b in range(B):  # the items of a row tile [begin, kv) without gaps or overlap
+        mine = sorted((lo, hi) for bb, lo, hi, s in items.tolist() if bb == b)
+        assert mine[0][0] == firsts[b] and mine[-1][1] == kv
+        assert all(a[1] == c[0] for a, c in zip(mine, mine[1:]))
+        assert all(lo % 64 == 0 for lo, _ in mine)
+
+
+def _run(q, k, v, mask, dtype, force_generic, cache_like=False):
+    from recurrent_drafting_amd import attention
+
+    tq, tk, tv = (_dev(x, torch.float32).to(dtype) for x in (q, k, v))
+    B, H, nq, D = tq.shape
+    # q arrives as the transpose view of (B, nq, H, D), as in the model
+    tq = tq.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    if cache_like:  # K/V as views into a longer pre-allocated cache
+        kv = tk.shape[2]
+        big_k = torch.zeros(B, tk.shape[1], kv + 37, D, dtype=dtype, device="cuda")
+        big_v = torch.full_like(big_k, 3.0)
+        big_k[:, :, :kv] = tk; big_v[:, :, :kv] = tv
+        tk, tv = big_k[:, :, :kv], big_v[:, :, :kv]
+    prep = attention.prepare(_dev(mask, torch.bool))
+    out = attention.masked_attention(tq, tk, tv, prep, force_generic=force_generic)
+    torch.cuda.synchronize()
+    ref_in = [x.float().cpu().numpy() for x in (tq, tk, tv)]  # the oracle sees the rounded inputs
+    # on a GPU the reference first turns empty rows into all-True rows (modeling_llama.py:264-265),
+    # so such a row attends to every key with its real scores
+    ref = O.masked_attention(*ref_in, T.fully_masked_rows_to_true(mask))
+    return out.float().cpu().numpy().reshape(B, nq, H, D).transpose(0, 2, 1, 3), ref
+
+
+def _assert_close(got, ref, dtype):
+    scale = np.abs(ref).max()
+    tol = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-3}[dtype]
+    err = np.abs(got - ref).max()
+    assert err <= tol * scale, f"max err {err:.3e} vs scale {scale:.3e} ({dtype})"
+
+
+def _tree_case(B, W, L, prev_lens, seed):
+    beams = T.synthetic_beams(B, W, L, vocab=50, seed=seed)
+    S = max(prev_lens)
+    pm = np.zeros((B, S), dtype=np.int64)
+    for b, n in enumerate(prev_lens):
+        pm[b, S - n :] = 1
+    _, _, mask, _, _ = T.pack(beams, pm)
+    return mask
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("H,Hkv,D", [(4, 4, 32), (4, 2, 64), (2, 1, 128), (3, 3, 80)])
+def test_generic_kernel_small(dtype, H, Hkv, D):
+    mask = _tree_case(2, 4, 3, [5, 9], seed=D)
+    rng = np.random.default_rng(D)
+    B, nq, kv = mask.shape
+    q = rng.standard_normal((B, H, nq, D)); k = rng.standard_normal((B, Hkv, kv, D)); v = rng.standard_normal((B, Hkv, kv, D))
+    got, ref = _run(q, k, v, mask, dtype, force_generic=True, cache_like=True)
+    _assert_close(got, ref, dtype)
+
+
+def test_generic_kernel_random_mask_with_empty_rows():
+    rng = np.random.default_rng(7)
+    B, H, nq, kv, D = 2, 2, 6, 700, 32
+    mask = rng.random((B, nq, kv)) > 0.7
+    mask[0, 2] = False
+    mask[1, :, :300] = False
+    q = rng.standard_normal((B, H, nq, D)); k = rng.standard_normal((B, H, kv, D)); v = rng.standard_normal((B, H, kv, D))
+    got, ref = _run(q, k, v, mask, torch.float32, force_generic=True)
+    _assert_close(got, ref, torch.float32)
+
+
+@pytest.mark.parametrize("B,H,Hkv,W,L,prev_lens", [
+    (1, 1, 1, 2, 3, [40]),            # one tile, one item
+    (2, 2, 2, 8, 5, [100, 37]),       # ragged prefix, < 64 queries
+    (2, 4, 2, 45, 5, [700, 1300]),    # > 32 queries per wave, split keys, GQA
+    (1, 2, 2, 64, 5, [64]),           # > 256 queries: two query tiles
+    (3, 2, 2, 16, 4, [2000, 5, 900]),  # several splits and a nearly empty prefix
+])
+def test_mfma_kernel(B, H, Hkv, W, L, prev_lens):
+    mask = _tree_case(B, W, L, prev_lens, seed=W)
+    rng = np.random.default_rng(W * 7 + L)
+    _, nq, kv = mask.shape
+    D = 128
+    q = rng.standard_normal((B, H, nq, D)); k = rng.standard_normal((B, Hkv, kv, D)); v = rng.standard_normal((B, Hkv, kv, D))
+    got, ref = _run(q, k, v, mask, torch.bfloat16, force_generic=False, cache_like=True)
+    _assert_close(got, ref, torch.bfloat16)
+    got2, _ = _run(q, k, v, mask, torch.bfloat16, force_generic=True, cache_like=True)
+    _assert_close(got2, ref, torch.bfloat16)
+
+
+def test_mfma_kernel_pad_tokens_inside_the_prefix_and_empty_rows():
+    """Keys masked by VALUE in the middle of the prefix, and a query row with no key at all."""
+    rng = np.random.default_rng(11)
+    mask = _tree_case(2, 6, 4, [333, 200], seed=3).copy()
+    mask[:, :, rng.integers(150, 300, size=20)] = False
+    mask[1, 4, :] = False
+    B, nq, kv = mask.shape
+    q = rng.standard_normal((B, 2, nq, 128)); k = rng.standard_normal((B, 2, kv, 128)); v = rng.standard_normal((B, 2, kv, 128))
+    got, ref = _run(q, k, v, mask, torch.bfloat16, force_generic=False)
+    _assert_close(got, ref, torch.bfloat16)
+
+
+def test_verify_attention_benchmark_shape():
+    """Config 3: 32 heads x 128, batch 8, cached length U[500,2548], tree from the config-2 beams.
+    Full size against a float32 torch reference on the GPU; two heads against the float64 oracle."""
+    from recurrent_drafting_amd import attention
+
+    rng = np.random.default_rng(123)
+    B, H, D = 8, 32, 128
+    lens = rng.integers(500, 2549, size=B)
+    beams = T.synthetic_beams(B, 45, 5, seed=123)
+    S = int(lens.max())
+    pm = np.zeros((B, S), dtype=np.int64)
+    for b in range(B):
+        pm[b, S - lens[b] :] = 1
+    _, _, mask, _, _ = T.pack(beams, pm)
+    _, nq, kv = mask.shape
+    torch.manual_seed(0)
+    cache = torch.randn(2, B, H, kv + 64, D, device="cuda", dtype=torch.bfloat16)
+    k, v = cache[0, :, :, :kv], cache[1, :, :, :kv]
+    q = torch.randn(B, nq, H, D, device="cuda", dtype=torch.bfloat16).permute(0, 2, 1, 3)
+    tmask = _dev(mask, torch.bool)
+    prep = attention.prepare(tmask)
+    out = attention.masked_attention(q, k, v, prep).view(B, nq, H, D).permute(0, 2, 1, 3).float()
+    s = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float()) / D ** 0.5
+    s = s.masked_fill(~tmask[:, None], float("-inf"))
+    ref = torch.einsum("bhqk,bhkd->bhqd", torch.softmax(s, dim=-1), v.float())
+    err = (out - ref).abs().max().item()
+    assert err <= 2e-2 * ref.abs().max().item(), err
+    heads = [0, 17]
+    ref64 = O.masked_attention(q[:, heads].float().cpu().numpy(), k[:, heads].float().cpu().numpy(),
+                               v[:, heads].float().cpu().numpy(), mask)
+    _assert_close(out[:, heads].cpu().numpy(), ref64, torch.bfloat16)
+
+
+def test_argument_errors():
+    from recurrent_drafting_amd import attention
+
+    mask = torch.ones(1, 2, 5, dtype=torch.bool, device="cuda")
+    prep = attention.prepare(mask)
+    q = torch.zeros(1, 2, 2, 16, device="cuda"); k = torch.zeros(1, 2, 6, 16, device="cuda")
+    with pytest.raises(AssertionError, match="mismatch"):
+        attention.masked_attention(q, k, k, prep)
+    k = torch.zeros(1, 3, 5, 16, device="cuda")
+    with pytest.raises(RuntimeError, match="multiple"):
+        attention.masked_attention(q, k, k, prep)
