@@ -85,12 +85,14 @@ RD_API int rd_tree_mask(const int64_t* unpacker, const int64_t* packed_token_ind
  * Row gather: out[b, t, :] = packed[b, index[b, t], :], t in [0, n_out).
  * Replaces tree_attention.unpack (tree_attention.py:341-387) for hidden states and logits, and
  * _select_one_per_row gathers (recurrent_drafting.py:37-40) when n_out == 1.
- * Rows are row_bytes long; batch strides are in bytes (packed) / elements (index).  An index
- * outside [0, n_src) leaves its output row untouched.
+ * Rows are row_bytes long; strides are in bytes (packed, out) / elements (index); output row t of
+ * batch row b starts at out + b*out_batch_stride_bytes + t*out_row_stride_bytes.  An index outside
+ * [0, n_src) leaves its output row untouched.
  * ------------------------------------------------------------------------------------------ */
 RD_API int rd_unpack_rows(const void* packed, int64_t packed_batch_stride_bytes, int64_t row_bytes,
                           const int64_t* index, int64_t index_batch_stride, int batch, int n_out,
-                          int n_src, void* out, int64_t out_batch_stride_bytes, void* stream);
+                          int n_src, void* out, int64_t out_batch_stride_bytes,
+                          int64_t out_row_stride_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * First maximal index of every row of a (rows, vocab) matrix; NaN counts as the largest value.

@@ -1,0 +1,196 @@
+"""Recurrent drafter head and its beam search.
+
+Module and parameter names follow the reference's recurrent_drafting/modeling_drafter.py, so its
+checkpoints load.  The dense layers stay on torch (rocBLAS/hipBLASLt GEMMs); everything after the
+vocabulary GEMM of one beam-search iteration -- max subtraction, top-50 filter, log-softmax, beam
+score, top-W over width*vocab, parent/token split, beam gather -- is one call of rd_beam_topk.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+import transformers
+
+from . import _hip, configuration_drafter, tree_attention
+
+LOG_0 = -50000.0
+LOG_1 = 0.0
+TOP_K = 50
+
+
+@dataclass
+class BeamShape:
+    width: int
+    length: int
+
+
+def register_auto_models() -> None:
+    cfg = configuration_drafter.DrafterConfig
+    transformers.AutoConfig.register(model_type=cfg.model_type, config=cfg)
+    transformers.AutoModel.register(config_class=cfg, model_class=Drafter)
+
+
+class ResBlock(torch.nn.Module):
+    def __init__(self, cfg: configuration_drafter.DrafterConfig):
+        super().__init__()
+        self.linear = torch.nn.Linear(cfg.exit_dim, cfg.exit_dim, bias=True)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return x + torch.nn.functional.silu(self.linear(x))
+
+
+def _gather_beams(x: torch.Tensor, selected_beams: torch.Tensor) -> torch.Tensor:
+    """x (B, W, ...) re-ordered along dim 1 by selected_beams (B, W) (modeling_drafter.py:42-53)."""
+    B, W = x.shape[0], x.shape[1]
+    out = tree_attention.gather_rows(x.reshape(B, W, -1), selected_beams.to(torch.long))
+    return out.view(x.shape)
+
+
+def _add_decoding_dim(x: torch.Tensor, beam_width: int) -> torch.Tensor:
+    """(B, ...) -> (B, beam_width, ...) by repetition (modeling_drafter.py:56-60)."""
+    return x.unsqueeze(1).repeat_interleave(beam_width, dim=1)
+
+
+def maintain_logits(logits: torch.Tensor) -> torch.Tensor:
+    """Row maximum subtracted (modeling_drafter.py:63-77).  The beam search fuses this step."""
+    return logits - logits.amax(dim=-1, keepdim=True)
+
+
+def warp_logits(logits: torch.Tensor, top_k: int = TOP_K, mask_value: float = LOG_0) -> torch.Tensor:
+    """Everything below the row's top_k-th largest value becomes mask_value
+    (modeling_drafter.py:80-99).  The beam search and the greedy decode loop never materialise
+    this tensor; the function is kept for callers that want it."""
+    top_k = min(top_k, logits.size(-1))
+    kth = torch.topk(logits, top_k).values[..., -1:]
+    return logits.masked_fill(logits < kth, mask_value)
+
+
+def beam_topk_step(
+    logits: torch.Tensor,
+    log_p_beam: torch.Tensor,
+    beams: torch.Tensor,
+    want_log_probs: bool,
+    force_fallback: bool = False,
+):
+    """One fused post-GEMM iteration.  logits (B, W, V); log_p_beam (B, W) f32; beams (B, W, t).
+
+    Returns (new_log_p_beam, tokens, parents, new_beams (B, W, t+1), log_p_new_token or None)."""
+    B, W, V = logits.shape
+    assert log_p_beam.dtype == torch.float32 and log_p_beam.shape == (B, W)
+    assert beams.dtype == torch.long and beams.shape[:2] == (B, W)
+    x = logits.reshape(B * W, V)
+    if x.stride(1) != 1 or (x.stride(0) * x.element_size()) % 16 or x.data_ptr() % 16:
+        x = x.contiguous()
+        if (V * x.element_size()) % 16:  # pad rows to a 16-byte multiple
+            pad = (-V) % (16 // x.element_size())
+            x = torch.nn.functional.pad(x, (0, pad), value=float("-inf"))[:, :V]
+    beams = beams.contiguous()
+    log_p_beam = log_p_beam.contiguous()
+    t = beams.shape[2]
+    dev = logits.device
+    lib = _hip.lib()
+    new_lpb = torch.empty((B, W), dtype=torch.float32, device=dev)
+    tok_par = torch.empty((2, B, W), dtype=torch.long, device=dev)
+    new_beams = torch.empty((B, W, t + 1), dtype=torch.long, device=dev)
+    logp = torch.empty((B, W, V), dtype=torch.float32, device=dev) if want_log_probs else None
+    ws_bytes = lib.rd_beam_topk_workspace_bytes(B, W)
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+    _hip.check(
+        lib.rd_beam_topk(
+            _hip.ptr(x), _hip.dtype_code(x.dtype), x.stride(0), B, W, V, _hip.ptr(log_p_beam),
+            TOP_K, LOG_0, _hip.ptr(beams), t, _hip.ptr(new_lpb), _hip.ptr(tok_par[0]),
+            _hip.ptr(tok_par[1]), _hip.ptr(new_beams), _hip.ptr(logp), V, _hip.ptr(ws), ws.numel(),
+            int(force_fallback), _hip.stream(),
+        )
+    )
+    return new_lpb, tok_par[0], tok_par[1], new_beams, logp
+
+
+class Drafter(transformers.PreTrainedModel):
+    config_class = configuration_drafter.DrafterConfig
+
+    def __init__(self, cfg: configuration_drafter.DrafterConfig):
+        super().__init__(cfg)
+        self.config = cfg
+        if 2 * cfg.hidden_size != cfg.exit_dim:  # optional projection of [context, state]
+            self.input_proj = torch.nn.Linear(2 * cfg.hidden_size, cfg.exit_dim, bias=True)
+        blocks = [ResBlock(cfg) for _ in range(cfg.num_draft_layers)]
+        self.lm_head = torch.nn.Sequential(
+            *blocks, torch.nn.Linear(cfg.exit_dim, cfg.vocab_size, bias=False)
+        )
+        if cfg.rnn:
+            self.rnn_u = torch.nn.Linear(cfg.hidden_size, cfg.hidden_size, bias=True)
+            self.rnn_w = torch.nn.Linear(cfg.hidden_size, cfg.hidden_size, bias=False)
+
+    def raw_logits(self, x: torch.Tensor) -> torch.Tensor:
+        """Vocabulary logits of [context, state] before any normalisation."""
+        return self.lm_head(self.input_proj(x) if hasattr(self, "input_proj") else x)
+
+    def compute_logits(self, x: torch.Tensor) -> torch.Tensor:
+        """Logits with the row maximum at zero and everything below the top 50 at LOG_0
+        (modeling_drafter.py:127-131)."""
+        return warp_logits(maintain_logits(self.raw_logits(x)))
+
+    def beam_search_candidates(
+        self,
+        prompt_state: torch.Tensor,
+        init_token: torch.Tensor,
+        embeddings: torch.nn.Embedding,
+        beam_shape: BeamShape = BeamShape(10, 4),
+        return_log_probs: bool = True,
+    ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        """beams (B, W, L) int64 and, unless return_log_probs is False, the drafter's
+        log-probabilities (B, W, L-1, V) float32 of every drafted position
+        (modeling_drafter.py:133-232).  Greedy decoding never reads the log-probabilities."""
+        assert init_token.dtype == torch.long
+        assert prompt_state.ndim == 2
+        assert init_token.ndim == 1
+        assert beam_shape.length > 1
+        B, hidden = prompt_state.shape
+        W, L = beam_shape.width, beam_shape.length
+        V = embeddings.num_embeddings
+        dev = prompt_state.device
+
+        # only beam 0 is alive at the start, so the first iteration fans out from it alone
+        log_p_beam = torch.full((B, W), LOG_0, dtype=torch.float32, device=dev)
+        log_p_beam[:, 0] = LOG_1
+        context = prompt_state.unsqueeze(1).expand(B, W, hidden)
+        beams = init_token.view(B, 1, 1).expand(B, W, 1).contiguous()
+        state = torch.zeros(B, W, hidden, device=dev, dtype=prompt_state.dtype)
+        step_log_probs: List[torch.Tensor] = []
+        step_parents: List[torch.Tensor] = []
+
+        for _ in range(L - 1):
+            last = embeddings(beams[..., -1])
+            if self.config.rnn:
+                state = torch.nn.functional.silu(self.rnn_w(last) + self.rnn_u(state))
+            else:
+                state = last + state
+            logits = self.raw_logits(torch.cat([context, state], dim=-1))
+            log_p_beam, _, parents, beams, logp = beam_topk_step(
+                logits, log_p_beam, beams, want_log_probs=return_log_probs
+            )
+            state = _gather_beams(state, parents)
+            if return_log_probs:
+                step_log_probs.append(logp)
+                step_parents.append(parents)
+
+        if not return_log_probs:
+            return beams, None
+        # history[b, w, t] = log-probs of step t under the ancestor of final beam w at step t:
+        # compose the parent maps backwards once instead of re-gathering the history every step
+        history = torch.empty((B, W, L - 1, V), dtype=torch.float32, device=dev)
+        ancestor = torch.arange(W, device=dev).expand(B, W)
+        for t in range(L - 2, -1, -1):
+            ancestor = torch.gather(step_parents[t], 1, ancestor)
+            tree_attention.gather_rows(step_log_probs[t], ancestor.contiguous(), out=history[:, :, t, :])
+        return beams, history
+
+    def assert_valid(self) -> None:
+        has_proj = hasattr(self, "input_proj")
+        assert has_proj == (2 * self.config.hidden_size != self.config.exit_dim)
+        assert isinstance(self.lm_head, torch.nn.Sequential)
+        assert len(self.lm_head) == self.config.num_draft_layers + 1

@@ -1,0 +1,199 @@
+"""Llama with the pre-allocated KV cache, attention on the HIP verification kernel.
+
+Module and parameter names match Hugging Face Llama checkpoints (and the reference's
+recurrent_drafting/modeling_llama.py), so `from_pretrained` works unchanged.  Projections, MLP and
+norms are torch ops (rocBLAS/hipBLASLt GEMMs).  Per forward the bool attention mask is packed to
+bits once; per layer the keys and values are appended to the cache in place and
+`attention.masked_attention` reads them through strided views -- no repeat_interleave copy, no
+additive bias tensor.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import nn
+from transformers.activations import ACT2FN
+from transformers.modeling_outputs import CausalLMOutput
+from transformers.modeling_utils import PreTrainedModel
+from transformers.models.llama.configuration_llama import LlamaConfig
+
+from . import attention, kv_cache
+
+KeyValue = Tuple[kv_cache.View, kv_cache.View]
+
+
+class LlamaRMSNorm(nn.Module):
+    def __init__(self, hidden_size: int, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.variance_epsilon = eps
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        # statistics in float32, result rounded to the activations' dtype before the gain
+        x = hidden_states.float()
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * x.to(hidden_states.dtype)
+
+
+class LlamaRotaryEmbedding(nn.Module):
+    """cos/sin tables indexed by absolute position; grown on demand (modeling_llama.py:35-72)."""
+
+    def __init__(self, dim: int, max_position_embeddings: int = 2048, base: float = 10000.0,
+                 device: Optional[torch.device] = None):
+        super().__init__()
+        self.dim, self.base = dim, base
+        inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2).float().to(device) / dim))
+        self.register_buffer("inv_freq", inv_freq)
+        self._build(max_position_embeddings, self.inv_freq.device, torch.get_default_dtype())
+
+    def _build(self, seq_len: int, device, dtype) -> None:
+        self.max_seq_len_cached = seq_len
+        t = torch.arange(seq_len, device=device, dtype=self.inv_freq.dtype)
+        angles = torch.outer(t, self.inv_freq.to(device))
+        table = torch.cat((angles, angles), dim=-1)
+        self.cos_cached = table.cos().to(dtype)
+        self.sin_cached = table.sin().to(dtype)
+        self._cast = {}
+
+    def forward(self, device: torch.device, dtype: torch.dtype, seq_len: int = 0):
+        if seq_len > self.max_seq_len_cached:
+            self._build(seq_len, device, dtype)
+        key = (device, dtype)
+        if key not in self._cast:  # the cast tables are reused by every layer call
+            self._cast[key] = (self.cos_cached.to(dtype=dtype).to(device),
+                               self.sin_cached.to(dtype=dtype).to(device))
+        cos, sin = self._cast[key]
+        return cos[:seq_len], sin[:seq_len]
+
+
+def _rotate_half(x: torch.Tensor) -> torch.Tensor:
+    half = x.shape[-1] // 2
+    return torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, position_ids):
+    """q, k (B, heads, n, D); cos/sin (positions, D); position_ids (B, n).  NeoX-style rotation."""
+    cos = cos[position_ids].unsqueeze(1)
+    sin = sin[position_ids].unsqueeze(1)
+    return (q * cos) + (_rotate_half(q) * sin), (k * cos) + (_rotate_half(k) * sin)
+
+
+class LlamaMLP(nn.Module):
+    def __init__(self, config: LlamaConfig) -> None:
+        super().__init__()
+        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
+        self.act_fn = ACT2FN[config.hidden_act]
+
+    def forward(self, x):
+        return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+
+
+def _rope_theta(config: LlamaConfig) -> float:
+    """`rope_theta` of older configs; newer transformers releases keep it in `rope_parameters`."""
+    theta = getattr(config, "rope_theta", None)
+    if theta is None:
+        params = getattr(config, "rope_parameters", None) or {}
+        theta = params.get("rope_theta", 10000.0)
+    return float(theta)
+
+
+class LlamaAttention(nn.Module):
+    def __init__(self, config: LlamaConfig):
+        super().__init__()
+        self.config = config
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.head_dim = self.hidden_size // self.num_heads
+        self.n_kv_heads = config.num_key_value_heads
+        self.n_kv_groups = self.num_heads // self.n_kv_heads
+        assert self.head_dim * self.num_heads == self.hidden_size
+        self.q_proj = nn.Linear(self.hidden_size, self.num_heads * self.head_dim, bias=False)
+        self.k_proj = nn.Linear(self.hidden_size, self.n_kv_heads * self.head_dim, bias=False)
+        self.v_proj = nn.Linear(self.hidden_size, self.n_kv_heads * self.head_dim, bias=False)
+        self.o_proj = nn.Linear(self.num_heads * self.head_dim, self.hidden_size, bias=False)
+        self.rotary_emb = LlamaRotaryEmbedding(dim=self.head_dim, base=_rope_theta(config))
+
+    def forward(self, hidden_states: torch.Tensor, position_ids: torch.LongTensor,
+                past_key_value: KeyValue, attention_mask: attention.PreparedMask) -> torch.Tensor:
+        bsz, q_len, _ = hidden_states.size()
+        q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+        k = self.k_proj(hidden_states).view(bsz, q_len, self.n_kv_heads, self.head_dim).transpose(1, 2)
+        v = self.v_proj(hidden_states).view(bsz, q_len, self.n_kv_heads, self.head_dim).transpose(1, 2)
+        cos, sin = self.rotary_emb(v.device, v.dtype, q_len + past_key_value[0].shape[-2])
+        q, k = apply_rotary_pos_emb(q, k, cos, sin, position_ids)
+        keys = past_key_value[0].cat(k)  # in place; strided view of the cache
+        values = past_key_value[1].cat(v)
+        out = attention.masked_attention(q, keys, values, attention_mask)  # (B, q_len, hidden)
+        return self.o_proj(out)
+
+
+class LlamaDecoderLayer(nn.Module):
+    def __init__(self, config: LlamaConfig) -> None:
+        super().__init__()
+        self.self_attn = LlamaAttention(config=config)
+        self.mlp = LlamaMLP(config)
+        self.input_layernorm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+
+    def forward(self, hidden_states, position_ids, past_key_value, attention_mask):
+        hidden_states += self.self_attn(self.input_layernorm(hidden_states), position_ids,
+                                        past_key_value, attention_mask)
+        hidden_states += self.mlp(self.post_attention_layernorm(hidden_states))
+        return hidden_states
+
+
+class LlamaPreTrainedModel(PreTrainedModel):
+    config_class = LlamaConfig
+    base_model_prefix = "model"
+
+
+class LlamaModel(LlamaPreTrainedModel):
+    def __init__(self, config: LlamaConfig):
+        super().__init__(config)
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size, config.pad_token_id)
+        self.layers = nn.ModuleList(LlamaDecoderLayer(config) for _ in range(config.num_hidden_layers))
+        self.norm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        self.post_init()
+
+    def get_input_embeddings(self):
+        return self.embed_tokens
+
+    def forward(self, input_ids, attention_mask, position_ids, past_key_values) -> torch.Tensor:
+        """attention_mask: (B, q, kv) bool, or an attention.PreparedMask built from one."""
+        if not isinstance(attention_mask, attention.PreparedMask):
+            attention_mask = attention.prepare(attention_mask, fix_empty_rows=False)
+        hidden_states = self.embed_tokens(input_ids)
+        for layer, key_value in zip(self.layers, past_key_values):
+            hidden_states = layer(hidden_states, position_ids, key_value, attention_mask)
+        return self.norm(hidden_states)
+
+
+class LlamaForCausalLM(LlamaPreTrainedModel):
+    _tied_weights_keys = ["lm_head.weight"]
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.model = LlamaModel(config)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        self.post_init()
+
+    def get_input_embeddings(self):
+        return self.model.embed_tokens
+
+    def get_output_embeddings(self):
+        return self.lm_head
+
+    def hidden_states(self, input_ids, attention_mask, position_ids, past_key_values) -> torch.Tensor:
+        """Final-norm hidden states (B, q, hidden); rows that attend to nothing attend to
+        everything, as the reference arranges on a GPU (modeling_llama.py:264-265)."""
+        prepared = attention.prepare(attention_mask, fix_empty_rows=True)
+        return self.model(input_ids=input_ids, attention_mask=prepared, position_ids=position_ids,
+                          past_key_values=past_key_values)
+
+    def forward(self, input_ids, attention_mask, position_ids, past_key_values) -> CausalLMOutput:
+        hidden = self.hidden_states(input_ids, attention_mask, position_ids, past_key_values)
+        return CausalLMOutput(logits=self.lm_head(hidden).float(), hidden_states=hidden)

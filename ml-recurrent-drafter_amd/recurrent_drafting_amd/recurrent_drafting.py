@@ -1,0 +1,201 @@
+"""The ReDrafter decode loop on the HIP hot path.
+
+`RecurrentDrafting.generate` keeps the reference's signature and yields the same token tensors
+(recurrent_drafting/recurrent_drafting.py:559-705).  One step is
+
+    draft   beam search on the drafter head          rd_beam_topk x (L-1)      (+ torch GEMMs)
+    verify  beams -> prefix tree, mask, LLM forward   rd_tree_build, rd_tree_mask, rd_attn_prepare,
+                                                      rd_verify_attention per layer (+ torch GEMMs)
+    accept  argmax over the packed rows, longest      rd_argmax_rows, rd_accept_greedy,
+            agreeing prefix, ids and KV re-aligned    rd_realign_plan, rd_kv_compact
+
+Greedy decoding never materialises the (B, W, L, V) logits, never unpacks the KV cache into W*L
+slots and never clones it: argmax commutes with the unpack and with the top-50 filter, and the
+accepted rows are taken straight from their packed slots.  Two host reads per step (packed tree
+length, new sequence length) where the reference has more than ten.
+
+The module-level helpers of the reference are re-exported with their names for code and tests that
+call them directly.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Generator, Optional, Tuple
+
+import torch
+import torch.distributions as dist
+import transformers
+
+from . import acceptance, attention, kv_cache, modeling_drafter, modeling_llama, stats, tree_attention
+from .acceptance import (  # noqa: F401  (re-exported: the reference's helper names)
+    _count_left_paddings,
+    _greedy_choose_from_candidates,
+    _greedy_prepare_next_input,
+    _select_one_per_row,
+    _update_kv_cache_and_input_ids,
+)
+
+dist.Distribution.set_default_validate_args(False)
+
+
+@dataclass
+class SamplingArgs:
+    temperature: float
+    greedy: bool
+
+
+@dataclass
+class SpecialTokens:
+    pad: int
+    eos: Optional[int] = 1
+
+
+def _comprehend_prompt(
+    llm: transformers.PreTrainedModel,
+    input_ids: torch.Tensor,
+    cache: kv_cache.Cache,
+    sampling_args: SamplingArgs,
+    pad_token_id: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Prefill: fills the cache from the prompt and returns (last hidden state (B, hidden), first
+    generated token (B,)) (recurrent_drafting.py:391-434)."""
+    assert input_ids.dtype in [torch.int32, torch.int64]
+    seq = input_ids.shape[1]
+    mask = attention.causal_mask(input_ids != pad_token_id, seq, input_ids.device)
+    pads = _count_left_paddings(input_ids.to(torch.long), pad_token_id)
+    position_ids = torch.arange(seq, dtype=torch.long, device=input_ids.device).expand(
+        input_ids.shape
+    ) - pads.unsqueeze(-1)
+    hidden = llm.hidden_states(input_ids, mask, position_ids, cache.sliced)
+    last_state = hidden[:, -1, :]
+    last_logits = llm.lm_head(last_state)  # argmax ignores the top-50 filter and the fp32 cast
+    if sampling_args.greedy:
+        next_token = acceptance.argmax_rows(last_logits)
+    else:
+        filtered = modeling_drafter.warp_logits(last_logits.float())
+        probs = torch.softmax(filtered / sampling_args.temperature, dim=-1)
+        next_token = dist.Categorical(probs=probs).sample()
+    return last_state, next_token
+
+
+def _verify_candidates(
+    step_record: stats.TextGeneration.Step,
+    llm: transformers.PreTrainedModel,
+    input_ids: torch.Tensor,
+    beams: torch.Tensor,
+    cache: kv_cache.Cache,
+    pad_token_id: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Drop-in for recurrent_drafting.py:437-465: returns unpacked (hidden (B,W,L,hid), filtered
+    logits (B,W,L,V) float32) and leaves the cache unpacked.  `generate` does not use this form."""
+    packed, unpacker, mask, offsets = tree_attention.pack(beams, input_ids != pad_token_id)
+    pads = _count_left_paddings(input_ids, pad_token_id)
+    position_ids = (cache.sliced[0][0].length - pads).unsqueeze(-1) + offsets
+    with step_record.time("base_forward"):
+        out = llm(packed, attention_mask=mask, past_key_values=cache.sliced, position_ids=position_ids)
+    logits = modeling_drafter.warp_logits(out.logits)
+    hidden = tree_attention.unpack(out.hidden_states, unpacker)
+    logits = tree_attention.unpack(logits, unpacker)
+    cache.unpack(input_ids.shape[-1], unpacker)
+    return hidden, logits
+
+
+class RecurrentDrafting(torch.nn.Module):
+    def __init__(self, llm: transformers.PreTrainedModel, drafter: modeling_drafter.Drafter):
+        super().__init__()
+        self.llm = llm
+        self.drafter = drafter
+
+    def llm_n_kv_heads(self) -> int:
+        if isinstance(self.llm, modeling_llama.LlamaForCausalLM):
+            return self.llm.config.num_key_value_heads
+        raise TypeError(f"Unsupported base model type {type(self.llm)}")
+
+    def generate(
+        self,
+        ledger: stats.Ledger,
+        input_ids: torch.Tensor,
+        max_length: int,
+        beam_shape: modeling_drafter.BeamShape = modeling_drafter.BeamShape(10, -1),
+        sampling_args: SamplingArgs = SamplingArgs(1.0, False),
+        special_tokens: SpecialTokens = SpecialTokens(0, 1),
+    ) -> Generator[torch.Tensor, None, None]:
+        with torch.inference_mode():
+            with stats.text_generation(ledger) as record:
+                yield from self._generate(
+                    record, input_ids, max_length, beam_shape, sampling_args, special_tokens
+                )
+
+    # -- one greedy step on the fused path ------------------------------------------------------
+    def _greedy_step(self, step_record, input_ids, context, init_tokens, cache, beam_shape, pad):
+        llm = self.llm
+        with step_record.time("generate_candidates"):
+            beams, _ = self.drafter.beam_search_candidates(
+                context, init_tokens, llm.base_model.get_input_embeddings(), beam_shape,
+                return_log_probs=False,
+            )
+        with step_record.time("verify_candidates"):
+            prev = input_ids.shape[1]
+            tree = tree_attention.build_tree(beams)
+            mask = tree_attention.build_mask(tree, input_ids != pad)
+            pads = _count_left_paddings(input_ids, pad)
+            position_ids = (prev - pads).unsqueeze(-1) + tree.position_offsets
+            with step_record.time("base_forward"):
+                hidden = llm.hidden_states(tree.packed_beams, mask, position_ids, cache.sliced)
+                logits = llm.lm_head(hidden)  # (B, n, V) in the model's dtype
+        with step_record.time("accept_candidate_tokens"):
+            llm_tokens = acceptance.argmax_rows(logits)  # per packed slot
+            with step_record.time("choose_from_candidates"):
+                n_tokens, seq_in_beam, next_tokens, last_slot = acceptance.greedy_accept(
+                    beams, llm_tokens, tree.unpacker
+                )
+            with step_record.time("update_kv_cache_and_input_ids"):
+                input_ids = acceptance.realign(
+                    input_ids, n_tokens, seq_in_beam, beams, cache, pad, unpacker=tree.unpacker
+                )
+            with step_record.time("greedy_prepare_next_input"):
+                context = tree_attention.gather_rows(hidden, last_slot.unsqueeze(-1))[:, 0, :]
+        return context, input_ids, next_tokens, n_tokens
+
+    def _generate(self, text_generation, input_ids, max_length, beam_shape, sampling_args,
+                  special_tokens) -> Generator[torch.Tensor, None, None]:
+        assert input_ids.dtype == torch.long, f"input_ids.dtype {input_ids.dtype} is not long"
+        if not sampling_args.greedy:
+            raise NotImplementedError(
+                "speculative sampling is not on the HIP path yet; use SamplingArgs(greedy=True)"
+            )
+        batch_size, seq_len = input_ids.shape
+        init_seq_len = seq_len
+        cfg = self.llm.config
+        cache = kv_cache.Cache(
+            batch_size=batch_size,
+            max_length=max_length + beam_shape.length * beam_shape.width,
+            n_layers=cfg.num_hidden_layers,
+            n_heads=self.llm_n_kv_heads(),
+            head_dim=cfg.hidden_size // cfg.num_attention_heads,
+            dtype=self.llm.dtype,
+            device=input_ids.device,
+        )
+        context, init_tokens = _comprehend_prompt(
+            self.llm, input_ids, cache, sampling_args, special_tokens.pad
+        )
+        while seq_len < max_length:
+            with text_generation.step() as step_record:
+                context, input_ids, init_tokens, n_tokens = self._greedy_step(
+                    step_record, input_ids, context, init_tokens, cache, beam_shape,
+                    special_tokens.pad,
+                )
+                output_tokens = torch.cat((input_ids, init_tokens.unsqueeze(-1)), dim=-1)
+                seq_len = output_tokens.shape[1]
+                step_record.set(
+                    {
+                        "input_id_length": seq_len,
+                        "avg_num_accepted": torch.sum(n_tokens).item() / batch_size,
+                    }
+                )
+                yield output_tokens[:, :max_length] if seq_len > max_length else output_tokens
+                if special_tokens.eos is not None:
+                    ended = (output_tokens[:, init_seq_len:] == special_tokens.eos).any(dim=-1)
+                    if bool(ended.all()):
+                        break

@@ -112,8 +112,13 @@ def _pack_beams(
     return t.packed_beams, t.packed_token_indices
 
 
-def gather_rows(packed: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
-    """out[b, t, :] = packed[b, index[b, t], :] for packed (B, n, F) and index (B, T) int64."""
+def gather_rows(
+    packed: torch.Tensor, index: torch.Tensor, out: Optional[torch.Tensor] = None
+) -> torch.Tensor:
+    """out[b, t, :] = packed[b, index[b, t], :] for packed (B, n, F) and index (B, T) int64.
+
+    `out`, if given, is a (B, T, F) view whose last dimension is contiguous (any row/batch stride),
+    e.g. one time slice of a (B, T, steps, F) history."""
     assert packed.dim() == 3 and index.dim() == 2 and index.dtype == torch.long
     B, n_src, F = packed.shape
     T = index.shape[1]
@@ -121,12 +126,14 @@ def gather_rows(packed: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
     if packed.stride(2) != 1 or packed.stride(1) != F:
         packed = packed.contiguous()
     index = index.contiguous()
-    out = torch.empty((B, T, F), dtype=packed.dtype, device=packed.device)
+    if out is None:
+        out = torch.empty((B, T, F), dtype=packed.dtype, device=packed.device)
+    assert out.shape == (B, T, F) and out.dtype == packed.dtype and out.stride(2) == 1
     es = packed.element_size()
     _hip.check(
         _hip.lib().rd_unpack_rows(
             _hip.ptr(packed), packed.stride(0) * es, F * es, _hip.ptr(index), T, B, T, n_src,
-            _hip.ptr(out), T * F * es, _hip.stream(),
+            _hip.ptr(out), out.stride(0) * es, out.stride(1) * es, _hip.stream(),
         )
     )
     return out

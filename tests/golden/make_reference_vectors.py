@@ -147,6 +147,56 @@ def beam_search_cases(rd):
     return out
 
 
+def end_to_end_cases(rd):
+    """Greedy token streams of the tiny float32 configuration, straight from the reference loop."""
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import tiny_models as tm
+    from transformers.models.llama.configuration_llama import LlamaConfig
+
+    out = []
+    try:
+        cfg = LlamaConfig(**tm.LLAMA, rope_theta=10000.0)
+        if not hasattr(cfg, "rope_theta"):
+            cfg.rope_theta = 10000.0
+        llm = rd.modeling_llama.LlamaForCausalLM(cfg)
+        drafter = rd.modeling_drafter.Drafter(rd.configuration_drafter.DrafterConfig(**tm.DRAFTER))
+    except Exception as e:  # library drift: an ordinary error
+        return dict(error=f"model construction failed: {type(e).__name__}: {e}")
+    llm.eval(); drafter.eval()
+    cases = [dict(seed=123, batch=1, prompt_len=16, left_pads=[], W=4, L=3, new_tokens=32),
+             dict(seed=7, batch=3, prompt_len=12, left_pads=[0, 3, 5], W=6, L=4, new_tokens=24),
+             dict(seed=11, batch=2, prompt_len=9, left_pads=[2, 0], W=5, L=5, new_tokens=20),
+             dict(seed=21, batch=4, prompt_len=10, left_pads=[0, 4, 1, 0], W=5, L=4, new_tokens=30,
+                  markov=True),
+             dict(seed=22, batch=2, prompt_len=6, left_pads=[0, 2], W=8, L=6, new_tokens=40,
+                  markov=True)]
+    for c in cases:
+        if c.get("markov"):
+            llama_sd, drafter_sd = tm.markov(c["seed"])
+        else:
+            llama_sd = tm.draw(tm.llama_shapes(), c["seed"])
+            drafter_sd = tm.draw(tm.drafter_shapes(), c["seed"] + 1000)
+        llm.load_state_dict(llama_sd, strict=False)  # rotary buffers are not part of the draw
+        drafter.load_state_dict(drafter_sd)
+        ids = tm.prompt(c["batch"], c["prompt_len"], tm.LLAMA["vocab_size"], c["seed"], c["left_pads"])
+        model = rd.recurrent_drafting.RecurrentDrafting(llm, drafter)
+        steps = []
+        try:
+            with torch.inference_mode():
+                gen = model._generate(
+                    text_generation=rd.stats.TextGeneration(), input_ids=ids,
+                    max_length=c["prompt_len"] + c["new_tokens"],
+                    beam_shape=rd.modeling_drafter.BeamShape(c["W"], c["L"]),
+                    sampling_args=rd.recurrent_drafting.SamplingArgs(1.0, True),
+                    special_tokens=rd.recurrent_drafting.SpecialTokens(0, None))
+                for tokens in gen:
+                    steps.append(tokens.tolist())
+        except Exception as e:
+            return dict(error=f"reference generate failed: {type(e).__name__}: {e}")
+        out.append(dict(config=c, steps=steps))
+    return out
+
+
 def main():
     rd = _import_reference()
     torch.set_num_threads(1)
@@ -156,6 +206,7 @@ def main():
         pack=pack_cases(rd),
         kv_update=kv_update_cases(rd),
         beam_search=beam_search_cases(rd),
+        end_to_end=end_to_end_cases(rd),
     )
     with open(OUT, "w") as f:
         json.dump(vec, f, separators=(",", ":"))

@@ -1,0 +1,173 @@
+"""GPU parity: one fused beam-search iteration (rd_beam_topk) and the whole beam search of the
+drafter head against the torch-CPU oracle.  Scores/log-probs: 1e-5 in fp32, 2e-2 in bf16; tokens
+and parents exact (inputs are either tie-free or ties are resolved by the documented rule)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp_oracle as O
+from oracle import torch_path as P
+
+sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
+import tiny_models as tm  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def _step(logits, lpb, beams, want_log_probs=True, force_fallback=False):
+    from recurrent_drafting_amd import modeling_drafter as md
+
+    out = md.beam_topk_step(logits.cuda(), lpb.cuda(), beams.cuda(), want_log_probs, force_fallback)
+    torch.cuda.synchronize()
+    return [None if t is None else t.cpu() for t in out]
+
+
+def _check_step(logits, lpb, beams, force_fallback, score_tol):
+    new_lpb, tok, par, new_beams, logp = _step(logits, lpb, beams, True, force_fallback)
+    o_lpb, o_tok, o_par, o_logp = O.beam_search_step(logits, lpb)
+    B, W, V = logits.shape
+    assert torch.allclose(logp, o_logp.float(), atol=score_tol, rtol=0), (logp - o_logp.float()).abs().max()
+    assert torch.allclose(new_lpb, o_lpb, atol=score_tol, rtol=0)
+    if not (torch.equal(tok, o_tok) and torch.equal(par, o_par)):
+        # selections may differ only where the oracle's own scores are closer than the tolerance
+        got = (par * V + tok).tolist(); want = (o_par * V + o_tok).tolist()
+        flat = (o_logp.float() + lpb[:, :, None]).reshape(B, -1)
+        for b in range(B):
+            cut = o_lpb[b, -1].item()
+            for i in set(got[b]) ^ set(want[b]):
+                assert abs(flat[b, i].item() - cut) <= score_tol, (b, i)
+    rows = torch.arange(B)[:, None]
+    assert torch.equal(new_beams[..., :-1], beams[rows, par]) and torch.equal(new_beams[..., -1], tok)
+    assert (new_lpb[:, :-1] >= new_lpb[:, 1:]).all()
+
+
+@pytest.mark.parametrize("force_fallback", [False, True])
+@pytest.mark.parametrize("B,W,V,t", [(2, 3, 64, 1), (1, 4, 1000, 2), (8, 45, 32000, 3), (2, 64, 32000, 1), (3, 5, 33, 1), (2, 6, 2500, 4)])
+def test_step_fp32_tie_free(B, W, V, t, force_fallback):
+    torch.manual_seed(V + W)
+    logits = torch.randn(B, W, V) * 2
+    lpb = -torch.rand(B, W) * 5
+    beams = torch.randint(0, V, (B, W, t))
+    _check_step(logits, lpb, beams, force_fallback, 1e-5)
+
+
+@pytest.mark.parametrize("force_fallback", [False, True])
+def test_step_first_iteration_only_beam_zero_alive(force_fallback):
+    """Scores [0, -50000, ...]: every winner descends from beam 0; W=64 > 50 needs filtered tokens,
+    which tie exactly and are taken in increasing token id."""
+    torch.manual_seed(1)
+    for W in (45, 64):
+        logits = torch.randn(2, 1, 32000).repeat(1, W, 1) * 3  # all beams share state at iteration 1
+        lpb = torch.full((2, W), O.LOG_0); lpb[:, 0] = O.LOG_1
+        beams = torch.randint(0, 32000, (2, 1, 1)).repeat(1, W, 1)
+        new_lpb, tok, par, new_beams, logp = _step(logits, lpb, beams, True, force_fallback)
+        o_lpb, o_tok, o_par, o_logp = O.beam_search_step(logits, lpb)
+        assert (par == 0).all() and torch.equal(tok, o_tok) and torch.equal(par, o_par)
+        assert torch.allclose(new_lpb, o_lpb, atol=1e-2, rtol=0)  # sums near -50000: fp32 spacing 4e-3
+
+
+@pytest.mark.parametrize("force_fallback", [False, True])
+def test_step_bf16_rounding_points(force_fallback):
+    """bf16 logits: values rounded after the max subtraction, filter value -49920, log-softmax
+    rounded to bf16, score float32.  Heavy ties among rounded scores -> lowest flat index wins."""
+    torch.manual_seed(2)
+    logits = (torch.randn(4, 45, 32000) * 1.3).to(torch.bfloat16)
+    lpb = (-torch.rand(4, 45) * 3).float()
+    beams = torch.randint(0, 32000, (4, 45, 2))
+    new_lpb, tok, par, new_beams, logp = _step(logits, lpb, beams, True, force_fallback)
+    o_lpb, o_tok, o_par, o_logp = O.beam_search_step(logits, lpb)
+    # log-probs agree to one bf16 step of the row (sum order may differ in the last float32 bit)
+    diff = (logp - o_logp.float()).abs()
+    assert diff.max() <= 2e-2 * o_logp.float()[o_logp.float() > -1000].abs().max()
+    exact = diff.max() == 0
+    if exact:
+        assert torch.equal(tok, o_tok) and torch.equal(par, o_par) and torch.equal(new_lpb, o_lpb)
+    else:
+        assert torch.allclose(new_lpb, o_lpb, atol=5e-2, rtol=0)
+    assert logp[0, 0].min().item() < -49000  # the filter value survives as a finite constant
+
+
+def test_step_many_ties_overflow_to_exact_path():
+    """All-equal and two-valued rows: every entry ties, the candidate list overflows, and the
+    lowest indices must win."""
+    V, W = 32000, 5
+    logits = torch.zeros(1, W, V)
+    logits[0, 1, 100:] = -1.0  # row 1: 100 large entries (> 50), the rest smaller
+    lpb = torch.zeros(1, W)
+    beams = torch.zeros(1, W, 1, dtype=torch.long)
+    new_lpb, tok, par, _, logp = _step(logits, lpb, beams)
+    o_lpb, o_tok, o_par, o_logp = O.beam_search_step(logits, lpb)
+    assert torch.equal(tok, o_tok) and torch.equal(par, o_par)
+    assert torch.allclose(new_lpb, o_lpb, atol=1e-5) and torch.allclose(logp, o_logp, atol=1e-5)
+
+
+def test_step_adversarial_layout_overflows_pivot():
+    """Large values concentrated where one thread sees them all defeats the per-wave pivot."""
+    V, W = 32000, 3
+    torch.manual_seed(3)
+    logits = torch.randn(1, W, V) * 0.01 - 10
+    idx = torch.arange(0, V, 8 * 1024)  # same thread, every vector chunk
+    for e in range(8):
+        logits[0, :, (idx + e).clamp(max=V - 1)] += 20 + torch.rand(len(idx))
+    lpb = torch.zeros(1, W)
+    beams = torch.zeros(1, W, 1, dtype=torch.long)
+    _check_step(logits, lpb, beams, False, 1e-5)
+
+
+def _models(seed, dtype):
+    import recurrent_drafting_amd as rd
+    from transformers.models.llama.configuration_llama import LlamaConfig
+
+    llm = rd.modeling_llama.LlamaForCausalLM(LlamaConfig(**tm.LLAMA))
+    drafter = rd.modeling_drafter.Drafter(rd.configuration_drafter.DrafterConfig(**tm.DRAFTER))
+    llm.load_state_dict(tm.draw(tm.llama_shapes(), seed), strict=False)
+    drafter.load_state_dict(tm.draw(tm.drafter_shapes(), seed + 1000))
+    return llm.to(dtype).eval(), drafter.to(dtype).eval()
+
+
+def test_beam_search_candidates_matches_reference_vectors(ref_vectors):
+    """The reference's own beams on tie-free float32 drafters (weights are multiples of 1/64)."""
+    import recurrent_drafting_amd as rd
+
+    for c in ref_vectors["beam_search"]:
+        W, L, V, hid = c["W"], c["L"], c["V"], c["hidden"]
+        drafter = rd.modeling_drafter.Drafter(rd.configuration_drafter.DrafterConfig(
+            vocab_size=V, hidden_size=hid, exit_dim=2 * hid, num_draft_layers=1, rnn=True))
+        sd = {k: torch.tensor(v, dtype=torch.float32).reshape(c["weight_shapes"][k]) / c["weight_scale"]
+              for k, v in c["weights_x64"].items()}
+        drafter.load_state_dict(sd)
+        drafter = drafter.cuda().eval()
+        emb = torch.nn.Embedding(V, hid)
+        emb.weight.data = torch.tensor(c["embedding_x64"], dtype=torch.float32).reshape(V, hid) / 64
+        emb = emb.cuda()
+        ctx = (torch.tensor(c["prompt_state_x64"], dtype=torch.float32).reshape(-1, hid) / 64).cuda()
+        with torch.inference_mode():
+            beams, hist = drafter.beam_search_candidates(
+                ctx, torch.tensor(c["init_token"]).cuda(), emb, rd.BeamShape(W, L))
+        assert beams.cpu().tolist() == c["beams"]
+        picked = torch.gather(hist, 3, beams[:, :, 1:, None]).squeeze(-1).cpu()
+        assert torch.allclose(picked, torch.tensor(c["log_prob_of_drafted"]), atol=1e-4)
+        assert torch.allclose(hist.max(-1).values.cpu(), torch.tensor(c["log_prob_row_max"]), atol=1e-4)
+
+
+@pytest.mark.parametrize("W,L", [(4, 3), (10, 4), (45, 5)])
+def test_beam_search_candidates_vs_torch_oracle_fp32(W, L):
+    import recurrent_drafting_amd as rd
+
+    llm, drafter = _models(5, torch.float32)
+    torch.manual_seed(W)
+    ctx = torch.randn(3, 128)
+    tok = torch.randint(1, 1000, (3,))
+    with torch.inference_mode():
+        o_beams, o_hist = P.beam_search(drafter, llm.model.embed_tokens, ctx, tok, W, L)
+        llm, drafter = llm.cuda(), drafter.cuda()
+        beams, hist = drafter.beam_search_candidates(ctx.cuda(), tok.cuda(), llm.model.embed_tokens, rd.BeamShape(W, L))
+        b2, none = drafter.beam_search_candidates(ctx.cuda(), tok.cuda(), llm.model.embed_tokens, rd.BeamShape(W, L), return_log_probs=False)
+    assert none is None and torch.equal(b2, beams)
+    assert hist.shape == (3, W, L - 1, 1000) and hist.dtype == torch.float32
+    assert torch.equal(beams.cpu(), o_beams)
+    assert torch.allclose(hist.cpu(), o_hist, atol=1e-4)
+    assert (beams[:, :, 0].cpu() == tok[:, None]).all()
