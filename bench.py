@@ -1,0 +1,277 @@
+"""Benchmark of the ReDrafter decode step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Workload (the configuration the headline metric is quoted on): random-init Vicuna-7B-shaped Llama
+in bf16 (32 layers, hidden 4096, 32 heads, FFN 11008, vocab 32000) with a ReDrafter head (hidden
+4096, exit_dim 8192, 2 residual blocks, recurrent state), weights N(0, 0.02) from a fixed seed;
+batch 8, prompts of 500 token ids uniform over the vocabulary (pad id excluded), beam 45 x 5,
+greedy, generation capped at 500 + 2048 tokens.  A step is one draft -> verify -> accept pass.
+
+One JSON line on stdout: tokens/sec over the K timed steps (all eight sequences together), the
+roofline entry of the dominant hand-written kernel (attn_mfma_kernel, timed with HIP events inside
+the library while the timed region runs), and a CPU baseline: the torch restatement of the same
+step (oracle/torch_path.py) timed on this machine's host cores on a bounded sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "ml-recurrent-drafter_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import torch  # noqa: E402
+
+LLAMA_7B = dict(vocab_size=32000, hidden_size=4096, intermediate_size=11008, num_hidden_layers=32,
+                num_attention_heads=32, num_key_value_heads=32, rms_norm_eps=1e-6, hidden_act="silu",
+                pad_token_id=0, max_position_embeddings=2048)
+DRAFTER_7B = dict(vocab_size=32000, hidden_size=4096, exit_dim=8192, num_draft_layers=2, rnn=True)
+BATCH, PROMPT, NEW_TOKENS, WIDTH, LENGTH, SEED = 8, 500, 2048, 45, 5, 123
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_models(device: str, dtype: torch.dtype, n_layers: int, seed: int):
+    """Random-init pair; every weight N(0, 0.02) from one seeded generator, norm gains 1."""
+    import recurrent_drafting_amd as rd
+    from transformers.models.llama.configuration_llama import LlamaConfig
+
+    prev = torch.get_default_dtype()
+    torch.set_default_dtype(dtype)
+    try:
+        with torch.device(device):
+            llm = rd.modeling_llama.LlamaForCausalLM(LlamaConfig(**dict(LLAMA_7B, num_hidden_layers=n_layers)))
+            drafter = rd.modeling_drafter.Drafter(rd.configuration_drafter.DrafterConfig(**DRAFTER_7B))
+    finally:
+        torch.set_default_dtype(prev)
+    gen = torch.Generator(device=device).manual_seed(seed)
+    with torch.no_grad():
+        for module in (llm, drafter):
+            for name, p in sorted(module.named_parameters()):
+                if name.endswith("layernorm.weight") or name.endswith("norm.weight"):
+                    p.fill_(1.0)
+                else:
+                    p.normal_(0.0, 0.02, generator=gen)
+    return llm.eval(), drafter.eval()
+
+
+def prompts(device: str) -> torch.Tensor:
+    gen = torch.Generator(device="cpu").manual_seed(SEED)
+    return torch.randint(1, LLAMA_7B["vocab_size"], (BATCH, PROMPT), generator=gen).to(device)
+
+
+# -------------------------------------------------------------------------------------------------
+# GPU run
+# -------------------------------------------------------------------------------------------------
+def gpu_run(steps: int, warmup: int):
+    import recurrent_drafting_amd as rd
+    from recurrent_drafting_amd import _hip, attention
+
+    dev = "cuda:0"
+    t0 = time.perf_counter()
+    llm, drafter = build_models(dev, torch.bfloat16, LLAMA_7B["num_hidden_layers"], SEED)
+    torch.cuda.synchronize()
+    log(f"[bench] models on {torch.cuda.get_device_name(0)} in {time.perf_counter() - t0:.1f}s")
+    model = rd.RecurrentDrafting(llm, drafter)
+    ids = prompts(dev)
+    max_length = PROMPT + NEW_TOKENS
+
+    def new_stream(ledger):
+        return model.generate(ledger, ids, max_length, rd.BeamShape(WIDTH, LENGTH),
+                              rd.SamplingArgs(1.0, True), rd.SpecialTokens(0, None))
+
+    ledger = rd.stats.Ledger(sync=False)
+    stream = new_stream(ledger)
+    done = 0
+    for _ in range(warmup):
+        next(stream)
+        done += 1
+    torch.cuda.synchronize()
+
+    shapes = []
+    attention.shape_log = shapes
+    _hip.timing_enable(True)
+    elapsed, tokens, timed = 0.0, 0, 0
+    first_len = last_len = None
+    while timed < steps:
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        seg = 0
+        exhausted = False
+        while timed + seg < steps:
+            try:
+                out = next(stream)
+            except StopIteration:
+                exhausted = True
+                break
+            seg += 1
+            first_len = out.shape[1] if first_len is None else first_len
+            last_len = out.shape[1]
+        torch.cuda.synchronize()
+        elapsed += time.perf_counter() - start
+        timed += seg
+        if exhausted:  # generation reached its cap: start another one (prefill is not timed)
+            stream = new_stream(ledger)
+            for _ in range(warmup):
+                next(stream)
+    kernels = _hip.timing_collect()
+    _hip.timing_enable(False)
+    attention.shape_log = None
+    accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
+    # the generator that is still open has not posted its record yet; close it to flush
+    stream.close()
+    accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
+    per_seq_tokens = sum(a + 1 for a in accepted) / max(len(accepted), 1)
+    tokens = per_seq_tokens * BATCH * timed
+    no_pads = bool((out[:, 0] != 0).all())
+
+    # stage breakdown with the reference's synchronised timers, on a few extra steps
+    ledger2 = rd.stats.Ledger(sync=True)
+    s2 = new_stream(ledger2)
+    for _ in range(6):
+        next(s2)
+    s2.close()
+    wt = ledger2.records[0]["wall_times"]
+    stage = {k: sum(v[2:]) / len(v[2:]) for k, v in wt.items()}
+    ref_style = (per_seq_tokens) / (stage["generate_candidates"] + stage["verify_candidates"] + stage["accept_candidate_tokens"])
+
+    result = dict(
+        elapsed=elapsed, steps=timed, tokens=tokens, per_seq_tokens=per_seq_tokens, kernels=kernels,
+        shapes=shapes, stage=stage, ref_style_tokens_per_second=ref_style,
+        context=(first_len, last_len), no_pads=no_pads,
+    )
+    del model, llm, drafter
+    torch.cuda.empty_cache()
+    return result
+
+
+def attention_roofline(run):
+    """Algorithmic FLOPs of every verify-attention launch in the timed region over the summed
+    duration of attn_mfma_kernel: 4 * heads * head_dim * n_q * sum_b(keys_b) per launch."""
+    H, D = LLAMA_7B["num_attention_heads"], LLAMA_7B["hidden_size"] // LLAMA_7B["num_attention_heads"]
+    count, total_ms = run["kernels"].get("attn_mfma_kernel", (0, 0.0))
+    shapes = run["shapes"][:count] if count else []
+    flops = sum(4.0 * H * D * n_q * B * kv for (B, n_q, kv) in shapes)
+    if not count or total_ms <= 0:
+        return None
+    achieved = flops / (total_ms * 1e-3) / 1e12
+    k_bytes = sum(2.0 * H * D * 2 * B * kv + 2.0 * B * H * n_q * D * 2 for (B, n_q, kv) in shapes)
+    traffic = None
+    path = os.path.join(ROOT, "profiles", "attn_mfma_kernel_traffic.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+    return dict(
+        kernel="attn_mfma_kernel", bound="mfma", achieved=round(achieved, 2), peak=MFMA_BF16_PEAK_TFLOPS,
+        unit="TFLOP/s", frac=round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), traffic=traffic,
+        launches=count, avg_us=round(total_ms * 1e3 / count, 2),
+        algorithmic_gflop_per_launch=round(flops / count / 1e9, 3),
+        algorithmic_mb_per_launch=round(k_bytes / count / 1e6, 2),
+        hbm_frac_of_peak=round(k_bytes / (total_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+    )
+
+
+# -------------------------------------------------------------------------------------------------
+# CPU baseline: the torch restatement of one step on the host cores, bounded sample
+# -------------------------------------------------------------------------------------------------
+def cpu_baseline(per_seq_tokens: float):
+    from oracle import torch_path as P
+
+    threads = torch.get_num_threads()
+    a = torch.randn(1448, 4096).bfloat16()
+    w = torch.randn(4096, 4096).bfloat16()
+    torch.nn.functional.linear(a, w)
+    t = time.perf_counter()
+    torch.nn.functional.linear(a, w)
+    gflops = 2 * 1448 * 4096 * 4096 / (time.perf_counter() - t) / 1e9
+    layers = (2, 4) if gflops > 300 else (1, 2)
+    log(f"[bench] cpu baseline: {threads} threads, bf16 GEMM {gflops:.0f} GFLOP/s, sample layers {layers}")
+    gen = torch.Generator().manual_seed(SEED)
+    times = []
+    for n_layers in layers:
+        llm, drafter = build_models("cpu", torch.bfloat16, n_layers, SEED)
+        cache = P.Cache(BATCH, PROMPT + NEW_TOKENS + WIDTH * LENGTH, n_layers, 32, 128, torch.bfloat16, "cpu")
+        cache.data[:, :, :, :, :PROMPT] = torch.randn(cache.data[:, :, :, :, :PROMPT].shape, generator=gen).bfloat16()
+        cache.set_length(PROMPT)
+        ids = prompts("cpu")
+        ctx = torch.randn(BATCH, 4096, generator=gen).bfloat16()
+        tok = torch.randint(1, 32000, (BATCH,), generator=gen)
+        with torch.inference_mode():
+            t = time.perf_counter()
+            P.greedy_step(llm, drafter, ids, ctx, tok, cache, WIDTH, LENGTH, 0, tie="topk")
+            times.append(time.perf_counter() - t)
+        log(f"[bench] cpu step with {n_layers} layers: {times[-1]:.2f}s")
+        del llm, drafter, cache
+    per_layer = (times[1] - times[0]) / (layers[1] - layers[0])
+    full = times[0] + (LLAMA_7B["num_hidden_layers"] - layers[0]) * per_layer
+    return dict(
+        value=round(per_seq_tokens * BATCH / full, 3), unit="tokens/s", cores=threads, kind="port",
+        sample=(f"one decode step of the same workload (batch {BATCH}, context {PROMPT}, beam {WIDTH}x{LENGTH}, bf16) "
+                f"through the torch restatement with {layers[0]} and {layers[1]} of 32 layers "
+                f"({times[0]:.2f}s, {times[1]:.2f}s), extrapolated linearly to 32 layers = {full:.2f}s/step; "
+                f"tokens per step taken from the GPU run"),
+        seconds_per_step=round(full, 3),
+    )
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on ONE GPU (the decode step shards by batch row with no "
+            "exchange; see DESIGN.md); --gpus must be 1")
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible; the HIP path has no CPU fallback")
+        sys.exit(2)
+
+    import recurrent_drafting_amd  # noqa: F401  (fails loudly if the HIP library is missing)
+
+    run = gpu_run(args.steps, args.warmup)
+    value = run["tokens"] / run["elapsed"]
+    line = {
+        "metric": "tokens/sec on 1 MI355X, Vicuna-7B-shape bs8 bw45 bl5 bf16; verify-step us",
+        "value": round(value, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": run["steps"],
+        "warmup": args.warmup,
+        "ms_per_step": round(run["elapsed"] / run["steps"] * 1e3, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic (seeded uniform prompts, random-init N(0,0.02) weights)",
+        "config": {
+            "workload": "end-to-end greedy decode step, Vicuna-7B-shaped Llama + ReDrafter head, "
+                        "batch 8, prompt 500, beam 45x5, generation cap 2048",
+            "context_tokens": list(run["context"]),
+            "tokens_per_step_per_sequence": round(run["per_seq_tokens"], 3),
+        },
+        "verify_step_us": round(run["stage"]["verify_candidates"] * 1e6, 1),
+        "stage_seconds_synchronised": {k: round(v, 6) for k, v in run["stage"].items()},
+        "reference_style_tokens_per_second_per_sequence": round(run["ref_style_tokens_per_second"], 2),
+        "roofline": attention_roofline(run),
+        "kernel_avg_us": {k: round(ms * 1e3 / n, 2) for k, (n, ms) in sorted(run["kernels"].items())},
+    }
+    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(run["per_seq_tokens"])
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

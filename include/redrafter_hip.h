@@ -45,6 +45,14 @@ RD_API int rd_version(void);
 /* Message of the last failed call on this thread ("" if none). */
 RD_API const char* rd_last_error(void);
 
+/* Optional measurement aid, off by default.  rd_timing_enable(1) creates a pool of HIP events
+ * (the one place this library allocates) and makes every entry point bracket each of its kernel
+ * launches with two events on the launch stream; rd_timing_collect waits for them and writes one
+ * text line per kernel, "<kernel> <launches> <total_ms>", into a HOST buffer, then resets the
+ * pool.  rd_timing_enable(0) stops recording. */
+RD_API int rd_timing_enable(int on);
+RD_API int rd_timing_collect(char* out, size_t out_bytes);
+
 /* ------------------------------------------------------------------------------------------
  * Draft beams -> prefix tree -> packed tokens.
  * Replaces tree_attention._dedup_prefix (tree_attention.py:14-38), _get_unpacker (:125-188),

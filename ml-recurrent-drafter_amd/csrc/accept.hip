@@ -180,11 +180,11 @@ int launch_argmax(const void* x, int64_t rows, int64_t V, int64_t row_stride, in
   constexpr int VEC = 16 / sizeof(T);
   const bool vec_ok = ((uintptr_t)x % 16 == 0) && (row_stride % VEC == 0);
   if (vec_ok)
-    hipLaunchKernelGGL((argmax_rows_kernel<T, VEC>), dim3(rows), dim3(kThreads), 0, s,
-                       reinterpret_cast<const T*>(x), row_stride, V, out);
+    { rd::ScopedTiming rd_t("argmax_rows_kernel", s); hipLaunchKernelGGL((argmax_rows_kernel<T, VEC>), dim3(rows), dim3(kThreads), 0, s,
+                       reinterpret_cast<const T*>(x), row_stride, V, out); }
   else
-    hipLaunchKernelGGL((argmax_rows_kernel<T, 1>), dim3(rows), dim3(kThreads), 0, s,
-                       reinterpret_cast<const T*>(x), row_stride, V, out);
+    { rd::ScopedTiming rd_t("argmax_rows_kernel", s); hipLaunchKernelGGL((argmax_rows_kernel<T, 1>), dim3(rows), dim3(kThreads), 0, s,
+                       reinterpret_cast<const T*>(x), row_stride, V, out); }
   return rd::check_launch("rd_argmax_rows");
 }
 
@@ -220,9 +220,9 @@ extern "C" int rd_accept_greedy(const int64_t* beams, const int64_t* llm_tokens,
              "rd_accept_greedy: null pointer");
   RD_REQUIRE(unpacker || llm_row_stride >= (int64_t)width * length, RD_EINVAL,
              "rd_accept_greedy: llm_row_stride %lld < width*length", (long long)llm_row_stride);
-  hipLaunchKernelGGL(accept_greedy_kernel, dim3(batch), dim3(kThreads), 0, rd::as_stream(stream),
+  { rd::ScopedTiming rd_t("accept_greedy_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(accept_greedy_kernel, dim3(batch), dim3(kThreads), 0, rd::as_stream(stream),
                      beams, llm_tokens, llm_row_stride, unpacker, width, length, n_tokens_in_seq,
-                     seq_in_beam, next_token, last_slot);
+                     seq_in_beam, next_token, last_slot); }
   return rd::check_launch("rd_accept_greedy");
 }
 
@@ -245,12 +245,12 @@ extern "C" int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride,
              RD_EINVAL, "rd_realign_plan: null pointer");
   hipStream_t s = rd::as_stream(stream);
   int32_t* pads = plan + 4 + (size_t)batch * (4 + length);
-  hipLaunchKernelGGL(count_pads_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
-                     ids_row_stride, prev, pad_token_id, pads);
+  { rd::ScopedTiming rd_t("count_pads_kernel", s); hipLaunchKernelGGL(count_pads_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
+                     ids_row_stride, prev, pad_token_id, pads); }
   if (int e = rd::check_launch("rd_realign_plan(pads)")) return e;
-  hipLaunchKernelGGL(realign_plan_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
+  { rd::ScopedTiming rd_t("realign_plan_kernel", s); hipLaunchKernelGGL(realign_plan_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
                      ids_row_stride, prev, n_tokens_in_seq, seq_in_beam, beams, unpacker, batch,
-                     width, length, pad_token_id, pads, plan, new_ids);
+                     width, length, pad_token_id, pads, plan, new_ids); }
   return rd::check_launch("rd_realign_plan");
 }
 
@@ -262,7 +262,7 @@ extern "C" int rd_count_left_paddings(const int64_t* input_ids, int64_t ids_row_
   RD_REQUIRE((prev == 0 || input_ids) && pads, RD_EINVAL, "rd_count_left_paddings: null pointer");
   RD_REQUIRE(prev == 0 || ids_row_stride >= prev, RD_EINVAL,
              "rd_count_left_paddings: ids_row_stride < prev");
-  hipLaunchKernelGGL(count_pads_kernel, dim3(batch), dim3(kThreads), 0, rd::as_stream(stream),
-                     input_ids, ids_row_stride, prev, pad_token_id, pads);
+  { rd::ScopedTiming rd_t("count_pads_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(count_pads_kernel, dim3(batch), dim3(kThreads), 0, rd::as_stream(stream),
+                     input_ids, ids_row_stride, prev, pad_token_id, pads); }
   return rd::check_launch("rd_count_left_paddings");
 }

@@ -150,10 +150,10 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
   const int max_splits = rd::attn_max_splits(kv_len);
   int32_t* row_first = plan + RD_PLAN_HDR + 4 * (size_t)batch + 4 * (size_t)batch * max_splits;
   hipStream_t s = rd::as_stream(stream);
-  hipLaunchKernelGGL(mask_bits_kernel, dim3(n_q, batch), dim3(kThreads), 0, s, mask, mask_stride_b,
-                     mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first);
+  { rd::ScopedTiming rd_t("mask_bits_kernel", s); hipLaunchKernelGGL(mask_bits_kernel, dim3(n_q, batch), dim3(kThreads), 0, s, mask, mask_stride_b,
+                     mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first); }
   if (int e = rd::check_launch("rd_attn_prepare(bits)")) return e;
-  hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 0, s, row_first, batch, n_q, kv_len,
-                     words, rd::kAttnChunk, max_splits, plan);
+  { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 0, s, row_first, batch, n_q, kv_len,
+                     words, rd::kAttnChunk, max_splits, plan); }
   return rd::check_launch("rd_attn_prepare(plan)");
 }

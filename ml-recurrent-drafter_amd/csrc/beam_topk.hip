@@ -408,8 +408,8 @@ int launch_rows(const void* logits, int64_t row_stride, int rows, int V, const f
   constexpr int VEC = 16 / sizeof(T);
   const int per_thread = (V + kRowThreads - 1) / kRowThreads;
 #define RD_ROWS(ITEMS)                                                                              \
-  hipLaunchKernelGGL((beam_row_kernel<T, ITEMS>), dim3(rows), dim3(kRowThreads), 0, s, x, row_stride, \
-                     V, lpb, W, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback)
+  do { rd::ScopedTiming rd_t("beam_row_kernel", s); hipLaunchKernelGGL((beam_row_kernel<T, ITEMS>), dim3(rows), dim3(kRowThreads), 0, s, x, row_stride, \
+                     V, lpb, W, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback); } while (0)
   if (per_thread <= 8 && VEC <= 8) RD_ROWS(8);
   else if (per_thread <= 32) RD_ROWS(32);
   else RD_ROWS(64);
@@ -462,7 +462,7 @@ extern "C" int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, i
     default: e = launch_rows<__half>(logits, row_stride, rows, vocab, log_p_beam, width, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback, s); break;
   }
   if (e) return e;
-  hipLaunchKernelGGL(beam_merge_kernel, dim3(batch), dim3(kMergeThreads), 0, s, cs, ct, width, vocab,
-                     beams_in, t_len, new_log_p_beam, tokens, parents, beams_out);
+  { rd::ScopedTiming rd_t("beam_merge_kernel", s); hipLaunchKernelGGL(beam_merge_kernel, dim3(batch), dim3(kMergeThreads), 0, s, cs, ct, width, vocab,
+                     beams_in, t_len, new_log_p_beam, tokens, parents, beams_out); }
   return rd::check_launch("rd_beam_topk(merge)");
 }

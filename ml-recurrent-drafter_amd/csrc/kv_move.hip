@@ -153,10 +153,10 @@ extern "C" int rd_unpack_rows(const void* packed, int64_t packed_batch_stride_by
                         (uintptr_t)packed_batch_stride_bytes | (uintptr_t)out_batch_stride_bytes |
                         (uintptr_t)out_row_stride_bytes;
   const int vec = (all % 16 == 0) ? 16 : (all % 4 == 0 ? 4 : 1);
-  hipLaunchKernelGGL(gather_rows_kernel, dim3(n_out, batch), dim3(kThreads), 0,
+  { rd::ScopedTiming rd_t("gather_rows_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(gather_rows_kernel, dim3(n_out, batch), dim3(kThreads), 0,
                      rd::as_stream(stream), reinterpret_cast<const char*>(packed),
                      packed_batch_stride_bytes, row_bytes, index, index_batch_stride, n_src,
-                     reinterpret_cast<char*>(out), out_batch_stride_bytes, out_row_stride_bytes, vec);
+                     reinterpret_cast<char*>(out), out_batch_stride_bytes, out_row_stride_bytes, vec); }
   return rd::check_launch("rd_unpack_rows");
 }
 
@@ -177,9 +177,9 @@ extern "C" int rd_kv_unpack(void* cache, int n_layers, int batch, int n_heads, i
   if (chunk > row_bytes) chunk = row_bytes;
   const size_t lds = (size_t)n_src * chunk;
   const int64_t slabs = (int64_t)n_layers * 2 * batch * n_heads;
-  hipLaunchKernelGGL(kv_unpack_kernel, dim3(slabs), dim3(kThreads), lds, rd::as_stream(stream),
+  { rd::ScopedTiming rd_t("kv_unpack_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(kv_unpack_kernel, dim3(slabs), dim3(kThreads), lds, rd::as_stream(stream),
                      reinterpret_cast<char*>(cache), batch, n_heads, max_len, row_bytes, prev, index,
-                     n_out, n_src, (int)chunk);
+                     n_out, n_src, (int)chunk); }
   return rd::check_launch("rd_kv_unpack");
 }
 
@@ -195,7 +195,7 @@ extern "C" int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, 
   const size_t lds = (size_t)length * row_bytes;
   RD_REQUIRE(lds <= 64 * 1024, RD_ELIMIT, "rd_kv_compact: length*row_bytes %zu > 65536", lds);
   const int64_t slabs = (int64_t)n_layers * 2 * batch * n_heads;
-  hipLaunchKernelGGL(kv_compact_kernel, dim3(slabs), dim3(kThreads), lds, rd::as_stream(stream),
-                     reinterpret_cast<char*>(cache), batch, n_heads, max_len, row_bytes, plan, length);
+  { rd::ScopedTiming rd_t("kv_compact_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(kv_compact_kernel, dim3(slabs), dim3(kThreads), lds, rd::as_stream(stream),
+                     reinterpret_cast<char*>(cache), batch, n_heads, max_len, row_bytes, plan, length); }
   return rd::check_launch("rd_kv_compact");
 }

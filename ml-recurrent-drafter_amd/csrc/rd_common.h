@@ -24,6 +24,19 @@ inline int check_launch(const char* what) {
   return RD_OK;
 }
 
+// Optional per-kernel timing with HIP events on the launch stream (off by default; see
+// rd_timing_enable).  Wrap one launch:  { rd::ScopedTiming t("kernel_name", stream); launch; }
+struct ScopedTiming {
+  ScopedTiming(const char* name, hipStream_t stream);
+  ~ScopedTiming();
+  ScopedTiming(const ScopedTiming&) = delete;
+  ScopedTiming& operator=(const ScopedTiming&) = delete;
+
+ private:
+  hipStream_t stream_;
+  int slot_;
+};
+
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 

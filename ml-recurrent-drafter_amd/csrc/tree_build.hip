@@ -206,8 +206,8 @@ extern "C" int rd_causal_mask(const void* padding_mask, int pm_elem_bytes, int64
   hipStream_t s = rd::as_stream(stream);
   const dim3 grid((unsigned)query_len, batch);
 #define RD_LAUNCH_CM(T)                                                                     \
-  hipLaunchKernelGGL(causal_mask_kernel<T>, grid, dim3(kThreads), 0, s,                      \
-                     reinterpret_cast<const T*>(padding_mask), pm_row_stride, kv_len, query_len, mask)
+  do { rd::ScopedTiming rd_t("causal_mask_kernel", s); hipLaunchKernelGGL(causal_mask_kernel<T>, grid, dim3(kThreads), 0, s,                      \
+                     reinterpret_cast<const T*>(padding_mask), pm_row_stride, kv_len, query_len, mask); } while (0)
   if (pm_elem_bytes == 1) RD_LAUNCH_CM(uint8_t);
   else if (pm_elem_bytes == 4) RD_LAUNCH_CM(int32_t);
   else RD_LAUNCH_CM(int64_t);
@@ -244,12 +244,12 @@ extern "C" int rd_tree_build(const int64_t* beams, int batch, int width, int len
   int32_t* sel_idx = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) +
                                                 rd::align_up(n * sizeof(int64_t), 256));
   hipStream_t s = rd::as_stream(stream);
-  hipLaunchKernelGGL(tree_rows_kernel, dim3(batch), dim3(kThreads), 0, s, beams, width, length,
-                     prefix_tree, unpacker, sel_tok, sel_idx, counts);
+  { rd::ScopedTiming rd_t("tree_rows_kernel", s); hipLaunchKernelGGL(tree_rows_kernel, dim3(batch), dim3(kThreads), 0, s, beams, width, length,
+                     prefix_tree, unpacker, sel_tok, sel_idx, counts); }
   if (int e = rd::check_launch("rd_tree_build(rows)")) return e;
-  hipLaunchKernelGGL(tree_fill_kernel, dim3(batch), dim3(kThreads), 0, s, sel_tok, sel_idx, batch,
+  { rd::ScopedTiming rd_t("tree_fill_kernel", s); hipLaunchKernelGGL(tree_fill_kernel, dim3(batch), dim3(kThreads), 0, s, sel_tok, sel_idx, batch,
                      width * length, length, counts, packed_tokens, packed_token_indices,
-                     position_offsets);
+                     position_offsets); }
   return rd::check_launch("rd_tree_build(fill)");
 }
 
@@ -275,9 +275,9 @@ extern "C" int rd_tree_mask(const int64_t* unpacker, const int64_t* packed_token
   const dim3 grid(width * length, batch);
   const int WL = width * length;
 #define RD_LAUNCH_MASK(T)                                                                       \
-  hipLaunchKernelGGL(tree_mask_kernel<T>, grid, dim3(kThreads), 0, s, unpacker,                  \
+  do { rd::ScopedTiming rd_t("tree_mask_kernel", s); hipLaunchKernelGGL(tree_mask_kernel<T>, grid, dim3(kThreads), 0, s, unpacker,                  \
                      packed_token_indices, counts, reinterpret_cast<const T*>(padding_mask),    \
-                     pm_row_stride, prev, batch, WL, length, mask)
+                     pm_row_stride, prev, batch, WL, length, mask); } while (0)
   if (pm_elem_bytes == 1) RD_LAUNCH_MASK(uint8_t);
   else if (pm_elem_bytes == 4) RD_LAUNCH_MASK(int32_t);
   else RD_LAUNCH_MASK(int64_t);

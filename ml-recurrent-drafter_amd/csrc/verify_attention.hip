@@ -396,19 +396,19 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
     const int max_items = batch * a.max_splits;
     const int q_tiles = (n_q + kRowsPerWG - 1) / kRowsPerWG;
     RD_REQUIRE(max_items <= 65535 && q_tiles <= 65535, RD_ELIMIT, "rd_verify_attention: grid too large");
-    hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_heads, max_items, q_tiles), dim3(kMfmaThreads), 0, s, a);
+    { rd::ScopedTiming rd_t("attn_mfma_kernel", s); hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_heads, max_items, q_tiles), dim3(kMfmaThreads), 0, s, a); }
     if (int e = rd::check_launch("rd_verify_attention(mfma)")) return e;
     if (a.max_splits > 1) {
-      hipLaunchKernelGGL(attn_combine_kernel, dim3(n_q, n_heads, batch), dim3(kD), 0, s, a);
+      { rd::ScopedTiming rd_t("attn_combine_kernel", s); hipLaunchKernelGGL(attn_combine_kernel, dim3(n_q, n_heads, batch), dim3(kD), 0, s, a); }
       return rd::check_launch("rd_verify_attention(combine)");
     }
     return RD_OK;
   }
   const dim3 grid(n_q, n_heads, batch);
   switch (dtype) {
-    case RD_BF16: hipLaunchKernelGGL(attn_generic_kernel<__hip_bfloat16>, grid, dim3(kGenThreads), 0, s, a); break;
-    case RD_F16: hipLaunchKernelGGL(attn_generic_kernel<__half>, grid, dim3(kGenThreads), 0, s, a); break;
-    default: hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(kGenThreads), 0, s, a); break;
+    case RD_BF16: { rd::ScopedTiming rd_t("attn_generic_kernel", s); hipLaunchKernelGGL(attn_generic_kernel<__hip_bfloat16>, grid, dim3(kGenThreads), 0, s, a); } break;
+    case RD_F16: { rd::ScopedTiming rd_t("attn_generic_kernel", s); hipLaunchKernelGGL(attn_generic_kernel<__half>, grid, dim3(kGenThreads), 0, s, a); } break;
+    default: { rd::ScopedTiming rd_t("attn_generic_kernel", s); hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(kGenThreads), 0, s, a); } break;
   }
   return rd::check_launch("rd_verify_attention(generic)");
 }

@@ -23,6 +23,8 @@ _P, _I, _L, _Z, _F = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 _PROTOTYPES = {
     "rd_version": (C.c_int, []),
     "rd_last_error": (C.c_char_p, []),
+    "rd_timing_enable": (_I, [_I]),
+    "rd_timing_collect": (_I, [C.c_char_p, _Z]),
     "rd_tree_workspace_bytes": (_Z, [_I, _I, _I]),
     "rd_tree_build": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "rd_tree_mask": (_I, [_P, _P, _P, _P, _I, _L, _L, _I, _I, _I, _P, _P]),
@@ -101,3 +103,19 @@ def dtype_code(dt: torch.dtype) -> int:
         return _DTYPES[dt]
     except KeyError:
         raise TypeError(f"unsupported dtype {dt}; expected bfloat16, float16 or float32") from None
+
+
+def timing_enable(on: bool) -> None:
+    """Per-kernel HIP-event timing inside the library (a measurement aid; off by default)."""
+    check(lib().rd_timing_enable(int(on)))
+
+
+def timing_collect() -> dict:
+    """{kernel name: (launches, total milliseconds)} since the last call; waits for the events."""
+    buf = C.create_string_buffer(1 << 16)
+    check(lib().rd_timing_collect(buf, len(buf)))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, count, total = line.split()
+        out[name] = (int(count), float(total))
+    return out

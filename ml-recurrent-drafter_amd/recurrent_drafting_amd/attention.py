@@ -80,6 +80,11 @@ def prepare(mask: torch.Tensor, fix_empty_rows: bool = True) -> PreparedMask:
     return PreparedMask(bits.view(B, n_q, -1), plan, B, n_q, kv_len)
 
 
+# When set to a list, every masked_attention call appends (batch, n_q, kv_len): measurement
+# harnesses pair it with the library's per-kernel event timing to price the work that was done.
+shape_log: Optional[list] = None
+
+
 def _strides3(t: torch.Tensor):
     assert t.dim() == 4 and t.stride(3) == 1, "last dimension must be contiguous"
     return (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
@@ -112,6 +117,8 @@ def masked_attention(
     ws_bytes = lib.rd_attention_workspace_bytes(B, H, n_q, kv_len, D)
     if prepared.workspace is None or prepared.workspace.numel() < ws_bytes:
         prepared.workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
+    if shape_log is not None:
+        shape_log.append((B, n_q, kv_len))
     _hip.check(
         lib.rd_verify_attention(
             _hip.ptr(q), _strides3(q), _hip.ptr(k), _strides3(k), _hip.ptr(v), _strides3(v),
