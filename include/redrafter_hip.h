@@ -237,6 +237,49 @@ RD_API int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, int b
                         int64_t logp_row_stride, void* workspace, size_t workspace_bytes,
                         int force_fallback, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Speculative-sampling acceptance.
+ *
+ * rd_verify_row_stats: per row of (rows, vocab) verify logits, the four floats from which the
+ * log-probability of any token follows: {thr, zmax, log_sum, mask_z} with thr the top_k-th largest
+ * logit, and zmax / log_sum / mask_z the maximum, log-sum-exp and filter value of
+ * z = (logit >= thr ? logit : mask_value) / temperature, all in float32:
+ *     log P(token) = (logit >= thr ? logit / T : mask_z) - zmax - log_sum.
+ * Replaces warp_logits on the verify logits (recurrent_drafting.py:460) and
+ * (logits / T).log_softmax (:86) without writing either tensor.  stats: rows * 4 floats.
+ *
+ * Both functions below take log P either as a dense float32 tensor (log_p_dense with HOST element
+ * strides {batch, beam, position}, vocabulary contiguous; shape (batch, width, length, vocab)) or,
+ * with log_p_dense == NULL, as packed logits (batch, n_rows, vocab) of `dtype` with HOST strides
+ * {batch, row} + stats + unpacker.  log_q is the drafter's (batch, width, length-1, vocab) float32
+ * tensor with HOST strides {batch, beam, position}.
+ *
+ * rd_accept_sample: token k+1 of a beam is accepted when uniforms[b,i,k] < exp(P - Q) at that
+ * token; n = leading accepted run; first beam with the longest run.  Replaces
+ * _choose_from_candidates (recurrent_drafting.py:499-556); the caller draws the uniforms
+ * (torch.rand upstream, :545-547).
+ *
+ * rd_residual_probs: probs (batch, vocab) f32 = relu(exp P - exp Q) at position n of the chosen
+ * beam, or exp P at position length-1 when n == length-1.  Replaces the arithmetic of
+ * _prepare_next_input (recurrent_drafting.py:304-339); the draw itself stays with the caller.
+ * ------------------------------------------------------------------------------------------ */
+RD_API int rd_verify_row_stats(const void* logits, int dtype, int64_t row_stride, int64_t rows,
+                               int vocab, int top_k, float mask_value, float temperature,
+                               float* stats, int force_fallback, void* stream);
+RD_API int rd_accept_sample(const int64_t* beams, const float* log_p_dense,
+                            const int64_t* log_p_strides, const void* logits, int dtype,
+                            const int64_t* logits_strides, const float* stats, int n_rows,
+                            const int64_t* unpacker, float temperature, const float* log_q,
+                            const int64_t* log_q_strides, const float* uniforms, int batch,
+                            int width, int length, int vocab, int64_t* n_tokens_in_seq,
+                            int64_t* seq_in_beam, void* stream);
+RD_API int rd_residual_probs(const float* log_p_dense, const int64_t* log_p_strides,
+                             const void* logits, int dtype, const int64_t* logits_strides,
+                             const float* stats, int n_rows, const int64_t* unpacker,
+                             float temperature, const float* log_q, const int64_t* log_q_strides,
+                             const int64_t* seq_in_beam, const int64_t* n_tokens_in_seq, int batch,
+                             int width, int length, int vocab, float* probs, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,104 +23,12 @@
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
-#include "rd_common.h"
+#include "row_select.h"
 
 namespace {
 
-constexpr int kRowThreads = 1024;
-constexpr int kRowWaves = kRowThreads / 64;
-constexpr int kCap = 2048;       // LDS candidate list
 constexpr int kMaxWidth = 64;    // beam width limit of the merge kernel (W*W <= 4096 LDS keys)
 constexpr int kMergeThreads = 256;
-
-template <typename T> struct Num;
-template <> struct Num<float> {
-  static __device__ float load(const float* p) { return *p; }
-  static __device__ float round(float v) { return v; }
-};
-template <> struct Num<__hip_bfloat16> {
-  static __device__ float load(const __hip_bfloat16* p) { return __bfloat162float(*p); }
-  static __device__ float round(float v) { return __bfloat162float(__float2bfloat16(v)); }
-};
-template <> struct Num<__half> {
-  static __device__ float load(const __half* p) { return __half2float(*p); }
-  static __device__ float round(float v) { return __half2float(__float2half(v)); }
-};
-
-// Monotone map float -> uint32 (larger float, larger integer; -inf lowest of the finite order).
-__device__ inline uint32_t ord(float f) {
-  const uint32_t u = __float_as_uint(f);
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-__device__ inline float unord(uint32_t k) {
-  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
-}
-// (score desc, index asc) as one integer: larger key = earlier in the result.
-__device__ inline uint64_t key64(float score, uint32_t idx) {
-  return ((uint64_t)ord(score) << 32) | (uint64_t)(0xffffffffu - idx);
-}
-
-__device__ inline float wave_max(float v) {
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-  return v;
-}
-__device__ inline float wave_sum(float v) {
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-  return v;
-}
-
-struct RowShared {
-  float cval[kCap];
-  int cidx[kCap];
-  float red[kRowWaves];
-  unsigned long long red64[kRowWaves];
-  int ired[kRowWaves];
-  int count;
-  int n_surv;
-  float thr;
-  float logsum;
-};
-
-__device__ inline float block_max(float v, RowShared& sh) {
-  v = wave_max(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float r = sh.red[0];
-  for (int w = 1; w < kRowWaves; ++w) r = fmaxf(r, sh.red[w]);
-  return r;
-}
-__device__ inline float block_min(float v, RowShared& sh) { return -block_max(-v, sh); }
-__device__ inline float block_sum(float v, RowShared& sh) {
-  v = wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float r = 0.f;
-  for (int w = 0; w < kRowWaves; ++w) r += sh.red[w];  // fixed order
-  return r;
-}
-__device__ inline int block_isum(int v, RowShared& sh) {
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sh.ired[threadIdx.x >> 6] = v;
-  __syncthreads();
-  int r = 0;
-  for (int w = 0; w < kRowWaves; ++w) r += sh.ired[w];
-  return r;
-}
-__device__ inline uint64_t block_max64(uint64_t v, RowShared& sh) {
-  for (int off = 32; off > 0; off >>= 1) {
-    const uint64_t o = __shfl_xor(v, off);
-    v = o > v ? o : v;
-  }
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) sh.red64[threadIdx.x >> 6] = v;
-  __syncthreads();
-  uint64_t r = sh.red64[0];
-  for (int w = 1; w < kRowWaves; ++w) r = sh.red64[w] > r ? sh.red64[w] : r;
-  return r;
-}
 
 // ITEMS elements per thread, held as ITEMS/VEC vectors of VEC = 16 bytes / sizeof(T).
 template <typename T, int ITEMS>

@@ -45,6 +45,15 @@ _PROTOTYPES = {
         [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P, _Z, _I, _P],
     ),
     "rd_causal_mask": (_I, [_P, _I, _L, _I, _L, _L, _P, _P]),
+    "rd_verify_row_stats": (_I, [_P, _I, _L, _L, _I, _I, _F, _F, _P, _I, _P]),
+    "rd_accept_sample": (
+        _I,
+        [_P, _P, _P, _P, _I, _P, _P, _I, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P],
+    ),
+    "rd_residual_probs": (
+        _I,
+        [_P, _P, _P, _I, _P, _P, _I, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P],
+    ),
     "rd_beam_topk_workspace_bytes": (_Z, [_I, _I]),
     "rd_beam_topk": (
         _I,
@@ -119,3 +128,16 @@ def timing_collect() -> dict:
         name, count, total = line.split()
         out[name] = (int(count), float(total))
     return out
+
+
+def aligned_rows(x: torch.Tensor) -> torch.Tensor:
+    """(rows, V) view whose rows start on 16-byte boundaries (the row kernels load 16-byte vectors).
+    Already-aligned tensors pass through; others are copied into a padded buffer once."""
+    es = x.element_size()
+    if x.stride(1) == 1 and (x.stride(0) * es) % 16 == 0 and x.data_ptr() % 16 == 0:
+        return x
+    rows, v = x.shape
+    per = 16 // es
+    padded = torch.empty((rows, (v + per - 1) // per * per), dtype=x.dtype, device=x.device)
+    padded[:, :v] = x
+    return padded[:, :v]

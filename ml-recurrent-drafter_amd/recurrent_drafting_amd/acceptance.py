@@ -163,3 +163,111 @@ def _update_kv_cache_and_input_ids(
 ) -> torch.Tensor:
     """Drop-in for recurrent_drafting.py:114-232: expects the cache unpacked by Cache.unpack."""
     return realign(input_ids, n_tokens_in_seq, seq_in_beam, beams, cache, pad_token_id)
+
+
+# ---------------------------------------------------------------------------------------------
+# speculative sampling
+# ---------------------------------------------------------------------------------------------
+import ctypes as _C  # noqa: E402
+from dataclasses import dataclass  # noqa: E402
+
+from . import modeling_drafter as _md  # noqa: E402
+
+
+def _host_strides(t: torch.Tensor, n: int):
+    assert t.stride(-1) == 1, "vocabulary dimension must be contiguous"
+    return (_C.c_int64 * n)(*[t.stride(i) for i in range(n)])
+
+
+@dataclass
+class PackedLogP:
+    """LLM log-probabilities in packed form: logits (B, n, V) + 4 floats per packed row."""
+
+    logits: torch.Tensor
+    stats: torch.Tensor  # (B, n, 4) float32
+    unpacker: torch.Tensor  # (B, W, L) int64
+    temperature: float
+
+
+def verify_row_stats(logits: torch.Tensor, temperature: float, force_fallback: bool = False) -> torch.Tensor:
+    """(B, n, V) verify logits -> (B, n, 4) float32 {thr, zmax, log_sum, mask_z}."""
+    B, n, V = logits.shape
+    x = _hip.aligned_rows(logits.reshape(B * n, V))
+    stats = torch.empty((B, n, 4), dtype=torch.float32, device=logits.device)
+    _hip.check(
+        _hip.lib().rd_verify_row_stats(
+            _hip.ptr(x), _hip.dtype_code(x.dtype), x.stride(0), B * n, V, _md.TOP_K, _md.LOG_0,
+            float(temperature), _hip.ptr(stats), int(force_fallback), _hip.stream(),
+        )
+    )
+    return stats
+
+
+def _p_args(log_p):
+    """Argument block (dense, dense_strides, logits, dtype, logits_strides, stats, n_rows, unpacker, T)."""
+    if isinstance(log_p, PackedLogP):
+        lg = log_p.logits
+        assert lg.dim() == 3
+        keep = (lg, log_p.stats, log_p.unpacker.contiguous())
+        return keep, (None, None, _hip.ptr(lg), _hip.dtype_code(lg.dtype), _host_strides(lg, 2),
+                      _hip.ptr(log_p.stats), lg.shape[1], _hip.ptr(keep[2]), float(log_p.temperature))
+    assert log_p.dim() == 4 and log_p.dtype == torch.float32
+    return (log_p,), (_hip.ptr(log_p), _host_strides(log_p, 3), None, 0, None, None, 0, None, 1.0)
+
+
+def sample_accept(beams, log_p, log_q, uniforms) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(n_tokens_in_seq, seq_in_beam) with caller-supplied uniforms (B, W, L-1).
+
+    log_p: dense (B, W, L, V) float32 or PackedLogP; log_q: (B, W, L-1, V) float32."""
+    B, W, L = beams.shape
+    V = log_q.shape[-1]
+    assert beams.dtype in (torch.int32, torch.int64)
+    beams = beams.to(torch.long).contiguous()
+    assert log_q.shape == (B, W, L - 1, V) and log_q.dtype == torch.float32
+    uniforms = uniforms.to(torch.float32).contiguous()
+    assert uniforms.shape == (B, W, L - 1)
+    keep, p_args = _p_args(log_p)
+    out = torch.empty((2, B), dtype=torch.long, device=beams.device)
+    _hip.check(
+        _hip.lib().rd_accept_sample(
+            _hip.ptr(beams), *p_args, _hip.ptr(log_q), _host_strides(log_q, 3), _hip.ptr(uniforms),
+            B, W, L, V, _hip.ptr(out[0]), _hip.ptr(out[1]), _hip.stream(),
+        )
+    )
+    return out[0], out[1]
+
+
+def residual_probs(log_q, log_p, seq_in_beam, n_tokens_in_seq) -> torch.Tensor:
+    """Unnormalised distribution of the next token, (B, V) float32."""
+    B, W, Lm1, V = log_q.shape
+    keep, p_args = _p_args(log_p)
+    seq_in_beam = seq_in_beam.to(torch.long).contiguous()
+    n_tokens_in_seq = n_tokens_in_seq.to(torch.long).contiguous()
+    probs = torch.empty((B, V), dtype=torch.float32, device=log_q.device)
+    _hip.check(
+        _hip.lib().rd_residual_probs(
+            *p_args, _hip.ptr(log_q), _host_strides(log_q, 3), _hip.ptr(seq_in_beam),
+            _hip.ptr(n_tokens_in_seq), B, W, Lm1 + 1, V, _hip.ptr(probs), _hip.stream(),
+        )
+    )
+    return probs
+
+
+def _choose_from_candidates(beams, log_probs_by_llm, log_probs_by_drafter):
+    """Drop-in for recurrent_drafting.py:499-556: draws torch.rand like the reference does."""
+    B, W, L = beams.shape
+    u = torch.rand((B, W, L - 1), device=log_probs_by_drafter.device)
+    return sample_accept(beams, log_probs_by_llm.float(), log_probs_by_drafter.float(), u)
+
+
+def _prepare_next_input(log_probs_by_drafter, log_probs_by_llm, last_hidden_state, seq_in_beam,
+                        n_tokens_in_seq):
+    """Drop-in for recurrent_drafting.py:271-343: (context (B, hidden), next_tokens (B,))."""
+    import torch.distributions as dist
+
+    probs = residual_probs(log_probs_by_drafter.float(), log_probs_by_llm.float(), seq_in_beam, n_tokens_in_seq)
+    next_tokens = dist.Categorical(probs=probs).sample()
+    B, W, L = last_hidden_state.shape[:3]
+    flat = (seq_in_beam * L + n_tokens_in_seq).to(torch.long)
+    state = _select_one_per_row(last_hidden_state.reshape(B, W * L, -1), flat)
+    return state, next_tokens

@@ -81,12 +81,7 @@ def beam_topk_step(
     B, W, V = logits.shape
     assert log_p_beam.dtype == torch.float32 and log_p_beam.shape == (B, W)
     assert beams.dtype == torch.long and beams.shape[:2] == (B, W)
-    x = logits.reshape(B * W, V)
-    if x.stride(1) != 1 or (x.stride(0) * x.element_size()) % 16 or x.data_ptr() % 16:
-        x = x.contiguous()
-        if (V * x.element_size()) % 16:  # pad rows to a 16-byte multiple
-            pad = (-V) % (16 // x.element_size())
-            x = torch.nn.functional.pad(x, (0, pad), value=float("-inf"))[:, :V]
+    x = _hip.aligned_rows(logits.reshape(B * W, V))
     beams = beams.contiguous()
     log_p_beam = log_p_beam.contiguous()
     t = beams.shape[2]

@@ -6,8 +6,11 @@
     draft   beam search on the drafter head          rd_beam_topk x (L-1)      (+ torch GEMMs)
     verify  beams -> prefix tree, mask, LLM forward   rd_tree_build, rd_tree_mask, rd_attn_prepare,
                                                       rd_verify_attention per layer (+ torch GEMMs)
-    accept  argmax over the packed rows, longest      rd_argmax_rows, rd_accept_greedy,
-            agreeing prefix, ids and KV re-aligned    rd_realign_plan, rd_kv_compact
+    accept  greedy: argmax over the packed rows,      rd_argmax_rows, rd_accept_greedy
+            longest agreeing prefix
+            sampling: row statistics of the packed    rd_verify_row_stats, rd_accept_sample,
+            logits, u < P/Q run, residual resample    rd_residual_probs
+            ids and KV re-aligned                     rd_realign_plan, rd_kv_compact
 
 Greedy decoding never materialises the (B, W, L, V) logits, never unpacks the KV cache into W*L
 slots and never clones it: argmax commutes with the unpack and with the top-50 filter, and the
@@ -29,9 +32,11 @@ import transformers
 
 from . import acceptance, attention, kv_cache, modeling_drafter, modeling_llama, stats, tree_attention
 from .acceptance import (  # noqa: F401  (re-exported: the reference's helper names)
+    _choose_from_candidates,
     _count_left_paddings,
     _greedy_choose_from_candidates,
     _greedy_prepare_next_input,
+    _prepare_next_input,
     _select_one_per_row,
     _update_kv_cache_and_input_ids,
 )
@@ -101,6 +106,37 @@ def _verify_candidates(
     return hidden, logits
 
 
+def _greedy_accept_candidate_tokens(input_ids, beams_by_drafter, logits_by_llm, last_hidden_state,
+                                    cache, pad_token_id, step_record):
+    """Drop-in for recurrent_drafting.py:43-72 (unpacked logits and hidden states, unpacked cache)."""
+    beams_by_llm = acceptance.argmax_rows(logits_by_llm)
+    with step_record.time("choose_from_candidates"):
+        n_tokens, seq_in_beam = _greedy_choose_from_candidates(beams_by_drafter, beams_by_llm)
+    with step_record.time("update_kv_cache_and_input_ids"):
+        input_ids = _update_kv_cache_and_input_ids(
+            input_ids, n_tokens, seq_in_beam, beams_by_drafter, cache, pad_token_id)
+    with step_record.time("greedy_prepare_next_input"):
+        state, next_tokens = _greedy_prepare_next_input(
+            beams_by_llm, last_hidden_state, seq_in_beam, n_tokens)
+    return state, input_ids, next_tokens, n_tokens
+
+
+def _accept_candidate_tokens(input_ids, beams, log_probs_by_drafter, logits_by_llm,
+                             last_hidden_state, cache, pad_token_id, temperature, step_record):
+    """Drop-in for recurrent_drafting.py:75-111.  This form materialises the (B, W, L, V)
+    log-softmax like the reference; `generate` uses the packed form instead."""
+    log_probs_by_llm = (logits_by_llm / temperature).log_softmax(dim=-1)
+    with step_record.time("choose_from_candidates"):
+        n_tokens, seq_in_beam = _choose_from_candidates(beams, log_probs_by_llm, log_probs_by_drafter)
+    with step_record.time("update_kv_cache_and_input_ids"):
+        input_ids = _update_kv_cache_and_input_ids(
+            input_ids, n_tokens, seq_in_beam, beams, cache, pad_token_id)
+    with step_record.time("prepare_next_input"):
+        state, next_tokens = _prepare_next_input(
+            log_probs_by_drafter, log_probs_by_llm, last_hidden_state, seq_in_beam, n_tokens)
+    return state, input_ids, next_tokens, n_tokens
+
+
 class RecurrentDrafting(torch.nn.Module):
     def __init__(self, llm: transformers.PreTrainedModel, drafter: modeling_drafter.Drafter):
         super().__init__()
@@ -158,13 +194,44 @@ class RecurrentDrafting(torch.nn.Module):
                 context = tree_attention.gather_rows(hidden, last_slot.unsqueeze(-1))[:, 0, :]
         return context, input_ids, next_tokens, n_tokens
 
+    # -- one speculative-sampling step on the fused path ------------------------------------------
+    def _sampling_step(self, step_record, input_ids, context, init_tokens, cache, beam_shape, pad,
+                       temperature):
+        llm = self.llm
+        with step_record.time("generate_candidates"):
+            beams, log_q = self.drafter.beam_search_candidates(
+                context, init_tokens, llm.base_model.get_input_embeddings(), beam_shape)
+        with step_record.time("verify_candidates"):
+            prev = input_ids.shape[1]
+            tree = tree_attention.build_tree(beams)
+            mask = tree_attention.build_mask(tree, input_ids != pad)
+            pads = _count_left_paddings(input_ids, pad)
+            position_ids = (prev - pads).unsqueeze(-1) + tree.position_offsets
+            with step_record.time("base_forward"):
+                hidden = llm.hidden_states(tree.packed_beams, mask, position_ids, cache.sliced)
+                logits = llm.lm_head(hidden)
+        with step_record.time("accept_candidate_tokens"):
+            # four floats per packed row stand in for the filtered, tempered log-softmax tensors
+            log_p = acceptance.PackedLogP(
+                logits, acceptance.verify_row_stats(logits, temperature), tree.unpacker, temperature)
+            with step_record.time("choose_from_candidates"):
+                B, W, L = beams.shape
+                uniforms = torch.rand((B, W, L - 1), device=beams.device)
+                n_tokens, seq_in_beam = acceptance.sample_accept(beams, log_p, log_q, uniforms)
+            with step_record.time("update_kv_cache_and_input_ids"):
+                input_ids = acceptance.realign(
+                    input_ids, n_tokens, seq_in_beam, beams, cache, pad, unpacker=tree.unpacker)
+            with step_record.time("prepare_next_input"):
+                probs = acceptance.residual_probs(log_q, log_p, seq_in_beam, n_tokens)
+                next_tokens = dist.Categorical(probs=probs).sample()
+                rows = torch.arange(B, device=beams.device)
+                last_slot = tree.unpacker[rows, seq_in_beam, n_tokens]
+                context = tree_attention.gather_rows(hidden, last_slot.unsqueeze(-1))[:, 0, :]
+        return context, input_ids, next_tokens, n_tokens
+
     def _generate(self, text_generation, input_ids, max_length, beam_shape, sampling_args,
                   special_tokens) -> Generator[torch.Tensor, None, None]:
         assert input_ids.dtype == torch.long, f"input_ids.dtype {input_ids.dtype} is not long"
-        if not sampling_args.greedy:
-            raise NotImplementedError(
-                "speculative sampling is not on the HIP path yet; use SamplingArgs(greedy=True)"
-            )
         batch_size, seq_len = input_ids.shape
         init_seq_len = seq_len
         cfg = self.llm.config
@@ -182,10 +249,16 @@ class RecurrentDrafting(torch.nn.Module):
         )
         while seq_len < max_length:
             with text_generation.step() as step_record:
-                context, input_ids, init_tokens, n_tokens = self._greedy_step(
-                    step_record, input_ids, context, init_tokens, cache, beam_shape,
-                    special_tokens.pad,
-                )
+                if sampling_args.greedy:
+                    context, input_ids, init_tokens, n_tokens = self._greedy_step(
+                        step_record, input_ids, context, init_tokens, cache, beam_shape,
+                        special_tokens.pad,
+                    )
+                else:
+                    context, input_ids, init_tokens, n_tokens = self._sampling_step(
+                        step_record, input_ids, context, init_tokens, cache, beam_shape,
+                        special_tokens.pad, sampling_args.temperature,
+                    )
                 output_tokens = torch.cat((input_ids, init_tokens.unsqueeze(-1)), dim=-1)
                 seq_len = output_tokens.shape[1]
                 step_record.set(

@@ -326,6 +326,49 @@ def greedy_step(llm, drafter, input_ids, context, init_tokens, cache: Cache, wid
     return context, input_ids, next_tokens, n_tokens, beams
 
 
+def sample_choose(beams, log_p_llm, log_q_drafter, uniforms):
+    """recurrent_drafting.py:532-556 with the uniforms supplied by the caller."""
+    tok = beams[..., 1:, None]
+    q = log_q_drafter.gather(-1, tok).squeeze(-1)
+    p = log_p_llm[:, :, :-1, :].gather(-1, tok).squeeze(-1)
+    ok = uniforms < torch.exp(p - q)
+    run = (ok.long().cumsum(-1) == torch.arange(1, ok.shape[-1] + 1, device=ok.device)).sum(-1)
+    best = run.max(dim=-1)
+    return best.values, best.indices
+
+
+def residual_distribution(log_q_drafter, log_p_llm, seq_in_beam, n_tokens):
+    """Unnormalised next-token distribution (recurrent_drafting.py:304-339)."""
+    B, W, Lm1, V = log_q_drafter.shape
+    rows = torch.arange(B, device=log_q_drafter.device)
+    q_sel, p_sel = log_q_drafter[rows, seq_in_beam], log_p_llm[rows, seq_in_beam]
+    whole = (n_tokens == Lm1)[:, None]
+    idx = n_tokens - (n_tokens == Lm1).long()
+    resid = torch.relu(torch.exp(p_sel[rows, idx]) - torch.exp(q_sel[rows, idx]))
+    return torch.where(whole, torch.exp(p_sel[:, -1]), resid)
+
+
+def sampling_step(llm, drafter, input_ids, context, init_tokens, cache: Cache, width, length, pad,
+                  temperature, draw_uniforms, draw_token, tie: str = "stable"):
+    """One speculative-sampling step (recurrent_drafting.py:75-111, :437-465).  draw_uniforms(shape)
+    and draw_token(probs) stand in for torch.rand and Categorical(probs).sample()."""
+    beams, log_q = beam_search(drafter, llm.model.embed_tokens, context, init_tokens, width, length, tie=tie)
+    packed, unpacker, mask, offsets = pack(beams, (input_ids != pad).to(input_ids.dtype))
+    prev = input_ids.shape[1]
+    pos = (prev - count_left_pads(input_ids, pad))[:, None] + offsets
+    logits, hidden = llama_forward(llm, packed, mask, pos, cache)
+    logits = unpack(top_k_filter(logits), unpacker)
+    hidden = unpack(hidden, unpacker)
+    cache.unpack(prev, unpacker)
+    log_p = (logits / temperature).log_softmax(dim=-1)
+    n_tokens, seq_in_beam = sample_choose(beams, log_p, log_q, draw_uniforms(log_q.shape[:3]))
+    input_ids = realign(input_ids, n_tokens, seq_in_beam, beams, cache, pad)
+    next_tokens = draw_token(residual_distribution(log_q, log_p, seq_in_beam, n_tokens))
+    rows = torch.arange(beams.shape[0], device=beams.device)
+    context = hidden[rows, seq_in_beam, n_tokens]
+    return context, input_ids, next_tokens, n_tokens, beams
+
+
 def generate_greedy(llm, drafter, input_ids, max_length: int, width: int, length: int, pad: int = 0,
                     eos: Optional[int] = 1, tie: str = "stable") -> Generator[Tuple[torch.Tensor, torch.Tensor], None, None]:
     """Yields (output tokens (B, <=max_length), n_tokens_in_seq (B,)) after every step."""
@@ -339,6 +382,31 @@ def generate_greedy(llm, drafter, input_ids, max_length: int, width: int, length
         while seq_len < max_length:
             context, input_ids, tokens, n_tokens, _ = greedy_step(
                 llm, drafter, input_ids, context, tokens, cache, width, length, pad, tie)
+            out = torch.cat((input_ids, tokens[:, None]), dim=-1)
+            seq_len = out.shape[1]
+            yield out[:, :max_length], n_tokens
+            if eos is not None and bool(((out[:, S:] == eos).sum(dim=-1) > 0).all()):
+                break
+
+
+def generate_sampling(llm, drafter, input_ids, max_length: int, width: int, length: int, temperature: float,
+                      draw_uniforms, draw_token, pad: int = 0, eos: Optional[int] = 1, tie: str = "stable"):
+    """Speculative-sampling decode loop; yields (output tokens, n_tokens_in_seq) per step."""
+    with torch.inference_mode():
+        B, S = input_ids.shape
+        cfg = llm.config
+        cache = Cache(B, max_length + width * length, cfg.num_hidden_layers, cfg.num_key_value_heads,
+                      cfg.hidden_size // cfg.num_attention_heads, llm.lm_head.weight.dtype, input_ids.device)
+        mask = causal_mask(input_ids != pad, S)
+        pos = torch.arange(S, device=input_ids.device).expand(input_ids.shape) - count_left_pads(input_ids, pad)[:, None]
+        logits, hidden = llama_forward(llm, input_ids, mask, pos, cache)
+        context = hidden[:, -1, :]
+        tokens = draw_token(torch.softmax(top_k_filter(logits[:, -1, :]) / temperature, dim=-1))
+        seq_len = S
+        while seq_len < max_length:
+            context, input_ids, tokens, n_tokens, _ = sampling_step(
+                llm, drafter, input_ids, context, tokens, cache, width, length, pad, temperature,
+                draw_uniforms, draw_token, tie)
             out = torch.cat((input_ids, tokens[:, None]), dim=-1)
             seq_len = out.shape[1]
             yield out[:, :max_length], n_tokens

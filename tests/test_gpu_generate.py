@@ -83,12 +83,3 @@ def test_generate_matches_torch_restatement_on_gpu_bigger_model():
     steps, _ = _run(llm, drafter, ids, 300 + 12, 12, 5)
     want = [t.cpu().tolist() for t, _ in P.generate_greedy(llm, drafter, ids.cuda(), 300 + 12, 12, 5, pad=0, eos=None)]
     assert steps == want
-
-
-def test_sampling_is_refused_loudly():
-    import recurrent_drafting_amd as rd
-
-    llm, drafter = _models(tm.draw(tm.llama_shapes(), 1), tm.draw(tm.drafter_shapes(), 2))
-    model = rd.RecurrentDrafting(llm, drafter)
-    with pytest.raises(NotImplementedError):
-        next(model.generate(rd.stats.Ledger(), tm.prompt(1, 4, 1000, 0).cuda(), 8, rd.BeamShape(2, 2), rd.SamplingArgs(1.0, False)))

@@ -110,3 +110,21 @@ def test_generate_matches_reference_token_streams(ref_vectors, case_index):
     steps = [t.tolist() for t, _ in P.generate_greedy(
         llm, drafter, ids, c["prompt_len"] + c["new_tokens"], c["W"], c["L"], pad=0, eos=None)]
     assert steps == case["steps"]
+
+
+@pytest.mark.parametrize("B,W,L", [(1, 1, 2), (4, 4, 4), (13, 13, 13)])
+def test_sampling_helpers_match_numpy_oracle(B, W, L):
+    """Injected uniforms, as the reference's cross-implementation test does."""
+    rng = np.random.default_rng(123)
+    V = 3
+    beams = rng.integers(0, V, size=(B, W, L))
+    lp = rng.uniform(-10, 0, size=(B, W, L, V))
+    lq = rng.uniform(-10, 0, size=(B, W, L - 1, V))
+    u = rng.random((B, W, L - 1))
+    n, s = P.sample_choose(torch.tensor(beams), torch.tensor(lp), torch.tensor(lq), torch.tensor(u))
+    on, os_ = Acc.sample_choose(beams, lp, lq, u)
+    assert np.array_equal(n.numpy(), on) and np.array_equal(s.numpy(), os_)
+    s2 = rng.integers(0, W, size=B)
+    n2 = rng.integers(0, L, size=B)
+    got = P.residual_distribution(torch.tensor(lq), torch.tensor(lp), torch.tensor(s2), torch.tensor(n2))
+    assert np.allclose(got.numpy(), Acc.residual_probs(lq, lp, s2, n2), atol=1e-12)
