@@ -176,7 +176,8 @@ RD_API int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, int6
  * given as 0/1 bytes with element strides mask_stride_b / mask_stride_q (keys contiguous), into
  * bits: rd_attn_bits_words() uint64, one word per (row, 64 keys); and writes the work plan
  * (rd_attn_plan_ints() int32): per batch row the first key any query attends to and the split of
- * its keys into work items.  fix_empty_rows != 0 turns a row that attends to nothing into a row
+ * its keys into work items; n_heads (query heads of the attention that will use the plan) sizes
+ * the items to one compute unit's share of the whole call.  fix_empty_rows != 0 turns a row that attends to nothing into a row
  * that attends to everything, which is what attention.set_sdpa_fully_masked_rows
  * (attention.py:58-72) does and what a finite-minimum additive bias amounts to.
  *
@@ -192,8 +193,8 @@ RD_API int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, int6
 RD_API size_t rd_attn_plan_ints(int batch, int n_q, int kv_len);
 RD_API size_t rd_attn_bits_words(int batch, int n_q, int kv_len);
 RD_API int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64_t mask_stride_q,
-                           int batch, int n_q, int kv_len, int fix_empty_rows, uint64_t* bits,
-                           int32_t* plan, void* stream);
+                           int batch, int n_q, int kv_len, int n_heads, int fix_empty_rows,
+                           uint64_t* bits, int32_t* plan, void* stream);
 RD_API size_t rd_attention_workspace_bytes(int batch, int n_heads, int n_q, int kv_len,
                                            int head_dim);
 RD_API int rd_verify_attention(const void* q, const int64_t* q_strides, const void* k,

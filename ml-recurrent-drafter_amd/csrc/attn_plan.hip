@@ -47,9 +47,11 @@ __global__ __launch_bounds__(kThreads) void mask_bits_kernel(
 
 __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __restrict__ row_first,
                                                              int B, int n_q, int kv_len, int words,
-                                                             int chunk, int max_splits,
+                                                             int min_chunk, int max_splits,
+                                                             int n_heads, int n_cu,
                                                              int32_t* __restrict__ plan) {
   __shared__ int s_n_items;
+  __shared__ int s_chunk;
   int32_t* per_row = plan + RD_PLAN_HDR;
   int32_t* items = plan + RD_PLAN_HDR + 4 * B;
   // pass 1: per batch row, first attended key and number of splits
@@ -59,13 +61,26 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
       const int f = row_first[(int64_t)b * n_q + q];
       first = f < first ? f : first;
     }
-    const int begin = (first / 64) * 64;
-    const int live = kv_len - begin;
-    int splits = (live + chunk - 1) / chunk;
-    splits = splits < 1 ? 1 : (splits > max_splits ? max_splits : splits);
-    per_row[4 * b + 0] = begin;
-    per_row[4 * b + 1] = splits;
+    per_row[4 * b + 0] = (first / 64) * 64;
     per_row[4 * b + 3] = 0;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    // Keys per work item: one compute unit's even share of all (row, head) work, but never below
+    // min_chunk.  Equal rows on a machine with batch*heads == compute units are then not split at
+    // all (no partials to merge); ragged rows are cut so that the longest item is about one share.
+    long long total = 0;
+    for (int b = 0; b < B; ++b) total += kv_len - per_row[4 * b + 0];
+    long long share = (total * n_heads + n_cu - 1) / n_cu;
+    share = (share + 63) / 64 * 64;
+    s_chunk = (int)(share > min_chunk ? share : min_chunk);
+  }
+  __syncthreads();
+  const int chunk = s_chunk;
+  for (int b = threadIdx.x; b < B; b += kThreads) {
+    const int live = kv_len - per_row[4 * b + 0];
+    int splits = (live + chunk - 1) / chunk;
+    per_row[4 * b + 1] = splits < 1 ? 1 : (splits > max_splits ? max_splits : splits);
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -136,11 +151,26 @@ extern "C" size_t rd_attn_bits_words(int batch, int n_q, int kv_len) {
   return (size_t)batch * n_q * ((kv_len + 63) / 64);
 }
 
+namespace {
+int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      n = prop.multiProcessorCount;
+    if (n <= 0) n = 256;
+  }
+  return n;
+}
+}  // namespace
+
 extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64_t mask_stride_q,
-                               int batch, int n_q, int kv_len, int fix_empty_rows, uint64_t* bits,
-                               int32_t* plan, void* stream) {
-  RD_REQUIRE(batch > 0 && n_q > 0 && kv_len > 0, RD_EINVAL,
-             "rd_attn_prepare: bad sizes (batch %d n_q %d kv_len %d)", batch, n_q, kv_len);
+                               int batch, int n_q, int kv_len, int n_heads, int fix_empty_rows,
+                               uint64_t* bits, int32_t* plan, void* stream) {
+  RD_REQUIRE(batch > 0 && n_q > 0 && kv_len > 0 && n_heads > 0, RD_EINVAL,
+             "rd_attn_prepare: bad sizes (batch %d n_q %d kv_len %d n_heads %d)", batch, n_q, kv_len,
+             n_heads);
   RD_REQUIRE(batch <= 65535 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
              "rd_attn_prepare: batch %d too large for kv_len %d", batch, kv_len);
   RD_REQUIRE(mask && bits && plan, RD_EINVAL, "rd_attn_prepare: null pointer");
@@ -154,6 +184,6 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
                      mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first); }
   if (int e = rd::check_launch("rd_attn_prepare(bits)")) return e;
   { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 0, s, row_first, batch, n_q, kv_len,
-                     words, rd::kAttnChunk, max_splits, plan); }
+                     words, rd::kAttnChunk, max_splits, n_heads, compute_units(), plan); }
   return rd::check_launch("rd_attn_prepare(plan)");
 }

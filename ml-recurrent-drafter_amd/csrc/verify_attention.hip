@@ -9,8 +9,8 @@
 // Two kernels behind one entry point:
 //   attn_mfma_kernel      bf16, head_dim 128: S^T = K Q^T and O^T = V^T P^T on
 //                         v_mfma_f32_32x32x16_bf16.  512 threads = 8 waves, each wave owns 32 query
-//                         rows; a 64-key K tile and the transposed V tile are staged in LDS and
-//                         shared by the 8 waves; online softmax in fp32.  With the transposed
+//                         rows; a 64-key K tile and the transposed V tile are staged in LDS (double
+//                         buffered) and shared by the 8 waves; online softmax in fp32.  With the transposed
 //                         products a query row lives in one lane pair, so the row maximum and sum
 //                         need a single cross-lane exchange, and P^T is already laid out as the
 //                         B operand of the second product.
@@ -52,25 +52,44 @@ constexpr int kD = 128;
 constexpr int kTile = 64;                  // keys per tile
 constexpr int kWaves = 8;
 constexpr int kMfmaThreads = kWaves * 64;  // 512
-constexpr int kRowsPerWG = kWaves * 32;    // 256 query rows
+constexpr int kRowsPerWG = kWaves * 32;    // 256 query rows: K/V tiles are staged once per key range
+constexpr int kBuffers = 2;                // LDS tile buffers (2: stage tile t+1 while t is consumed)
 constexpr int kKsStride = kD + 8;          // bf16 elements; 272-byte rows spread 16 lanes over all banks
 constexpr int kVtStride = kTile + 4;       // bf16 elements; 136-byte rows
 
+// max over the two lanes (l, l^32) that share a query row
+__device__ inline float pair_max(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // r[0]: low half's value, r[1]: high half's
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ inline float pair_sum(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
 __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) __bf16 s_k[kTile * kKsStride];
-  __shared__ __attribute__((aligned(16))) __bf16 s_vt[kD * kVtStride];
+  __shared__ __attribute__((aligned(16))) __bf16 s_k[kBuffers][kTile * kKsStride];
+  __shared__ __attribute__((aligned(16))) __bf16 s_vt[kBuffers][kD * kVtStride];
 
   const int item = blockIdx.y;
   if (item >= a.plan[0]) return;
   const int32_t* it = a.plan + RD_PLAN_HDR + 4 * a.B + 4 * item;
   const int b = it[0], lo = it[1], hi = it[2], split = it[3];
   const int n_splits = a.plan[RD_PLAN_HDR + 4 * b + 1];
-  const int h = blockIdx.x;
+  // query tiles of one (row, head, key range) are neighbours in dispatch order, so they run
+  // together and the second read of the K/V tiles is served by the L2
+  const int q_tiles = gridDim.x / a.H;
+  const int h = blockIdx.x / q_tiles, q_tile = blockIdx.x - h * q_tiles;
   const int hk = h / (a.H / a.Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 5, r = lane & 31;
-  const int q_row = blockIdx.z * kRowsPerWG + wave * 32 + r;
-  const bool wave_active = blockIdx.z * kRowsPerWG + wave * 32 < a.n_q;
+  const int q_row = q_tile * kRowsPerWG + wave * 32 + r;
+  const bool wave_active = q_tile * kRowsPerWG + wave * 32 < a.n_q;
   const bool row_valid = q_row < a.n_q;
 
   const __bf16* kbase = reinterpret_cast<const __bf16*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh;
@@ -94,114 +113,147 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   for (int db = 0; db < 4; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
-  float m = -INFINITY, l = 0.f;
+  float m = -INFINITY, l = 0.f;  // m in log2 units (already scaled)
   const float scale_log2 = a.scale * 1.4426950408889634f;
 
-  // Loader roles: threads [0,256) stage K rows, threads [256,512) stage V transposed.
+  // Loader roles: threads [0,256) stage K rows (keys lrow+16*i), threads [256,512) stage V
+  // transposed (keys 4*lrow+i); four 16-byte chunks each per tile.
   const bool k_loader = tid < 256;
   const int lt = tid & 255;
   const int chunk = lt & 15;  // 16-byte column chunk of a 256-byte row
-  const int lrow = lt >> 4;   // K: keys lrow+16*i ; V: keys 4*lrow+i
+  const int lrow = lt >> 4;
   bf16x8 pre[4];
   auto prefetch = [&](int key0) {
+    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = key0 + (k_loader ? lrow + 16 * i : 4 * lrow + i);
-      bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
       const __bf16* p = (k_loader ? kbase + (int64_t)key * a.k_ss : vbase + (int64_t)key * a.v_ss) + 8 * chunk;
       pre[i] = key < a.kv_len ? *reinterpret_cast<const bf16x8*>(p) : z;
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](int buf) {
     if (k_loader) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        *reinterpret_cast<bf16x8*>(&s_k[(lrow + 16 * i) * kKsStride + 8 * chunk]) = pre[i];
+        *reinterpret_cast<bf16x8*>(&s_k[buf][(lrow + 16 * i) * kKsStride + 8 * chunk]) = pre[i];
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         bf16x4 t = {pre[0][e], pre[1][e], pre[2][e], pre[3][e]};
-        *reinterpret_cast<bf16x4*>(&s_vt[(8 * chunk + e) * kVtStride + 4 * lrow]) = t;
+        *reinterpret_cast<bf16x4*>(&s_vt[buf][(8 * chunk + e) * kVtStride + 4 * lrow]) = t;
       }
     }
   };
 
   const int n_tiles = (hi - lo + kTile - 1) / kTile;
-  if (n_tiles > 0) prefetch(lo);
+  // Vector-memory loads complete in issue order, so a load that is needed soon must be issued
+  // BEFORE the long-latency tile prefetch: the mask word of tile t+1 is fetched one iteration
+  // ahead, in front of the K/V loads of tile t+2.
+  uint64_t word_next = 0ull;
+  if (n_tiles > 0) {
+    word_next = row_valid ? brow[lo >> 6] : 0ull;
+    prefetch(lo);
+    stage(0);
+    if (kBuffers == 2 && n_tiles > 1) prefetch(lo + kTile);
+  }
+  __syncthreads();
   for (int t = 0; t < n_tiles; ++t) {
     const int key0 = lo + t * kTile;
-    __syncthreads();  // every wave is done with the previous tile
-    stage();
-    __syncthreads();
-    if (t + 1 < n_tiles) prefetch(key0 + kTile);
-    if (!wave_active) continue;
-
-    // S^T tile: 64 keys x 32 queries, two 32x32 blocks
-    f32x16 s[2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&s_k[(32 * kb + r) * kKsStride + 16 * ks + 8 * g]);
-        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[ks], s[kb], 0, 0, 0);
-      }
+    const int buf = kBuffers == 2 ? (t & 1) : 0;
+    if (kBuffers == 2) {
+      // the other buffer was last read in iteration t-1, which every wave has left
+      if (t + 1 < n_tiles) stage(buf ^ 1);
     }
-    // accumulator i of block kb is key 32*kb + 8*(i/4) + 4*g + i%4 of the tile
-    const uint64_t word = row_valid ? brow[key0 >> 6] : 0ull;
-    const bool all_on = __all(word == ~0ull);
-    float tmax = -INFINITY;
+    const uint64_t word = word_next;
+    if (t + 1 < n_tiles) word_next = row_valid ? brow[(key0 + kTile) >> 6] : 0ull;
+    if (t + kBuffers < n_tiles) prefetch(key0 + kBuffers * kTile);
+    if (wave_active) {
+      const __bf16* sk = s_k[buf];
+      const __bf16* sv = s_vt[buf];
+      // S^T tile: 64 keys x 32 queries, two 32x32 blocks
+      f32x16 s[2];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float x = s[kb][i] * scale_log2;
-        if (!all_on) {
-          const int bit = 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
-          x = ((word >> bit) & 1ull) ? x : -INFINITY;
+        for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+          const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&sk[(32 * kb + r) * kKsStride + 16 * ks + 8 * g]);
+          s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[ks], s[kb], 0, 0, 0);
         }
-        s[kb][i] = x;
-        tmax = fmaxf(tmax, x);
       }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-    const float m_new = fmaxf(m, tmax);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = fast_exp2(m - m_use);
-    float psum = 0.f;
-    bf16x8 pf[4];
+      // accumulator i of block kb is key 32*kb + 8*(i/4) + 4*g + i%4 of the tile
+      if (!__all(word == ~0ull)) {
+        const uint32_t w[2] = {(uint32_t)(word >> (4 * g)), (uint32_t)(word >> (32 + 4 * g))};
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float p = fast_exp2(s[kb][i] - m_use);
-        psum += p;
-        pf[2 * kb + (i >> 3)][i & 7] = static_cast<__bf16>(p);
+          for (int i = 0; i < 16; ++i) {
+            const bool on = (w[kb] >> (8 * (i >> 2) + (i & 3))) & 1u;
+            s[kb][i] = on ? s[kb][i] : -INFINITY;
+          }
       }
-    l = l * alpha + psum;
-    if (!__all(alpha == 1.f)) {
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[kb][i]);
+      tmax = pair_max(tmax) * scale_log2;
+      // The running maximum only has to bound the exponents, not equal the true maximum: it is
+      // raised (and O, l rescaled) only when the tile exceeds it by more than kSlack, so most
+      // tiles skip the 64-register rescale.  p <= 2^kSlack stays far inside bf16/fp32 range.
+      constexpr float kSlack = 8.f;
+      const bool raise = tmax > m + kSlack || m == -INFINITY;
+      if (__any(raise)) {
+        const float m_new = raise ? tmax : m;
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = fast_exp2(m - m_safe);  // m == -inf -> 0 (o and l are 0 then)
+        l *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        m = m_new;
+      }
+      const float m_use = m == -INFINITY ? 0.f : m;
+      float psum = 0.f;
+      bf16x8 pf[4];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const float p0 = fast_exp2(fmaf(s[kb][i], scale_log2, -m_use));
+          const float p1 = fast_exp2(fmaf(s[kb][i + 1], scale_log2, -m_use));
+          psum += p0 + p1;
+          const f32x2 pp = {p0, p1};
+          const bf16x2 pb = __builtin_convertvector(pp, bf16x2);
+          pf[2 * kb + (i >> 3)][i & 7] = pb[0];
+          pf[2 * kb + (i >> 3)][(i & 7) + 1] = pb[1];
+        }
+      l += psum;
+      // O^T += V^T P^T ; k-slot j of lane group g is key 16*t + 4*g + (j%4) + 8*(j/4)
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+          const __bf16* vp = &sv[(32 * db + r) * kVtStride + 16 * tt + 4 * g];
+          const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vp);
+          const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vp + 8);
+          const bf16x8 va = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pf[tt], o[db], 0, 0, 0);
+        }
+      }
     }
-    m = m_new;
-    // O^T += V^T P^T ; k-slot j of lane group g is key 16*t + 4*g + (j%4) + 8*(j/4)
-#pragma unroll
-    for (int db = 0; db < 4; ++db) {
-#pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        const __bf16* vp = &s_vt[(32 * db + r) * kVtStride + 16 * tt + 4 * g];
-        const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vp);
-        const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vp + 8);
-        const bf16x8 va = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pf[tt], o[db], 0, 0, 0);
-      }
+    __syncthreads();
+    if (kBuffers == 1 && t + 1 < n_tiles) {
+      stage(0);  // every wave has left tile t
+      __syncthreads();
     }
   }
 
   if (!wave_active) return;
-  l += __shfl_xor(l, 32);
+  l = pair_sum(l);
   if (!row_valid) return;
   // accumulator i of block db is d = 32*db + 8*(i/4) + 4*g + i%4
   if (n_splits == 1) {
@@ -234,26 +286,30 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   }
 }
 
-// Merges the partials of rows whose keys were split (m in log2 units).
+// Merges the partials of rows whose keys were split (m in log2 units).  One workgroup per
+// (head, batch row, query slice); rows that were not split cost one early exit per workgroup.
+constexpr int kCombineSlices = 32;
 __global__ __launch_bounds__(kD) void attn_combine_kernel(AttnArgs a) {
-  const int q = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int h = blockIdx.x, b = blockIdx.y;
   const int n_splits = a.plan[RD_PLAN_HDR + 4 * b + 1];
   if (n_splits <= 1) return;
   const int d = threadIdx.x;
   const int64_t slot0 = ((int64_t)b * a.H + h) * a.max_splits;
-  float mx = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, a.part_ml[((slot0 + s) * a.n_q + q) * 2]);
-  float acc = 0.f, lsum = 0.f;
-  if (mx > -INFINITY) {
-    for (int s = 0; s < n_splits; ++s) {
-      const float* pm = a.part_ml + ((slot0 + s) * a.n_q + q) * 2;
-      const float w = fast_exp2(pm[0] - mx);
-      lsum += w * pm[1];
-      acc += w * a.part_o[((slot0 + s) * a.n_q + q) * kD + d];
+  for (int q = blockIdx.z; q < a.n_q; q += kCombineSlices) {
+    float mx = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, a.part_ml[((slot0 + s) * a.n_q + q) * 2]);
+    float acc = 0.f, lsum = 0.f;
+    if (mx > -INFINITY) {
+      for (int s = 0; s < n_splits; ++s) {
+        const float* pm = a.part_ml + ((slot0 + s) * a.n_q + q) * 2;
+        const float w = fast_exp2(pm[0] - mx);
+        lsum += w * pm[1];
+        acc += w * a.part_o[((slot0 + s) * a.n_q + q) * kD + d];
+      }
     }
+    __bf16* op = reinterpret_cast<__bf16*>(a.out) + (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss;
+    op[d] = static_cast<__bf16>(lsum > 0.f ? acc / lsum : 0.f);
   }
-  __bf16* op = reinterpret_cast<__bf16*>(a.out) + (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss;
-  op[d] = static_cast<__bf16>(lsum > 0.f ? acc / lsum : 0.f);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -395,11 +451,12 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
                                          rd::align_up(slots * n_q * head_dim * sizeof(float), 256));
     const int max_items = batch * a.max_splits;
     const int q_tiles = (n_q + kRowsPerWG - 1) / kRowsPerWG;
-    RD_REQUIRE(max_items <= 65535 && q_tiles <= 65535, RD_ELIMIT, "rd_verify_attention: grid too large");
-    { rd::ScopedTiming rd_t("attn_mfma_kernel", s); hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_heads, max_items, q_tiles), dim3(kMfmaThreads), 0, s, a); }
+    RD_REQUIRE(max_items <= 65535 && (int64_t)q_tiles * n_heads <= 2147483647LL, RD_ELIMIT,
+               "rd_verify_attention: grid too large");
+    { rd::ScopedTiming rd_t("attn_mfma_kernel", s); hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, a); }
     if (int e = rd::check_launch("rd_verify_attention(mfma)")) return e;
     if (a.max_splits > 1) {
-      { rd::ScopedTiming rd_t("attn_combine_kernel", s); hipLaunchKernelGGL(attn_combine_kernel, dim3(n_q, n_heads, batch), dim3(kD), 0, s, a); }
+      { rd::ScopedTiming rd_t("attn_combine_kernel", s); hipLaunchKernelGGL(attn_combine_kernel, dim3(n_heads, batch, kCombineSlices), dim3(kD), 0, s, a); }
       return rd::check_launch("rd_verify_attention(combine)");
     }
     return RD_OK;

@@ -38,7 +38,7 @@ _PROTOTYPES = {
     "rd_kv_compact": (_I, [_P, _I, _I, _I, _L, _L, _L, _I, _P, _P]),
     "rd_attn_plan_ints": (_Z, [_I, _I, _I]),
     "rd_attn_bits_words": (_Z, [_I, _I, _I]),
-    "rd_attn_prepare": (_I, [_P, _L, _L, _I, _I, _I, _I, _P, _P, _P]),
+    "rd_attn_prepare": (_I, [_P, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P]),
     "rd_attention_workspace_bytes": (_Z, [_I, _I, _I, _I, _I]),
     "rd_verify_attention": (
         _I,

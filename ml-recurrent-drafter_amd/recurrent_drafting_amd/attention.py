@@ -61,8 +61,9 @@ class PreparedMask:
     workspace: Optional[torch.Tensor] = None
 
 
-def prepare(mask: torch.Tensor, fix_empty_rows: bool = True) -> PreparedMask:
-    """mask: (B, n_q, kv_len) bool/uint8, keys contiguous."""
+def prepare(mask: torch.Tensor, fix_empty_rows: bool = True, n_heads: int = 32) -> PreparedMask:
+    """mask: (B, n_q, kv_len) bool/uint8, keys contiguous.  n_heads: query heads of the attention
+    calls that will use the result (only sizes the work items)."""
     assert mask.dim() == 3 and mask.dtype in (torch.bool, torch.uint8)
     if mask.stride(2) != 1:
         mask = mask.contiguous()
@@ -73,7 +74,8 @@ def prepare(mask: torch.Tensor, fix_empty_rows: bool = True) -> PreparedMask:
     plan = torch.empty(lib.rd_attn_plan_ints(B, n_q, kv_len), dtype=torch.int32, device=dev)
     _hip.check(
         lib.rd_attn_prepare(
-            _hip.ptr(mask), mask.stride(0), mask.stride(1), B, n_q, kv_len, int(fix_empty_rows),
+            _hip.ptr(mask), mask.stride(0), mask.stride(1), B, n_q, kv_len, int(n_heads),
+            int(fix_empty_rows),
             _hip.ptr(bits), _hip.ptr(plan), _hip.stream(),
         )
     )

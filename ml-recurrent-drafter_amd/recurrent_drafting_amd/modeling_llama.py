@@ -165,7 +165,8 @@ class LlamaModel(LlamaPreTrainedModel):
     def forward(self, input_ids, attention_mask, position_ids, past_key_values) -> torch.Tensor:
         """attention_mask: (B, q, kv) bool, or an attention.PreparedMask built from one."""
         if not isinstance(attention_mask, attention.PreparedMask):
-            attention_mask = attention.prepare(attention_mask, fix_empty_rows=False)
+            attention_mask = attention.prepare(
+                attention_mask, fix_empty_rows=False, n_heads=self.config.num_attention_heads)
         hidden_states = self.embed_tokens(input_ids)
         for layer, key_value in zip(self.layers, past_key_values):
             hidden_states = layer(hidden_states, position_ids, key_value, attention_mask)
@@ -190,7 +191,8 @@ class LlamaForCausalLM(LlamaPreTrainedModel):
     def hidden_states(self, input_ids, attention_mask, position_ids, past_key_values) -> torch.Tensor:
         """Final-norm hidden states (B, q, hidden); rows that attend to nothing attend to
         everything, as the reference arranges on a GPU (modeling_llama.py:264-265)."""
-        prepared = attention.prepare(attention_mask, fix_empty_rows=True)
+        prepared = attention.prepare(
+            attention_mask, fix_empty_rows=True, n_heads=self.config.num_attention_heads)
         return self.model(input_ids=input_ids, attention_mask=prepared, position_ids=position_ids,
                           past_key_values=past_key_values)
 

@@ -51,7 +51,7 @@ def test_mask_bits_and_plan():
     mask[1, 3, :] = False  # an empty row gets all keys
     mask[2, :, :64] = False
     mask[2, 5, 70] = True
-    prep = attention.prepare(_dev(mask, torch.bool))
+    prep = attention.prepare(_dev(mask, torch.bool), n_heads=4096)  # many heads: minimum-size items
     words = prep.bits.cpu().numpy().view(np.uint64)
     fixed = T.fully_masked_rows_to_true(mask)
     for b in range(B):
@@ -76,7 +76,7 @@ def test_mask_bits_and_plan():
         assert all(lo % 64 == 0 for lo, _ in mine)
 
 
-def _run(q, k, v, mask, dtype, force_generic, cache_like=False):
+def _run(q, k, v, mask, dtype, force_generic, cache_like=False, n_heads_for_plan=None):
     from recurrent_drafting_amd import attention
 
     tq, tk, tv = (_dev(x, torch.float32).to(dtype) for x in (q, k, v))
@@ -89,7 +89,7 @@ def _run(q, k, v, mask, dtype, force_generic, cache_like=False):
         big_v = torch.full_like(big_k, 3.0)
         big_k[:, :, :kv] = tk; big_v[:, :, :kv] = tv
         tk, tv = big_k[:, :, :kv], big_v[:, :, :kv]
-    prep = attention.prepare(_dev(mask, torch.bool))
+    prep = attention.prepare(_dev(mask, torch.bool), n_heads=n_heads_for_plan or H)
     out = attention.masked_attention(tq, tk, tv, prep, force_generic=force_generic)
     torch.cuda.synchronize()
     ref_in = [x.float().cpu().numpy() for x in (tq, tk, tv)]  # the oracle sees the rounded inputs
@@ -153,6 +153,9 @@ def test_mfma_kernel(B, H, Hkv, W, L, prev_lens):
     q = rng.standard_normal((B, H, nq, D)); k = rng.standard_normal((B, Hkv, kv, D)); v = rng.standard_normal((B, Hkv, kv, D))
     got, ref = _run(q, k, v, mask, torch.bfloat16, force_generic=False, cache_like=True)
     _assert_close(got, ref, torch.bfloat16)
+    # a plan made for many heads cuts every row into minimum-size items: exercises the partials
+    got3, _ = _run(q, k, v, mask, torch.bfloat16, force_generic=False, cache_like=True, n_heads_for_plan=4096)
+    _assert_close(got3, ref, torch.bfloat16)
     got2, _ = _run(q, k, v, mask, torch.bfloat16, force_generic=True, cache_like=True)
     _assert_close(got2, ref, torch.bfloat16)
 
@@ -189,7 +192,7 @@ def test_verify_attention_benchmark_shape():
     k, v = cache[0, :, :, :kv], cache[1, :, :, :kv]
     q = torch.randn(B, nq, H, D, device="cuda", dtype=torch.bfloat16).permute(0, 2, 1, 3)
     tmask = _dev(mask, torch.bool)
-    prep = attention.prepare(tmask)
+    prep = attention.prepare(tmask, n_heads=H)
     out = attention.masked_attention(q, k, v, prep).view(B, nq, H, D).permute(0, 2, 1, 3).float()
     s = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float()) / D ** 0.5
     s = s.masked_fill(~tmask[:, None], float("-inf"))
