@@ -5,17 +5,19 @@
 //   per batch row: top-W of the W*V scores, sorted descending; token = idx % V, parent = idx / V;
 //                  beams gathered by parent and extended by the token
 //
-// beam_row_kernel (one 1024-thread workgroup per beam row, the whole row in registers):
+// beam_row_kernel (one workgroup per beam row, the whole row in registers: 256 threads x 128 values
+// up to a vocabulary of 32768, so that several rows share a compute unit; 1024 x 64 above):
 //   After the filter only ~50 entries of a row differ from one constant, so the row's contribution
 //   to the batch row's top-W is: its W best survivors, then (if W exceeds them) filtered tokens in
 //   increasing id order, all with the same score.  Survivors are found without sorting the row:
 //   a pivot p -- the minimum over waves of each wave's r-th largest per-thread maximum,
-//   r = ceil(50/16) -- has at least 50 entries above it and, on ordinary data, not many more;
-//   entries >= p are appended to an LDS list, which is ranked by counting.  If the list overflows
-//   (heavy ties, adversarial layouts) the row falls back to a bisection on the value bits plus W
-//   rounds of block-wide argmax: slow, exact for any input.
-// beam_merge_kernel (one workgroup per batch row): the W sorted lists are cut at
-//   max(min head, max tail), the few entries above the cut are ranked by counting.
+//   r = ceil(50/waves) -- has at least 50 entries above it and, on ordinary data, not many more;
+//   entries >= p go to an LDS list, which is sorted by counting.  The max subtraction and the
+//   rounding are applied to the listed entries only.  If the list overflows or cannot decide a tie
+//   at the 50th value (heavy ties, adversarial layouts) the row falls back to a bisection on the
+//   value bits plus W rounds of block-wide argmax: slow, exact for any input.
+// beam_merge_kernel (one workgroup per batch row): the W sorted lists are cut at the W-th largest
+//   of their leading entries, the few entries above the cut are ranked by counting.
 //
 // Rounding follows the drafter's dtype T at the points where a tensor in that dtype is
 // materialised upstream (after the max subtraction, the filter value, the log-softmax output); the
@@ -30,126 +32,89 @@ namespace {
 constexpr int kMaxWidth = 64;    // beam width limit of the merge kernel (W*W <= 4096 LDS keys)
 constexpr int kMergeThreads = 256;
 
+// The exact path for rows whose candidate list overflows: k-th largest value by bisection, then W
+// rounds of block-wide argmax over (score, index).  Works from memory (the row is in L2), not from
+// the caller's register copy, so that it costs the common path no registers.
+template <typename T, int THREADS>
+__device__ void beam_row_fallback(const T* __restrict__ x_row, int V, float row_max, int k_eff,
+                                  float mask_t, float lpb, int W, float* __restrict__ c_score,
+                                  int32_t* __restrict__ c_tok, float* __restrict__ lo_row,
+                                  RowShared& sh) {
+  const int tid = threadIdx.x;
+  auto value = [&](int i) { return Num<T>::round(Num<T>::load(x_row + i) - row_max); };
+  const float thr = row_kth_bisect<T, THREADS>(x_row, V, row_max, k_eff, sh);
+  float part = 0.f;
+  for (int i = tid; i < V; i += THREADS) {
+    const float v = value(i);
+    part += v >= thr ? expf(v) : 0.f;
+  }
+  const float logsum = logf(block_sum<THREADS>(part, sh));
+  const float masked_lp = Num<T>::round(mask_t - logsum);
+  auto log_prob = [&](float v) { return v >= thr ? Num<T>::round(v - logsum) : masked_lp; };
+  uint64_t last = ~0ull;
+  for (int w = 0; w < W; ++w) {
+    uint64_t best = 0ull;
+    for (int i = tid; i < V; i += THREADS) {
+      const uint64_t k = key64(log_prob(value(i)) + lpb, (uint32_t)i);
+      if (k < last && k > best) best = k;
+    }
+    best = block_max64<THREADS>(best, sh);
+    if (tid == 0) {
+      if (best == 0ull) { c_score[w] = -INFINITY; c_tok[w] = -1; }
+      else { c_score[w] = unord((uint32_t)(best >> 32)); c_tok[w] = (int32_t)(0xffffffffu - (uint32_t)best); }
+    }
+    last = best;
+  }
+  if (lo_row)
+    for (int i = tid; i < V; i += THREADS) lo_row[i] = log_prob(value(i));
+}
+
 // ITEMS elements per thread, held as ITEMS/VEC vectors of VEC = 16 bytes / sizeof(T).
-template <typename T, int ITEMS>
-__global__ __launch_bounds__(kRowThreads) void beam_row_kernel(
+template <typename T, int ITEMS, int THREADS>
+__global__ __launch_bounds__(THREADS) void beam_row_kernel(
     const T* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ log_p_beam,
     int W, int top_k, float mask_value, float* __restrict__ cand_score,
     int32_t* __restrict__ cand_tok, float* __restrict__ logp_out, int64_t logp_row_stride,
     int force_fallback) {
   constexpr int VEC = 16 / sizeof(T);
-  constexpr int NV = ITEMS / VEC;
   __shared__ RowShared sh;
   const int row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const T* x_row = logits + (int64_t)row * row_stride;
-  auto index_of = [&](int j) { return ((j / VEC) * kRowThreads + tid) * VEC + (j % VEC); };
 
-  // ---- load the row, row maximum ------------------------------------------------------------
+  // ---- load the row; maximum; pivot on the raw values -------------------------------------------
   float x[ITEMS];
+  load_row<T, ITEMS, THREADS>(x_row, V, x);
   float tmax = -INFINITY;
 #pragma unroll
-  for (int c = 0; c < NV; ++c) {
-    const int i0 = (c * kRowThreads + tid) * VEC;
-    if (i0 + VEC <= V) {
-      struct alignas(16) Pack { T v[VEC]; };
-      const Pack p = *reinterpret_cast<const Pack*>(x_row + i0);
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) x[c * VEC + e] = Num<T>::load(&p.v[e]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) x[c * VEC + e] = (i0 + e < V) ? Num<T>::load(x_row + i0 + e) : -INFINITY;
-    }
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) tmax = fmaxf(tmax, x[c * VEC + e]);
-  }
-  const float row_max = block_max(tmax, sh);
-  tmax = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    x[j] = index_of(j) < V ? Num<T>::round(x[j] - row_max) : -INFINITY;
-    tmax = fmaxf(tmax, x[j]);
-  }
+  for (int j = 0; j < ITEMS; ++j) tmax = fmaxf(tmax, x[j]);
+  const float row_max = block_max<THREADS>(tmax, sh);
   const int k_eff = top_k < V ? top_k : V;
   const float mask_t = Num<T>::round(mask_value);
   const float lpb = log_p_beam[row];
   float* c_score = cand_score + (int64_t)row * W;
   int32_t* c_tok = cand_tok + (int64_t)row * W;
+  const float pivot = row_pivot<THREADS>(tmax, k_eff, sh);
 
-  // ---- pivot: at least k_eff entries are >= pivot ----------------------------------------------
-  const int rounds = (k_eff + kRowWaves - 1) / kRowWaves;
-  float cur = tmax, wave_pivot = -INFINITY;
-  for (int it = 0; it < rounds; ++it) {
-    const float wm = wave_max(cur);
-    wave_pivot = wm;
-    const uint64_t holders = __ballot(cur == wm);
-    if (holders != 0 && lane == __builtin_ctzll(holders)) cur = -INFINITY;
-  }
-  const float pivot = block_min(wave_pivot, sh);
+  // ---- candidates: entries >= pivot, keyed by their value after the max subtraction ------------
+  // t(x) = round_T(x - max) is monotone, so the k-th largest t comes from the list; an entry
+  // below the pivot could only tie with it when that k-th value equals t(pivot).
+  int n_c = -1;
+  if (!force_fallback)
+    n_c = row_sorted_candidates<ITEMS, VEC, THREADS>(
+        x, pivot, sh, [&](float v, int i) { return key64(Num<T>::round(v - row_max), (uint32_t)i); });
+  bool fast = n_c >= k_eff;
+  if (fast && n_c < V) fast = key_value(sh.skey[k_eff - 1]) > Num<T>::round(pivot - row_max);
 
-  if (tid == 0) sh.count = 0;
-  __syncthreads();
-  if (!force_fallback) {
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      if (x[j] >= pivot && index_of(j) < V) {
-        const int pos = atomicAdd(&sh.count, 1);
-        if (pos < kCap) { sh.cval[pos] = x[j]; sh.cidx[pos] = index_of(j); }
-      }
-    }
-  }
-  __syncthreads();
-  const int n_c = force_fallback ? kCap + 1 : sh.count;
-
-  if (n_c <= kCap) {
-    // ---- ranked candidate list -------------------------------------------------------------
-    // order: value descending, index ascending.  rank = number of candidates strictly before.
-    int my_rank = -1;
-    float my_v = 0.f;
-    int my_i = 0;
-    if (tid < n_c) {
-      my_v = sh.cval[tid];
-      my_i = sh.cidx[tid];
-      int gt = 0, ge = 0, before = 0;
-      for (int o = 0; o < n_c; ++o) {
-        const float ov = sh.cval[o];
-        const int oi = sh.cidx[o];
-        gt += ov > my_v;
-        ge += ov >= my_v;
-        before += (ov > my_v) || (ov == my_v && oi < my_i);
-      }
-      my_rank = before;
-      if (gt < k_eff && k_eff <= ge) { sh.thr = my_v; sh.n_surv = ge; }
-    }
-    // entries beyond the first 1024 candidates (tid covers only kRowThreads of up to kCap)
-    int my_rank2 = -1;
-    float my_v2 = 0.f;
-    int my_i2 = 0;
-    if (tid + kRowThreads < n_c) {
-      my_v2 = sh.cval[tid + kRowThreads];
-      my_i2 = sh.cidx[tid + kRowThreads];
-      int gt = 0, ge = 0, before = 0;
-      for (int o = 0; o < n_c; ++o) {
-        const float ov = sh.cval[o];
-        const int oi = sh.cidx[o];
-        gt += ov > my_v2;
-        ge += ov >= my_v2;
-        before += (ov > my_v2) || (ov == my_v2 && oi < my_i2);
-      }
-      my_rank2 = before;
-      if (gt < k_eff && k_eff <= ge) { sh.thr = my_v2; sh.n_surv = ge; }
-    }
-    __syncthreads();
-    const float thr = sh.thr;
-    const int n_s = sh.n_surv;
-    // survivors, sorted, back into the list (all reads of the unsorted list are done)
-    if (my_rank >= 0 && my_v >= thr) { sh.cval[my_rank] = my_v; sh.cidx[my_rank] = my_i; }
-    if (my_rank2 >= 0 && my_v2 >= thr) { sh.cval[my_rank2] = my_v2; sh.cidx[my_rank2] = my_i2; }
-    __syncthreads();
+  if (fast) {
+    const int n_s = row_survivors<THREADS>(n_c, k_eff, sh);  // skey[0 .. n_s) survive the filter
+    const float thr = key_value(sh.skey[k_eff - 1]);
+    auto s_val = [&](int o) { return key_value(sh.skey[o]); };
+    auto s_idx = [&](int o) { return key_index(sh.skey[o]); };
     // log-sum-exp over the survivors in sorted order (filtered entries add exp(-5e4) == 0)
     if (wave == 0) {
       float part = 0.f;
-      for (int o = lane; o < n_s; o += 64) part += expf(sh.cval[o]);
+      for (int o = lane; o < n_s; o += 64) part += expf(s_val(o));
       part = wave_sum(part);
       if (lane == 0) sh.logsum = logf(part);
     }
@@ -157,136 +122,120 @@ __global__ __launch_bounds__(kRowThreads) void beam_row_kernel(
     const float logsum = sh.logsum;
     const float masked_score = Num<T>::round(mask_t - logsum) + lpb;
     // survivors -> scores; equal scores are re-ordered by index (rounding can merge values)
-    for (int s = tid; s < n_s; s += kRowThreads) {
-      const float sc = Num<T>::round(sh.cval[s] - logsum) + lpb;
-      const int si = sh.cidx[s];
+    for (int s = tid; s < n_s; s += THREADS) {
+      const float sc = Num<T>::round(s_val(s) - logsum) + lpb;
+      const int si = s_idx(s);
       // entries with the same rounded score are contiguous in the sorted list
-      int lo = s, pos = s;
-      while (lo > 0 && Num<T>::round(sh.cval[lo - 1] - logsum) + lpb == sc) --lo;
+      int lo = s;
+      while (lo > 0 && Num<T>::round(s_val(lo - 1) - logsum) + lpb == sc) --lo;
       int hi = s;
-      while (hi + 1 < n_s && Num<T>::round(sh.cval[hi + 1] - logsum) + lpb == sc) ++hi;
-      pos = lo;
-      for (int o = lo; o <= hi; ++o) pos += sh.cidx[o] < si;
+      while (hi + 1 < n_s && Num<T>::round(s_val(hi + 1) - logsum) + lpb == sc) ++hi;
+      int pos = lo;
+      for (int o = lo; o <= hi; ++o) pos += s_idx(o) < si;
       if (pos < W) { c_score[pos] = sc; c_tok[pos] = si; }
     }
     // W beyond the survivors: filtered tokens in increasing id, all with masked_score
     if (n_s < W) {
       const int need = W - n_s;
-      for (int u = tid; u < need + n_s && u < V; u += kRowThreads) {
+      for (int u = tid; u < need + n_s && u < V; u += THREADS) {
         bool surv = false;
         int before = 0;
-        for (int o = 0; o < n_s; ++o) { surv |= sh.cidx[o] == u; before += sh.cidx[o] < u; }
+        for (int o = 0; o < n_s; ++o) { surv |= s_idx(o) == u; before += s_idx(o) < u; }
         const int pos = u - before;
         if (!surv && pos < need) { c_score[n_s + pos] = masked_score; c_tok[n_s + pos] = u; }
       }
       const int avail = V - n_s;  // fewer tokens than W in a tiny vocabulary
-      for (int u = tid; u < need; u += kRowThreads)
+      for (int u = tid; u < need; u += THREADS)
         if (u >= avail) { c_score[n_s + u] = -INFINITY; c_tok[n_s + u] = -1; }
     }
     if (logp_out) {
       float* lo_row = logp_out + (int64_t)row * logp_row_stride;
       const float masked_lp = Num<T>::round(mask_t - logsum);
+      const int base = row_base<VEC>();
 #pragma unroll
-      for (int j = 0; j < ITEMS; ++j) {
-        const int i = index_of(j);
-        if (i < V) lo_row[i] = x[j] >= thr ? Num<T>::round(x[j] - logsum) : masked_lp;
+      for (int c = 0; c < ITEMS / 4; ++c) {
+        // float4 stores where the four values are contiguous in the row (VEC is 4 or 8)
+        const int i = row_index_at<VEC, THREADS>(base, c * 4);
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float t = Num<T>::round(x[c * 4 + e] - row_max);
+          o[e] = t >= thr ? Num<T>::round(t - logsum) : masked_lp;
+        }
+        if (i + 4 <= V && ((reinterpret_cast<uintptr_t>(lo_row + i) & 15) == 0)) {
+          *reinterpret_cast<float4*>(lo_row + i) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) if (i + e < V) lo_row[i + e] = o[e];
+        }
       }
     }
     return;
   }
 
-  // ---- fallback: exact for any input -----------------------------------------------------------
-  // k-th largest value by bisection on the ordered bit pattern
-  uint32_t lo_k = 0u, hi_k = 0xffffffffu;  // invariant: count(>= lo_k) >= k_eff
-  while (lo_k < hi_k) {
-    const uint32_t mid = lo_k + (uint32_t)(((uint64_t)hi_k - lo_k + 1) >> 1);
-    int cnt = 0;
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) cnt += (index_of(j) < V) && ord(x[j]) >= mid;
-    cnt = block_isum(cnt, sh);
-    if (cnt >= k_eff) lo_k = mid; else hi_k = mid - 1;
-  }
-  const float thr = unord(lo_k);
-  float part = 0.f;
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) part += (index_of(j) < V && x[j] >= thr) ? expf(x[j]) : 0.f;
-  const float logsum = logf(block_sum(part, sh));
-  const float masked_lp = Num<T>::round(mask_t - logsum);
-  auto score_of = [&](int j) { return (x[j] >= thr ? Num<T>::round(x[j] - logsum) : masked_lp) + lpb; };
-  uint64_t last = ~0ull;
-  for (int w = 0; w < W; ++w) {
-    uint64_t best = 0ull;
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      const int i = index_of(j);
-      if (i < V) {
-        const uint64_t k = key64(score_of(j), (uint32_t)i);
-        if (k < last && k > best) best = k;
-      }
-    }
-    best = block_max64(best, sh);
-    if (tid == 0) {
-      if (best == 0ull) { c_score[w] = -INFINITY; c_tok[w] = -1; }
-      else { c_score[w] = unord((uint32_t)(best >> 32)); c_tok[w] = (int32_t)(0xffffffffu - (uint32_t)best); }
-    }
-    last = best == 0ull ? 0ull : best;
-  }
-  if (logp_out) {
-    float* lo_row = logp_out + (int64_t)row * logp_row_stride;
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      const int i = index_of(j);
-      if (i < V) lo_row[i] = x[j] >= thr ? Num<T>::round(x[j] - logsum) : masked_lp;
-    }
-  }
+  beam_row_fallback<T, THREADS>(x_row, V, row_max, k_eff, mask_t, lpb, W, c_score, c_tok,
+                                logp_out ? logp_out + (int64_t)row * logp_row_stride : nullptr, sh);
 }
 
-// One workgroup per batch row.
+// One workgroup per batch row: top-W of W sorted lists of W candidates.
+//   1. the W-th largest key of a subset (the first m entries of every list, m*W <= threads) is a
+//      lower bound of the W-th largest key overall: the cut;
+//   2. the keys >= cut -- usually not many more than W -- are listed and ranked by counting.
 __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(
     const float* __restrict__ cand_score, const int32_t* __restrict__ cand_tok, int W, int V,
     const int64_t* __restrict__ beams_in, int t_len, float* __restrict__ new_log_p_beam,
     int64_t* __restrict__ tokens, int64_t* __restrict__ parents, int64_t* __restrict__ beams_out) {
-  __shared__ unsigned long long s_keys[kMaxWidth * kMaxWidth];
-  __shared__ unsigned long long s_cut[2][kMergeThreads / 64];
+  __shared__ __attribute__((aligned(16))) unsigned long long s_keys[kMaxWidth * kMaxWidth + 2];
+  __shared__ __attribute__((aligned(16))) unsigned long long s_head[kMergeThreads + 2];
+  __shared__ unsigned long long s_cut;
   __shared__ int s_count;
   __shared__ int s_parent[kMaxWidth];
-  const int b = blockIdx.x, tid = threadIdx.x;
+  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
   const float* cs = cand_score + (int64_t)b * W * W;
   const int32_t* ct = cand_tok + (int64_t)b * W * W;
   auto key_at = [&](int w, int j) -> uint64_t {
     const int tok = ct[w * W + j];
     return tok < 0 ? 0ull : key64(cs[w * W + j], (uint32_t)(w * V + tok));
   };
-  // cut = max(min over rows of the head, max over rows of the tail): the W-th best key is >= cut
-  uint64_t min_head = ~0ull, max_tail = 0ull;
-  for (int w = tid; w < W; w += kMergeThreads) {
-    const uint64_t h = key_at(w, 0), t = key_at(w, W - 1);
-    min_head = h < min_head ? h : min_head;
-    max_tail = t > max_tail ? t : max_tail;
-  }
-  for (int off = 32; off > 0; off >>= 1) {
-    const uint64_t a = __shfl_xor(min_head, off), c = __shfl_xor(max_tail, off);
-    min_head = a < min_head ? a : min_head;
-    max_tail = c > max_tail ? c : max_tail;
-  }
-  if ((tid & 63) == 0) { s_cut[0][tid >> 6] = min_head; s_cut[1][tid >> 6] = max_tail; }
-  if (tid == 0) s_count = 0;
+  auto count_above = [&](const unsigned long long* keys, int n, uint64_t mine) {
+    const ulonglong2* k2 = reinterpret_cast<const ulonglong2*>(keys);  // keys[n] is a zero pad
+    int before = 0;
+    for (int o = 0; 2 * o < n; ++o) {
+      const ulonglong2 kk = k2[o];
+      before += (kk.x > mine) + (kk.y > mine);
+    }
+    return before;
+  };
+  const int m = W < kMergeThreads / W ? W : kMergeThreads / W;
+  const int n_sub = W * m;
+  uint64_t mine = 0ull;
+  if (tid < n_sub) mine = key_at(tid / m, tid % m);
+  s_head[tid] = mine;
+  if (tid == 0) { s_head[kMergeThreads] = 0ull; s_count = 0; s_cut = 0ull; }
   __syncthreads();
-  for (int w = 0; w < kMergeThreads / 64; ++w) {
-    min_head = s_cut[0][w] < min_head ? s_cut[0][w] : min_head;
-    max_tail = s_cut[1][w] > max_tail ? s_cut[1][w] : max_tail;
-  }
-  const uint64_t cut = min_head > max_tail ? min_head : max_tail;
-  for (int c = tid; c < W * W; c += kMergeThreads) {
-    const uint64_t k = key_at(c / W, c % W);
-    if (k >= cut && k != 0ull) s_keys[atomicAdd(&s_count, 1)] = k;
+  // distinct nonzero keys: exactly one thread has W - 1 keys above it (none if fewer than W exist)
+  if (mine != 0ull && count_above(s_head, kMergeThreads, mine) == W - 1) s_cut = mine;
+  __syncthreads();
+  const uint64_t cut = s_cut;
+  for (int c0 = 0; c0 < W * W; c0 += kMergeThreads) {
+    const int c = c0 + tid;
+    const uint64_t k = c < W * W ? key_at(c / W, c % W) : 0ull;
+    const bool take = k != 0ull && k >= cut;
+    const uint64_t votes = __ballot(take);
+    if (votes == 0) continue;
+    int first = 0;
+    const int leader = __builtin_ctzll(votes);
+    if (lane == leader) first = atomicAdd(&s_count, __builtin_popcountll(votes));
+    first = __shfl(first, leader);
+    if (take) s_keys[first + __builtin_popcountll(votes & ((1ull << lane) - 1ull))] = k;
   }
   __syncthreads();
   const int n = s_count;
+  if (tid == 0) s_keys[n] = 0ull;
+  __syncthreads();
   for (int c = tid; c < n; c += kMergeThreads) {
     const uint64_t k = s_keys[c];
-    int rank = 0;
-    for (int o = 0; o < n; ++o) rank += s_keys[o] > k;
+    const int rank = count_above(s_keys, n, k);
     if (rank < W) {
       const uint32_t flat = 0xffffffffu - (uint32_t)k;
       const int parent = (int)(flat / (uint32_t)V);
@@ -313,14 +262,16 @@ int launch_rows(const void* logits, int64_t row_stride, int rows, int V, const f
                 int top_k, float mask_value, float* cs, int32_t* ct, float* logp_out,
                 int64_t logp_row_stride, int force_fallback, hipStream_t s) {
   const T* x = reinterpret_cast<const T*>(logits);
-  constexpr int VEC = 16 / sizeof(T);
-  const int per_thread = (V + kRowThreads - 1) / kRowThreads;
-#define RD_ROWS(ITEMS)                                                                              \
-  do { rd::ScopedTiming rd_t("beam_row_kernel", s); hipLaunchKernelGGL((beam_row_kernel<T, ITEMS>), dim3(rows), dim3(kRowThreads), 0, s, x, row_stride, \
-                     V, lpb, W, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback); } while (0)
-  if (per_thread <= 8 && VEC <= 8) RD_ROWS(8);
-  else if (per_thread <= 32) RD_ROWS(32);
-  else RD_ROWS(64);
+#define RD_ROWS(ITEMS, THREADS)                                                                     \
+  do { rd::ScopedTiming rd_t("beam_row_kernel", s);                                                  \
+    hipLaunchKernelGGL((beam_row_kernel<T, ITEMS, THREADS>), dim3(rows), dim3(THREADS), 0, s, x,     \
+                       row_stride, V, lpb, W, top_k, mask_value, cs, ct, logp_out, logp_row_stride,  \
+                       force_fallback); } while (0)
+  switch (row_geometry(V)) {
+    case 0: RD_ROWS(32, 256); break;
+    case 1: RD_ROWS(128, 256); break;
+    default: RD_ROWS(64, 1024); break;
+  }
 #undef RD_ROWS
   return rd::check_launch("rd_beam_topk(rows)");
 }
@@ -342,7 +293,7 @@ extern "C" int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, i
   RD_REQUIRE(batch > 0 && width > 0 && vocab > 0 && top_k > 0, RD_EINVAL,
              "rd_beam_topk: bad sizes (batch %d width %d vocab %d top_k %d)", batch, width, vocab, top_k);
   RD_REQUIRE(width <= kMaxWidth, RD_ELIMIT, "rd_beam_topk: width %d > %d", width, kMaxWidth);
-  RD_REQUIRE(vocab <= 64 * kRowThreads, RD_ELIMIT, "rd_beam_topk: vocab %d > %d", vocab, 64 * kRowThreads);
+  RD_REQUIRE(row_geometry(vocab) >= 0, RD_ELIMIT, "rd_beam_topk: vocab %d > 65536", vocab);
   RD_REQUIRE((int64_t)width * vocab < 4294967295LL, RD_ELIMIT, "rd_beam_topk: width*vocab too large");
   RD_REQUIRE(top_k <= 512, RD_ELIMIT, "rd_beam_topk: top_k %d > 512", top_k);
   RD_REQUIRE(logits && log_p_beam && new_log_p_beam && tokens && parents && workspace, RD_EINVAL,

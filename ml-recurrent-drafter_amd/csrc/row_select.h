@@ -1,7 +1,10 @@
 // Whole-row selection helpers shared by the beam-search and verify-logits kernels: a vocabulary
-// row lives in the registers of one 1024-thread workgroup; reductions go through wave shuffles and
-// a few LDS words; the k-th largest value is found from a pivoted candidate list or, when that
-// overflows, by bisection on the value bits.
+// row lives in the registers of one workgroup (THREADS threads, ITEMS values each).  The largest
+// entries are found without sorting the row: a pivot with at least k entries above it comes from
+// the per-thread maxima, entries >= pivot go to an LDS list (a private segment per wave: no
+// atomics, a deterministic order), and the list is sorted by counting.  The per-element work is a
+// load, a max and a compare; everything else touches only the ~2k listed entries.  Rows whose list
+// overflows take a bisection on the value bits over the row in memory: slow, exact for any input.
 #pragma once
 
 #include <hip/hip_bf16.h>
@@ -11,9 +14,8 @@
 
 namespace {
 
-constexpr int kRowThreads = 1024;
-constexpr int kRowWaves = kRowThreads / 64;
-constexpr int kCap = 2048;       // LDS candidate list
+constexpr int kMaxRowWaves = 16;
+constexpr int kCap = 2048;  // LDS candidate list
 
 template <typename T> struct Num;
 template <> struct Num<float> {
@@ -42,55 +44,82 @@ __device__ inline uint64_t key64(float score, uint32_t idx) {
   return ((uint64_t)ord(score) << 32) | (uint64_t)(0xffffffffu - idx);
 }
 
+// Wave-wide reductions on the cross-lane data path of the vector ALU (no LDS round trips): two
+// quad permutes and two mirrors reduce each row of 16 lanes, row_bcast:15 / row_bcast:31 carry the
+// row results up to lane 63, which is read back as a wave-uniform value.
+template <int CTRL, int ROW_MASK>
+__device__ inline float dpp_move(float old, float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(v), CTRL,
+                                                    ROW_MASK, 0xf, false));
+}
 __device__ inline float wave_max(float v) {
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-  return v;
+  v = fmaxf(v, dpp_move<0xB1, 0xf>(v, v));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp_move<0x4E, 0xf>(v, v));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp_move<0x141, 0xf>(v, v));  // row_half_mirror
+  v = fmaxf(v, dpp_move<0x140, 0xf>(v, v));  // row_mirror
+  v = fmaxf(v, dpp_move<0x142, 0xa>(v, v));  // row_bcast:15 into rows 1 and 3
+  v = fmaxf(v, dpp_move<0x143, 0xc>(v, v));  // row_bcast:31 into rows 2 and 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 __device__ inline float wave_sum(float v) {
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-  return v;
+  v += dpp_move<0xB1, 0xf>(0.f, v);
+  v += dpp_move<0x4E, 0xf>(0.f, v);
+  v += dpp_move<0x141, 0xf>(0.f, v);
+  v += dpp_move<0x140, 0xf>(0.f, v);
+  v += dpp_move<0x142, 0xa>(0.f, v);
+  v += dpp_move<0x143, 0xc>(0.f, v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Candidate list: WAVES segments of kCap / WAVES keys (+2 so that a segment can be padded to an
+// even count for 16-byte reads); skey receives the same keys sorted descending.
 struct RowShared {
-  float cval[kCap];
-  int cidx[kCap];
-  float red[kRowWaves];
-  unsigned long long red64[kRowWaves];
-  int ired[kRowWaves];
-  int count;
+  unsigned long long ckey[kCap + 2 * kMaxRowWaves];
+  unsigned long long skey[kCap];
+  float red[kMaxRowWaves];
+  unsigned long long red64[kMaxRowWaves];
+  int ired[kMaxRowWaves];
+  int seg_count[kMaxRowWaves];
   int n_surv;
-  float thr;
   float logsum;
 };
 
+__device__ inline float key_value(unsigned long long k) { return unord((uint32_t)(k >> 32)); }
+__device__ inline int key_index(unsigned long long k) { return (int)(0xffffffffu - (uint32_t)k); }
+
+template <int THREADS>
 __device__ inline float block_max(float v, RowShared& sh) {
   v = wave_max(v);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = v;
   __syncthreads();
   float r = sh.red[0];
-  for (int w = 1; w < kRowWaves; ++w) r = fmaxf(r, sh.red[w]);
+  for (int w = 1; w < THREADS / 64; ++w) r = fmaxf(r, sh.red[w]);
   return r;
 }
-__device__ inline float block_min(float v, RowShared& sh) { return -block_max(-v, sh); }
+template <int THREADS>
+__device__ inline float block_min(float v, RowShared& sh) { return -block_max<THREADS>(-v, sh); }
+template <int THREADS>
 __device__ inline float block_sum(float v, RowShared& sh) {
   v = wave_sum(v);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = v;
   __syncthreads();
   float r = 0.f;
-  for (int w = 0; w < kRowWaves; ++w) r += sh.red[w];  // fixed order
+  for (int w = 0; w < THREADS / 64; ++w) r += sh.red[w];  // fixed order
   return r;
 }
+template <int THREADS>
 __device__ inline int block_isum(int v, RowShared& sh) {
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) sh.ired[threadIdx.x >> 6] = v;
   __syncthreads();
   int r = 0;
-  for (int w = 0; w < kRowWaves; ++w) r += sh.ired[w];
+  for (int w = 0; w < THREADS / 64; ++w) r += sh.ired[w];
   return r;
 }
+template <int THREADS>
 __device__ inline uint64_t block_max64(uint64_t v, RowShared& sh) {
   for (int off = 32; off > 0; off >>= 1) {
     const uint64_t o = __shfl_xor(v, off);
@@ -100,25 +129,35 @@ __device__ inline uint64_t block_max64(uint64_t v, RowShared& sh) {
   if ((threadIdx.x & 63) == 0) sh.red64[threadIdx.x >> 6] = v;
   __syncthreads();
   uint64_t r = sh.red64[0];
-  for (int w = 1; w < kRowWaves; ++w) r = sh.red64[w] > r ? sh.red64[w] : r;
+  for (int w = 1; w < THREADS / 64; ++w) r = sh.red64[w] > r ? sh.red64[w] : r;
   return r;
 }
 
-
-// Row index held in register j of this thread: 16-byte vectors interleaved over the workgroup.
+// Register j of a thread holds row index (j / VEC * THREADS + threadIdx.x) * VEC + j % VEC: 16-byte
+// vectors interleaved over the workgroup.  row_index_at() gives that index from an opaque copy of
+// threadIdx.x * VEC.  Loops over the register row call
+// row_base() right before they start: with a plain threadIdx.x the compiler computes all ITEMS
+// indices of every later loop at the top of the kernel and keeps them in registers.
 template <int VEC>
-__device__ inline int row_index_of(int j) {
-  return ((j / VEC) * kRowThreads + (int)threadIdx.x) * VEC + (j % VEC);
+__device__ inline int row_base() {
+  int base = (int)threadIdx.x * VEC;
+  asm volatile("" : "+v"(base));
+  return base;
+}
+template <int VEC, int THREADS>
+__device__ inline int row_index_at(int base, int j) {
+  return base + (j / VEC) * THREADS * VEC + (j % VEC);
 }
 
-// Loads one row (V elements of T) into x[ITEMS] as float; slots past V hold -inf.
-template <typename T, int ITEMS>
+// Loads one row (V elements of T) into x[ITEMS] as float; slots past V hold NaN, which no
+// comparison selects and fmaxf skips.
+template <typename T, int ITEMS, int THREADS>
 __device__ inline void load_row(const T* __restrict__ x_row, int V, float (&x)[ITEMS]) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int NV = ITEMS / VEC;
 #pragma unroll
   for (int c = 0; c < NV; ++c) {
-    const int i0 = (c * kRowThreads + (int)threadIdx.x) * VEC;
+    const int i0 = (c * THREADS + (int)threadIdx.x) * VEC;
     if (i0 + VEC <= V) {
       struct alignas(16) Pack { T v[VEC]; };
       const Pack p = *reinterpret_cast<const Pack*>(x_row + i0);
@@ -126,21 +165,18 @@ __device__ inline void load_row(const T* __restrict__ x_row, int V, float (&x)[I
       for (int e = 0; e < VEC; ++e) x[c * VEC + e] = Num<T>::load(&p.v[e]);
     } else {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) x[c * VEC + e] = (i0 + e < V) ? Num<T>::load(x_row + i0 + e) : -INFINITY;
+      for (int e = 0; e < VEC; ++e) x[c * VEC + e] = (i0 + e < V) ? Num<T>::load(x_row + i0 + e) : __builtin_nanf("");
     }
   }
 }
 
-// k-th largest value (with multiplicity) of the row held in x; every thread gets the result.
-// Ordinary rows: pivot + LDS candidate list + counting.  Overflowing rows: 32-step bisection.
-template <int ITEMS, int VEC>
-__device__ inline float row_kth_largest(const float (&x)[ITEMS], int V, int k_eff, RowShared& sh,
-                                        bool force_fallback) {
-  const int tid = threadIdx.x, lane = tid & 63;
-  float tmax = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) tmax = fmaxf(tmax, x[j]);
-  const int rounds = (k_eff + kRowWaves - 1) / kRowWaves;
+// Pivot with at least k_eff row entries >= it, from the per-thread maxima: the minimum over waves
+// of each wave's r-th largest maximum, r = ceil(k_eff / waves).
+template <int THREADS>
+__device__ inline float row_pivot(float tmax, int k_eff, RowShared& sh) {
+  constexpr int WAVES = THREADS / 64;
+  const int lane = threadIdx.x & 63;
+  const int rounds = (k_eff + WAVES - 1) / WAVES;
   float cur = tmax, wave_pivot = -INFINITY;
   for (int it = 0; it < rounds; ++it) {
     const float wm = wave_max(cur);
@@ -148,44 +184,105 @@ __device__ inline float row_kth_largest(const float (&x)[ITEMS], int V, int k_ef
     const uint64_t holders = __ballot(cur == wm);
     if (holders != 0 && lane == __builtin_ctzll(holders)) cur = -INFINITY;
   }
-  const float pivot = block_min(wave_pivot, sh);
-  if (tid == 0) sh.count = 0;
-  __syncthreads();
-  if (!force_fallback) {
+  return block_min<THREADS>(wave_pivot, sh);
+}
+
+// Lists key_of(x[j], row index) for every register entry >= pivot and sorts the list descending
+// into sh.skey.  Returns the number of keys, or -1 when a wave's segment overflowed.  Keys must be
+// distinct and nonzero (key64 of distinct indices is).  Ends with a barrier.
+template <int ITEMS, int VEC, int THREADS, typename KeyFn>
+__device__ inline int row_sorted_candidates(const float (&x)[ITEMS], float pivot, RowShared& sh,
+                                            KeyFn key_of) {
+  constexpr int WAVES = THREADS / 64, SEG = kCap / WAVES, STRIDE = SEG + 2;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  {
+    unsigned long long* seg = sh.ckey + wave * STRIDE;
+    const int base = row_base<VEC>();
+    int count = 0;  // wave-uniform
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
-      if (x[j] >= pivot && row_index_of<VEC>(j) < V) {
-        const int pos = atomicAdd(&sh.count, 1);
-        if (pos < kCap) sh.cval[pos] = x[j];
+      const bool take = x[j] >= pivot;
+      const uint64_t votes = __ballot(take);
+      if (votes != 0) {
+        if (take) {
+          const int pos = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(votes >> 32),
+                                       __builtin_amdgcn_mbcnt_lo((uint32_t)votes, 0u));
+          if (pos < SEG) seg[pos] = key_of(x[j], row_index_at<VEC, THREADS>(base, j));
+        }
+        count += __builtin_popcountll(votes);
       }
+    }
+    if (lane == 0) {
+      sh.seg_count[wave] = count;
+      if (count < SEG) seg[count] = 0ull;  // pad to an even count with a key below every real key
     }
   }
   __syncthreads();
-  const int n_c = force_fallback ? kCap + 1 : sh.count;
-  if (n_c <= kCap) {
-    for (int c = tid; c < n_c; c += kRowThreads) {
-      const float v = sh.cval[c];
-      int gt = 0, ge = 0;
-      for (int o = 0; o < n_c; ++o) {
-        const float ov = sh.cval[o];
-        gt += ov > v;
-        ge += ov >= v;
-      }
-      if (gt < k_eff && k_eff <= ge) sh.thr = v;
-    }
-    __syncthreads();
-    return sh.thr;
+  int n = 0;
+  bool overflow = false;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const int c = sh.seg_count[w];
+    overflow |= c > SEG;
+    n += c;
   }
+  if (overflow) return -1;
+  for (int c = tid; c < n; c += THREADS) {
+    int w = 0, off = c;
+    while (off >= sh.seg_count[w]) off -= sh.seg_count[w++];
+    const unsigned long long mine = sh.ckey[w * STRIDE + off];
+    int before = 0;
+    for (int w2 = 0; w2 < WAVES; ++w2) {
+      const int n2 = sh.seg_count[w2];
+      const ulonglong2* seg2 = reinterpret_cast<const ulonglong2*>(sh.ckey + w2 * STRIDE);
+      for (int o = 0; 2 * o < n2; ++o) {
+        const ulonglong2 kk = seg2[o];
+        before += (kk.x > mine) + (kk.y > mine);
+      }
+    }
+    sh.skey[before] = mine;
+  }
+  __syncthreads();
+  return n;
+}
+
+// Number of sorted keys whose value part is >= the value part of sh.skey[k - 1] (k <= n): the
+// entries that are >= the k-th largest value, ties included.  Ends with a barrier.
+template <int THREADS>
+__device__ inline int row_survivors(int n, int k, RowShared& sh) {
+  const uint32_t thr_hi = (uint32_t)(sh.skey[k - 1] >> 32);
+  for (int r = threadIdx.x; r < n; r += THREADS) {
+    const bool in = (uint32_t)(sh.skey[r] >> 32) >= thr_hi;
+    const bool next_in = r + 1 < n && (uint32_t)(sh.skey[r + 1] >> 32) >= thr_hi;
+    if (in && !next_in) sh.n_surv = r + 1;
+  }
+  __syncthreads();
+  return sh.n_surv;
+}
+
+// k-th largest value of round_T(x_row[i] - shift), i < V, by bisection on the ordered bit pattern:
+// exact for any input, 32 passes over the row in memory.  The rare path: it reads memory again
+// rather than the register copy so that it adds nothing to the register budget of its caller.
+template <typename T, int THREADS>
+__device__ inline float row_kth_bisect(const T* __restrict__ x_row, int V, float shift, int k_eff,
+                                       RowShared& sh) {
   uint32_t lo_k = 0u, hi_k = 0xffffffffu;  // invariant: count(>= lo_k) >= k_eff
   while (lo_k < hi_k) {
     const uint32_t mid = lo_k + (uint32_t)(((uint64_t)hi_k - lo_k + 1) >> 1);
     int cnt = 0;
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) cnt += (row_index_of<VEC>(j) < V) && ord(x[j]) >= mid;
-    cnt = block_isum(cnt, sh);
+    for (int i = threadIdx.x; i < V; i += THREADS)
+      cnt += ord(Num<T>::round(Num<T>::load(x_row + i) - shift)) >= mid;
+    cnt = block_isum<THREADS>(cnt, sh);
     if (cnt >= k_eff) lo_k = mid; else hi_k = mid - 1;
   }
   return unord(lo_k);
 }
+
+// Launch geometry for a vocabulary of V elements: threads per row x values per thread (a multiple
+// of the 16-byte vector for every dtype).  -1 when V is beyond the compiled limit.
+//   V <= 8192        256 threads x 32
+//   V <= 32768       256 threads x 128   (two workgroups per compute unit)
+//   V <= 65536      1024 threads x 64
+inline int row_geometry(int V) { return V <= 8192 ? 0 : (V <= 32768 ? 1 : (V <= 65536 ? 2 : -1)); }
 
 }  // namespace

@@ -19,29 +19,51 @@ constexpr int kThreads = 256;
 
 struct RowStats { float thr, zmax, log_sum, mask_z; };  // of z = filtered logits / T
 
-template <typename T, int ITEMS>
-__global__ __launch_bounds__(kRowThreads) void row_stats_kernel(
+template <typename T, int ITEMS, int THREADS>
+__global__ __launch_bounds__(THREADS) void row_stats_kernel(
     const T* __restrict__ logits, int64_t row_stride, int V, int top_k, float mask_value,
     float temperature, RowStats* __restrict__ stats, int force_fallback) {
   constexpr int VEC = 16 / sizeof(T);
   __shared__ RowShared sh;
+  const int tid = threadIdx.x;
+  const T* x_row = logits + (int64_t)blockIdx.x * row_stride;
   float x[ITEMS];
-  load_row<T, ITEMS>(logits + (int64_t)blockIdx.x * row_stride, V, x);
+  load_row<T, ITEMS, THREADS>(x_row, V, x);
   float tmax = -INFINITY;
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) tmax = fmaxf(tmax, x[j]);
-  const float row_max = block_max(tmax, sh);
+  const float row_max = block_max<THREADS>(tmax, sh);
   const int k_eff = top_k < V ? top_k : V;
-  const float thr = row_kth_largest<ITEMS, VEC>(x, V, k_eff, sh, force_fallback != 0);
   const float zmax = row_max / temperature;
   const float mask_z = mask_value / temperature;
-  float part = 0.f;
-#pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    if (row_index_of<VEC>(j) < V) part += expf((x[j] >= thr ? x[j] / temperature : mask_z) - zmax);
+  const float pivot = row_pivot<THREADS>(tmax, k_eff, sh);
+  int n_c = -1;
+  if (!force_fallback)
+    n_c = row_sorted_candidates<ITEMS, VEC, THREADS>(
+        x, pivot, sh, [](float v, int i) { return key64(v, (uint32_t)i); });
+  if (n_c >= k_eff) {
+    // the filter keeps skey[0 .. n_s); every other entry of the row counts as mask_z
+    const int n_s = row_survivors<THREADS>(n_c, k_eff, sh);
+    if (tid < 64) {
+      float part = 0.f;
+      for (int o = tid; o < n_s; o += 64) part += expf(key_value(sh.skey[o]) / temperature - zmax);
+      part = wave_sum(part);
+      if (tid == 0) {
+        const float sum = part + (float)(V - n_s) * expf(mask_z - zmax);
+        stats[blockIdx.x] = RowStats{key_value(sh.skey[k_eff - 1]), zmax, logf(sum), mask_z};
+      }
+    }
+    return;
   }
-  const float sum = block_sum(part, sh);
-  if (threadIdx.x == 0) stats[blockIdx.x] = RowStats{thr, zmax, logf(sum), mask_z};
+  // exact path from memory
+  const float thr = row_kth_bisect<T, THREADS>(x_row, V, 0.f, k_eff, sh);
+  float part = 0.f;
+  for (int i = tid; i < V; i += THREADS) {
+    const float v = Num<T>::load(x_row + i);
+    part += expf((v >= thr ? v / temperature : mask_z) - zmax);
+  }
+  const float sum = block_sum<THREADS>(part, sh);
+  if (tid == 0) stats[blockIdx.x] = RowStats{thr, zmax, logf(sum), mask_z};
 }
 
 __device__ inline float load_any(const void* p, int dtype, int64_t i) {
@@ -146,15 +168,15 @@ int launch_stats(const void* logits, int64_t row_stride, int64_t rows, int V, in
                  float temperature, void* stats, int force_fallback, hipStream_t s) {
   const T* x = reinterpret_cast<const T*>(logits);
   RowStats* st = reinterpret_cast<RowStats*>(stats);
-  constexpr int VEC = 16 / sizeof(T);
-  const int per_thread = (V + kRowThreads - 1) / kRowThreads;
-#define RD_STATS(ITEMS)                                                                              \
+#define RD_STATS(ITEMS, THREADS)                                                                     \
   do { rd::ScopedTiming rd_t("row_stats_kernel", s);                                                 \
-    hipLaunchKernelGGL((row_stats_kernel<T, ITEMS>), dim3(rows), dim3(kRowThreads), 0, s, x, row_stride, \
-                       V, top_k, mask_value, temperature, st, force_fallback); } while (0)
-  if (per_thread <= 8 && VEC <= 8) RD_STATS(8);
-  else if (per_thread <= 32) RD_STATS(32);
-  else RD_STATS(64);
+    hipLaunchKernelGGL((row_stats_kernel<T, ITEMS, THREADS>), dim3(rows), dim3(THREADS), 0, s, x,    \
+                       row_stride, V, top_k, mask_value, temperature, st, force_fallback); } while (0)
+  switch (row_geometry(V)) {
+    case 0: RD_STATS(32, 256); break;
+    case 1: RD_STATS(128, 256); break;
+    default: RD_STATS(64, 1024); break;
+  }
 #undef RD_STATS
   return rd::check_launch("rd_verify_row_stats");
 }
@@ -166,8 +188,8 @@ extern "C" int rd_verify_row_stats(const void* logits, int dtype, int64_t row_st
                                    float* stats, int force_fallback, void* stream) {
   RD_REQUIRE(rows > 0 && vocab > 0 && top_k > 0 && rows <= 2147483647LL, RD_EINVAL,
              "rd_verify_row_stats: bad sizes (rows %lld vocab %d top_k %d)", (long long)rows, vocab, top_k);
-  RD_REQUIRE(vocab <= 64 * kRowThreads && top_k <= 512, RD_ELIMIT,
-             "rd_verify_row_stats: vocab %d (<= %d), top_k %d (<= 512)", vocab, 64 * kRowThreads, top_k);
+  RD_REQUIRE(row_geometry(vocab) >= 0 && top_k <= 512, RD_ELIMIT,
+             "rd_verify_row_stats: vocab %d (<= 65536), top_k %d (<= 512)", vocab, top_k);
   RD_REQUIRE(logits && stats, RD_EINVAL, "rd_verify_row_stats: null pointer");
   RD_REQUIRE(temperature > 0.f, RD_EINVAL, "rd_verify_row_stats: temperature must be positive");
   RD_REQUIRE(dtype == RD_F32 || dtype == RD_BF16 || dtype == RD_F16, RD_EINVAL, "rd_verify_row_stats: unknown dtype %d", dtype);
