@@ -169,6 +169,29 @@ RD_API int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, int6
                          void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Rotary position embedding of the new queries and keys, fused with the in-place append of the
+ * new keys and values to one layer's cache slabs.  Replaces apply_rotary_pos_emb
+ * (modeling_llama.py:87-110) and the two View.cat calls (modeling_llama.py:148-159,
+ * kv_cache.py:24-32).
+ *
+ * q (batch, n_new, n_heads, head_dim), k and v (batch, n_new, n_kv_heads, head_dim): head_dim
+ * contiguous, heads head_dim apart, *_strides = {batch, token} element strides.  cos/sin: tables
+ * (table_rows, head_dim) in the same dtype, row p = the angles of position p (halves repeated,
+ * NeoX layout).  position_ids (batch, n_new) int64, clamped to the table.  q_out: same layout as q
+ * (may be q itself).  k_cache / v_cache: (batch, n_kv_heads, max_len, head_dim) slabs with element
+ * strides cache_strides = {batch, head, row}; rows [row0, row0 + n_new) are written.
+ * Every product and the sum are rounded to dtype, as the separate torch kernels round them.
+ * ------------------------------------------------------------------------------------------ */
+RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k,
+                          const int64_t* k_strides, const void* v, const int64_t* v_strides,
+                          int dtype, int batch, int n_new, int n_heads, int n_kv_heads,
+                          int head_dim, const void* cos, const void* sin, int64_t table_rows,
+                          const int64_t* position_ids, int64_t pos_batch_stride, void* q_out,
+                          const int64_t* q_out_strides, void* k_cache, void* v_cache,
+                          const int64_t* cache_strides, int64_t row0, int64_t max_len,
+                          void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Verification attention.
  *
  * rd_attn_prepare: once per LLM forward (where the reference builds the additive bias,

@@ -14,8 +14,8 @@
 //   r = ceil(50/waves) -- has at least 50 entries above it and, on ordinary data, not many more;
 //   entries >= p go to an LDS list, which is sorted by counting.  The max subtraction and the
 //   rounding are applied to the listed entries only.  If the list overflows or cannot decide a tie
-//   at the 50th value (heavy ties, adversarial layouts) the row falls back to a bisection on the
-//   value bits plus W rounds of block-wide argmax: slow, exact for any input.
+//   at the 50th value (heavy ties, adversarial layouts) the row falls back to a radix selection
+//   over the row in memory: several passes, exact for any input.
 // beam_merge_kernel (one workgroup per batch row): the W sorted lists are cut at the W-th largest
 //   of their leading entries, the few entries above the cut are ranked by counting.
 //
@@ -32,9 +32,12 @@ namespace {
 constexpr int kMaxWidth = 64;    // beam width limit of the merge kernel (W*W <= 4096 LDS keys)
 constexpr int kMergeThreads = 256;
 
-// The exact path for rows whose candidate list overflows: k-th largest value by bisection, then W
-// rounds of block-wide argmax over (score, index).  Works from memory (the row is in L2), not from
-// the caller's register copy, so that it costs the common path no registers.
+// The exact path for rows whose candidate list overflows or cannot settle a tie.  Works from memory
+// (the row is in L2), not from the caller's register copy, so that it costs the common path no
+// registers.  With t = round_T(x - max) and thr = the k-th largest t, the first W entries in
+// (score descending, index ascending) order are among: every entry with t > thr (fewer than k),
+// the first W entries by index with t == thr, and the first W by index with t < thr (the filtered
+// class, one common score).  Those are listed, scored and ranked by counting.
 template <typename T, int THREADS>
 __device__ void beam_row_fallback(const T* __restrict__ x_row, int V, float row_max, int k_eff,
                                   float mask_t, float lpb, int W, float* __restrict__ c_score,
@@ -42,31 +45,71 @@ __device__ void beam_row_fallback(const T* __restrict__ x_row, int V, float row_
                                   RowShared& sh) {
   const int tid = threadIdx.x;
   auto value = [&](int i) { return Num<T>::round(Num<T>::load(x_row + i) - row_max); };
-  const float thr = row_kth_bisect<T, THREADS>(x_row, V, row_max, k_eff, sh);
+  const float thr = row_kth_radix<T, THREADS>(x_row, V, row_max, k_eff, sh);
+  // every thread owns a contiguous index range, so that "first by index" is a prefix over threads
+  const int span = (V + THREADS - 1) / THREADS;
+  const int i_lo = tid * span < V ? tid * span : V, i_hi = i_lo + span < V ? i_lo + span : V;
+  int* n_eq = reinterpret_cast<int*>(sh.ckey);  // [THREADS] entries equal to thr per thread
+  int* n_lt = n_eq + THREADS;                   // [THREADS] entries below thr per thread
+  if (tid == 0) sh.n_surv = 0;                  // length of the list of entries above thr
+  __syncthreads();
   float part = 0.f;
-  for (int i = tid; i < V; i += THREADS) {
-    const float v = value(i);
-    part += v >= thr ? expf(v) : 0.f;
+  int eq = 0, lt = 0;
+  for (int i = i_lo; i < i_hi; ++i) {
+    const float t = value(i);
+    if (t >= thr) part += expf(t);
+    if (t > thr) sh.skey[atomicAdd(&sh.n_surv, 1)] = key64(t, (uint32_t)i);  // fewer than k_eff <= 512
+    eq += t == thr;
+    lt += t < thr;
   }
-  const float logsum = logf(block_sum<THREADS>(part, sh));
+  n_eq[tid] = eq;
+  n_lt[tid] = lt;
+  const float logsum = logf(block_sum<THREADS>(part, sh));  // has barriers
   const float masked_lp = Num<T>::round(mask_t - logsum);
-  auto log_prob = [&](float v) { return v >= thr ? Num<T>::round(v - logsum) : masked_lp; };
-  uint64_t last = ~0ull;
-  for (int w = 0; w < W; ++w) {
-    uint64_t best = 0ull;
-    for (int i = tid; i < V; i += THREADS) {
-      const uint64_t k = key64(log_prob(value(i)) + lpb, (uint32_t)i);
-      if (k < last && k > best) best = k;
-    }
-    best = block_max64<THREADS>(best, sh);
-    if (tid == 0) {
-      if (best == 0ull) { c_score[w] = -INFINITY; c_tok[w] = -1; }
-      else { c_score[w] = unord((uint32_t)(best >> 32)); c_tok[w] = (int32_t)(0xffffffffu - (uint32_t)best); }
-    }
-    last = best;
+  const int n_gt = sh.n_surv;
+  int eq_before = 0, lt_before = 0, eq_all = 0, lt_all = 0;
+  for (int j = 0; j < THREADS; ++j) {
+    const int e = n_eq[j], l = n_lt[j];
+    if (j < tid) { eq_before += e; lt_before += l; }
+    eq_all += e;
+    lt_all += l;
   }
+  const int take_eq = eq_all < W ? eq_all : W, take_lt = lt_all < W ? lt_all : W;
+  // list: [0, n_gt) above thr, [n_gt, n_gt + take_eq) equal, then take_lt filtered entries
+  if ((eq_before < W && eq > 0) || (lt_before < W && lt > 0)) {
+    int e = eq_before, l = lt_before;
+    for (int i = i_lo; i < i_hi; ++i) {
+      const float t = value(i);
+      if (t == thr) { if (e < W) sh.skey[n_gt + e] = key64(t, (uint32_t)i); ++e; }
+      else if (t < thr) { if (l < W) sh.skey[n_gt + take_eq + l] = key64(t, (uint32_t)i); ++l; }
+    }
+  }
+  __syncthreads();
+  // score keys (the per-thread counts in ckey are dead after the barrier above)
+  const int n_list = n_gt + take_eq + take_lt;
+  for (int c = tid; c < n_list; c += THREADS) {
+    const unsigned long long e = sh.skey[c];
+    const float lp = c < n_gt + take_eq ? Num<T>::round(key_value(e) - logsum) : masked_lp;
+    sh.ckey[c] = key64(lp + lpb, (uint32_t)key_index(e));
+  }
+  if (tid == 0) sh.ckey[n_list] = 0ull;
+  __syncthreads();
+  for (int c = tid; c < n_list; c += THREADS) {
+    const unsigned long long mine = sh.ckey[c];
+    const ulonglong2* k2 = reinterpret_cast<const ulonglong2*>(sh.ckey);
+    int rank = 0;
+    for (int o = 0; 2 * o < n_list; ++o) {
+      const ulonglong2 kk = k2[o];
+      rank += (kk.x > mine) + (kk.y > mine);
+    }
+    if (rank < W) { c_score[rank] = key_value(mine); c_tok[rank] = key_index(mine); }
+  }
+  for (int w = n_list + tid; w < W; w += THREADS) { c_score[w] = -INFINITY; c_tok[w] = -1; }  // V < W
   if (lo_row)
-    for (int i = tid; i < V; i += THREADS) lo_row[i] = log_prob(value(i));
+    for (int i = tid; i < V; i += THREADS) {
+      const float t = value(i);
+      lo_row[i] = t >= thr ? Num<T>::round(t - logsum) : masked_lp;
+    }
 }
 
 // ITEMS elements per thread, held as ITEMS/VEC vectors of VEC = 16 bytes / sizeof(T).

@@ -260,22 +260,55 @@ __device__ inline int row_survivors(int n, int k, RowShared& sh) {
   return sh.n_surv;
 }
 
-// k-th largest value of round_T(x_row[i] - shift), i < V, by bisection on the ordered bit pattern:
-// exact for any input, 32 passes over the row in memory.  The rare path: it reads memory again
-// rather than the register copy so that it adds nothing to the register budget of its caller.
+// k-th largest value of round_T(x_row[i] - shift), i < V, for any input: radix selection on the
+// ordered bit pattern, four passes over the row in memory (it sits in L2) with a 256-bin LDS
+// histogram each.  This is the rare path; it reads memory rather than the caller's register copy so
+// that it adds nothing to the caller's register budget.  Uses sh.ckey as the histogram.
 template <typename T, int THREADS>
-__device__ inline float row_kth_bisect(const T* __restrict__ x_row, int V, float shift, int k_eff,
-                                       RowShared& sh) {
-  uint32_t lo_k = 0u, hi_k = 0xffffffffu;  // invariant: count(>= lo_k) >= k_eff
-  while (lo_k < hi_k) {
-    const uint32_t mid = lo_k + (uint32_t)(((uint64_t)hi_k - lo_k + 1) >> 1);
-    int cnt = 0;
-    for (int i = threadIdx.x; i < V; i += THREADS)
-      cnt += ord(Num<T>::round(Num<T>::load(x_row + i) - shift)) >= mid;
-    cnt = block_isum<THREADS>(cnt, sh);
-    if (cnt >= k_eff) lo_k = mid; else hi_k = mid - 1;
+__device__ inline float row_kth_radix(const T* __restrict__ x_row, int V, float shift, int k_eff,
+                                      RowShared& sh) {
+  int* hist = reinterpret_cast<int*>(sh.ckey);
+  const int tid = threadIdx.x, lane = tid & 63;
+  uint32_t prefix = 0u, known = 0u;  // bits of the answer found so far, and their mask
+  int k = k_eff;                     // rank of the answer among the keys that match the prefix
+  for (int shift_bits = 24; shift_bits >= 0; shift_bits -= 8) {
+    __syncthreads();
+    for (int i = tid; i < 256; i += THREADS) hist[i] = 0;
+    __syncthreads();
+    for (int i0 = 0; i0 < V; i0 += THREADS) {
+      const int i = i0 + tid;
+      bool live = false;
+      int bin = 0;
+      if (i < V) {
+        const uint32_t key = ord(Num<T>::round(Num<T>::load(x_row + i) - shift));
+        live = (key & known) == prefix;
+        bin = (key >> shift_bits) & 255;
+      }
+      // tied rows put whole waves into one bin: the first live lane's bin is added once per wave
+      const uint64_t lives = __ballot(live);
+      if (lives == 0) continue;
+      const int lead_bin = __shfl(bin, __builtin_ctzll(lives));
+      const uint64_t same = __ballot(live && bin == lead_bin);
+      if (lane == __builtin_ctzll(lives)) atomicAdd(&hist[lead_bin], __builtin_popcountll(same));
+      if (live && bin != lead_bin) atomicAdd(&hist[bin], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      int above = 0, b = 255;
+      for (; b > 0; --b) {
+        if (above + hist[b] >= k) break;
+        above += hist[b];
+      }
+      sh.ired[0] = b;
+      sh.ired[1] = k - above;
+    }
+    __syncthreads();
+    prefix |= (uint32_t)sh.ired[0] << shift_bits;
+    known |= 255u << shift_bits;
+    k = sh.ired[1];
   }
-  return unord(lo_k);
+  __syncthreads();
+  return unord(prefix);
 }
 
 // Launch geometry for a vocabulary of V elements: threads per row x values per thread (a multiple

@@ -56,7 +56,7 @@ __global__ __launch_bounds__(THREADS) void row_stats_kernel(
     return;
   }
   // exact path from memory
-  const float thr = row_kth_bisect<T, THREADS>(x_row, V, 0.f, k_eff, sh);
+  const float thr = row_kth_radix<T, THREADS>(x_row, V, 0.f, k_eff, sh);
   float part = 0.f;
   for (int i = tid; i < V; i += THREADS) {
     const float v = Num<T>::load(x_row + i);

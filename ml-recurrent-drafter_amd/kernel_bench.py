@@ -188,7 +188,26 @@ def case_kv(rows, reps):
                {"kv_compact_kernel": "GB/s"})
 
 
-CASES = dict(tree=case_tree, tree_x64=lambda r, n: case_tree(r, n, 64), attention=case_attention, beam=case_beam,
+def case_rope(rows, reps):
+    prev, n = 1500, 181
+    cache = kv_cache.Cache(B, prev + n + 8, 1, H, D, torch.bfloat16, torch.device("cuda"))
+    torch.manual_seed(2)
+    q, k, v = (torch.randn(B, n, H * D, device="cuda").to(torch.bfloat16) for _ in range(3))
+    ang = torch.outer(torch.arange(prev + n, device="cuda").float(),
+                      1.0 / (10000.0 ** (torch.arange(0, D, 2, device="cuda").float() / D)))
+    cos, sin = (torch.cat((f, f), -1).to(torch.bfloat16) for f in (ang.cos(), ang.sin()))
+    pos = torch.randint(prev, prev + 5, (B, n), device="cuda")
+
+    def step():
+        cache.set_length(prev)
+        kv_cache.rope_append(q, k, v, cos, sin, pos, cache.sliced[0])
+
+    kt = timed(step, reps)
+    report(rows, f"rope + append prev {prev} n {n}", kt, {"rope_append_kernel": 2 * 3 * B * n * H * D * 2},
+           {"rope_append_kernel": "GB/s"})
+
+
+CASES = dict(rope=case_rope, tree=case_tree, tree_x64=lambda r, n: case_tree(r, n, 64), attention=case_attention, beam=case_beam,
              logits=case_logits, kv=case_kv)
 
 

@@ -36,6 +36,10 @@ _PROTOTYPES = {
     "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P]),
     "rd_kv_unpack": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _I, _I, _P]),
     "rd_kv_compact": (_I, [_P, _I, _I, _I, _L, _L, _L, _I, _P, _P]),
+    "rd_rope_append": (
+        _I,
+        [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _L, _P],
+    ),
     "rd_attn_plan_ints": (_Z, [_I, _I, _I]),
     "rd_attn_bits_words": (_Z, [_I, _I, _I]),
     "rd_attn_prepare": (_I, [_P, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P]),

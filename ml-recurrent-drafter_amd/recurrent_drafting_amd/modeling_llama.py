@@ -120,13 +120,10 @@ class LlamaAttention(nn.Module):
     def forward(self, hidden_states: torch.Tensor, position_ids: torch.LongTensor,
                 past_key_value: KeyValue, attention_mask: attention.PreparedMask) -> torch.Tensor:
         bsz, q_len, _ = hidden_states.size()
-        q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-        k = self.k_proj(hidden_states).view(bsz, q_len, self.n_kv_heads, self.head_dim).transpose(1, 2)
-        v = self.v_proj(hidden_states).view(bsz, q_len, self.n_kv_heads, self.head_dim).transpose(1, 2)
+        q, k, v = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
         cos, sin = self.rotary_emb(v.device, v.dtype, q_len + past_key_value[0].shape[-2])
-        q, k = apply_rotary_pos_emb(q, k, cos, sin, position_ids)
-        keys = past_key_value[0].cat(k)  # in place; strided view of the cache
-        values = past_key_value[1].cat(v)
+        # rotation of q (in place) and k, append of k and v to the cache: one kernel
+        q, keys, values = kv_cache.rope_append(q, k, v, cos, sin, position_ids, past_key_value)
         out = attention.masked_attention(q, keys, values, attention_mask)  # (B, q_len, hidden)
         return self.o_proj(out)
 
