@@ -8,18 +8,24 @@
 //
 // Two kernels behind one entry point:
 //   attn_mfma_kernel      bf16, head_dim 128: S^T = K Q^T and O^T = V^T P^T on
-//                         v_mfma_f32_32x32x16_bf16.  512 threads = 8 waves, each wave owns 32 query
-//                         rows; a 64-key K tile and the transposed V tile are staged in LDS (double
-//                         buffered) and shared by the 8 waves; online softmax in fp32.  With the transposed
-//                         products a query row lives in one lane pair, so the row maximum and sum
-//                         need a single cross-lane exchange, and P^T is already laid out as the
-//                         B operand of the second product.
+//                         v_mfma_f32_32x32x16_bf16.  512 threads = 8 waves; a wave owns 32 query
+//                         rows (with at most 128 rows per workgroup, two waves share a row block
+//                         and split every tile's keys).  64-key K tiles and transposed V tiles
+//                         travel global -> register ring -> LDS and are shared by the waves.  The
+//                         loop is a software pipeline over 32-key units: while the vector ALU turns
+//                         the scores of one unit into probabilities (online softmax in fp32, lazy
+//                         rescale), the matrix pipeline already multiplies the next unit's keys.
+//                         With the transposed products a query row lives in one lane pair, so the
+//                         row maximum and sum need a single cross-lane exchange, and P^T is already
+//                         laid out as the B operand of the second product.
 //   attn_generic_kernel   any dtype, head_dim <= 256, one workgroup per (row, head, query); the
 //                         correctness path for shapes the MFMA kernel does not cover.
 // Work items come from the plan (attn_plan.h): (batch row, key range) chunks, longest first; rows
 // whose keys are split over several items write fp32 partials that attn_combine_kernel merges.
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
+
+#include <type_traits>
 
 #include "attn_plan.h"
 
@@ -52,10 +58,25 @@ constexpr int kD = 128;
 constexpr int kTile = 64;                  // keys per tile
 constexpr int kWaves = 8;
 constexpr int kMfmaThreads = kWaves * 64;  // 512
-constexpr int kRowsPerWG = kWaves * 32;    // 256 query rows: K/V tiles are staged once per key range
-constexpr int kBuffers = 2;                // LDS tile buffers (2: stage tile t+1 while t is consumed)
+// The 8 waves split into kWaves / KSPLIT row blocks of 32 query rows and KSPLIT key parts: with
+// KSPLIT = 2 (at most 128 query rows per workgroup) waves 0-3 take the first 32 keys of every tile
+// and waves 4-7 the last 32, each with its own running maximum, sum and accumulators, merged
+// through LDS at the end -- otherwise half of the waves would have no rows and the other half would
+// serialise their MFMA and softmax phases alone on their SIMDs.
+constexpr int rows_per_wg(int ksplit) { return (kWaves / ksplit) * 32; }
+constexpr int kKBuffers = 3;               // K tiles in LDS: K(t+1) is multiplied while K(t+2) is staged
+constexpr int kVBuffers = 2;               // V tiles in LDS: V(t) is multiplied while V(t+1) is staged
+constexpr int kRing = 2;                   // register stages of tiles on their way from memory
+
+template <int N, typename F, int I = 0>
+__device__ __attribute__((always_inline)) inline void rd_static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    rd_static_for<N, F, I + 1>(static_cast<F&&>(f));
+  }
+}
 constexpr int kKsStride = kD + 8;          // bf16 elements; 272-byte rows spread 16 lanes over all banks
-constexpr int kVtStride = kTile + 4;       // bf16 elements; 136-byte rows
+constexpr int kVtStride = kTile + 8;       // bf16 elements; 144-byte rows: 16-byte aligned, conflict-free
 
 // max over the two lanes (l, l^32) that share a query row
 __device__ inline float pair_max(float v) {
@@ -72,9 +93,16 @@ __device__ inline float pair_sum(float v) {
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
+template <int KSPLIT>
 __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) __bf16 s_k[kBuffers][kTile * kKsStride];
-  __shared__ __attribute__((aligned(16))) __bf16 s_vt[kBuffers][kD * kVtStride];
+  constexpr int kRowWaves = kWaves / KSPLIT;  // row blocks per workgroup
+  constexpr int kRowsPerWG = kRowWaves * 32;
+  constexpr int kKeys = kTile / KSPLIT;       // keys of a tile that one wave handles
+  constexpr int kKeyBlocks = kKeys / 32, kKeySteps = kKeys / 16;
+  constexpr int kKBytes = kKBuffers * kTile * kKsStride * 2, kVBytes = kVBuffers * kD * kVtStride * 2;
+  __shared__ __attribute__((aligned(16))) char smem[kKBytes + kVBytes];
+  __bf16 (*s_k)[kTile * kKsStride] = reinterpret_cast<__bf16 (*)[kTile * kKsStride]>(smem);
+  __bf16 (*s_vt)[kD * kVtStride] = reinterpret_cast<__bf16 (*)[kD * kVtStride]>(smem + kKBytes);
 
   const int item = blockIdx.y;
   if (item >= a.plan[0]) return;
@@ -86,10 +114,12 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const int q_tiles = gridDim.x / a.H;
   const int h = blockIdx.x / q_tiles, q_tile = blockIdx.x - h * q_tiles;
   const int hk = h / (a.H / a.Hkv);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and the compiler knows it
   const int g = lane >> 5, r = lane & 31;
-  const int q_row = q_tile * kRowsPerWG + wave * 32 + r;
-  const bool wave_active = q_tile * kRowsPerWG + wave * 32 < a.n_q;
+  const int row_wave = wave % kRowWaves, kp = wave / kRowWaves;  // row block and key part of this wave
+  const int q_row = q_tile * kRowsPerWG + row_wave * 32 + r;
+  const bool wave_active = q_tile * kRowsPerWG + row_wave * 32 < a.n_q;
   const bool row_valid = q_row < a.n_q;
 
   const __bf16* kbase = reinterpret_cast<const __bf16*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh;
@@ -117,92 +147,159 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const float scale_log2 = a.scale * 1.4426950408889634f;
 
   // Loader roles: threads [0,256) stage K rows (keys lrow+16*i), threads [256,512) stage V
-  // transposed (keys 4*lrow+i); four 16-byte chunks each per tile.
-  const bool k_loader = tid < 256;
+  // transposed (keys 4*lrow+i); four 16-byte chunks each per tile.  The V threads map lanes to
+  // (chunk, key quad) so that the 16 lanes of one LDS write cycle hit 16 different bank pairs: lane
+  // bits 0-1 and 4-5 select the chunk, bits 2-3 and 6-7 the key quad.
+  const bool k_loader = wave < kWaves / 2;
   const int lt = tid & 255;
-  const int chunk = lt & 15;  // 16-byte column chunk of a 256-byte row
-  const int lrow = lt >> 4;
-  bf16x8 pre[4];
-  auto prefetch = [&](int key0) {
-    const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = key0 + (k_loader ? lrow + 16 * i : 4 * lrow + i);
-      const __bf16* p = (k_loader ? kbase + (int64_t)key * a.k_ss : vbase + (int64_t)key * a.v_ss) + 8 * chunk;
-      pre[i] = key < a.kv_len ? *reinterpret_cast<const bf16x8*>(p) : z;
-    }
-  };
-  auto stage = [&](int buf) {
-    if (k_loader) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        *reinterpret_cast<bf16x8*>(&s_k[buf][(lrow + 16 * i) * kKsStride + 8 * chunk]) = pre[i];
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        bf16x4 t = {pre[0][e], pre[1][e], pre[2][e], pre[3][e]};
-        *reinterpret_cast<bf16x4*>(&s_vt[buf][(8 * chunk + e) * kVtStride + 4 * lrow]) = t;
-      }
-    }
-  };
+  const int chunk = k_loader ? (lt & 15) : ((lt & 3) | (((lt >> 4) & 3) << 2));  // 16-byte column chunk of a row
+  const int lrow = k_loader ? (lt >> 4) : (((lt >> 2) & 3) | ((lt >> 6) << 2));
+  // V^T rows hold the keys of every 16-key group in the order [0-3, 8-11, 4-7, 12-15]: the eight
+  // keys that one lane feeds to a 16-key MFMA step are then 16 contiguous bytes.
+  const int vt_col = 16 * (lrow >> 2) + 4 * (((lrow & 1) << 1) | ((lrow >> 1) & 1));
 
   const int n_tiles = (hi - lo + kTile - 1) / kTile;
-  // Vector-memory loads complete in issue order, so a load that is needed soon must be issued
-  // BEFORE the long-latency tile prefetch: the mask word of tile t+1 is fetched one iteration
-  // ahead, in front of the K/V loads of tile t+2.
-  uint64_t word_next = 0ull;
-  if (n_tiles > 0) {
-    word_next = row_valid ? brow[lo >> 6] : 0ull;
-    prefetch(lo);
-    stage(0);
-    if (kBuffers == 2 && n_tiles > 1) prefetch(lo + kTile);
-  }
-  __syncthreads();
-  for (int t = 0; t < n_tiles; ++t) {
-    const int key0 = lo + t * kTile;
-    const int buf = kBuffers == 2 ? (t & 1) : 0;
-    if (kBuffers == 2) {
-      // the other buffer was last read in iteration t-1, which every wave has left
-      if (t + 1 < n_tiles) stage(buf ^ 1);
+  // Tiles in flight: a ring of kRing register stages between global memory and LDS; tile j
+  // passes through slot j % kRing.  The mask words travel in a ring of their own.
+  // Every step issues the same loads on every path (tile indices past the end are clamped to the
+  // last tile, keys past kv_len to the last key): with loads under divergent or data-dependent
+  // branches the compiler can no longer count which loads are still in flight and waits for all
+  // of them at every use, which would cap the ring at one tile.
+  static_assert(kRing == 2, "two named register stages");
+  // the four 16-byte chunks a thread carries per tile, for ring slots 0 (a) and 1 (b); plain
+  // variables: grouped in arrays or structs they are left in scratch memory
+  bf16x8 a0, a1, a2, a3, b0, b1, b2, b3;
+  uint64_t wring[kRing];
+  // address of a 16-byte chunk = wave-uniform part (tile, i) + 32-bit lane part
+  const char* base = reinterpret_cast<const char*>(k_loader ? kbase : vbase);
+  const int64_t row_bytes = (k_loader ? a.k_ss : a.v_ss) * 2;
+  const int key_step = k_loader ? 16 : 1;   // this thread's keys within a tile: first_key + i * key_step
+  const int first_key = k_loader ? lrow : 4 * lrow;
+  const uint32_t lane_off = (uint32_t)(first_key * row_bytes + 16 * chunk);
+  auto fetch_into = [&](bf16x8& c0, bf16x8& c1, bf16x8& c2, bf16x8& c3, int j) __attribute__((always_inline)) {
+    const int key0 = lo + (j < n_tiles ? j : n_tiles - 1) * kTile;
+    const char* tile = base + (int64_t)key0 * row_bytes;
+    const int64_t step_bytes = key_step * row_bytes;
+    int64_t o0 = lane_off, o1 = step_bytes + lane_off, o2 = 2 * step_bytes + lane_off, o3 = 3 * step_bytes + lane_off;
+    if (key0 + kTile > a.kv_len) {
+      // the last tile of a row: keys past kv_len re-read the last key
+      auto clamped = [&](int i) __attribute__((always_inline)) {
+        const int rel = first_key + i * key_step;
+        const int use = key0 + rel < a.kv_len ? rel : a.kv_len - 1 - key0;
+        return (int64_t)use * row_bytes + 16 * chunk;
+      };
+      o0 = clamped(0); o1 = clamped(1); o2 = clamped(2); o3 = clamped(3);
     }
-    const uint64_t word = word_next;
-    if (t + 1 < n_tiles) word_next = row_valid ? brow[(key0 + kTile) >> 6] : 0ull;
-    if (t + kBuffers < n_tiles) prefetch(key0 + kBuffers * kTile);
+    c0 = *reinterpret_cast<const bf16x8*>(tile + o0);
+    c1 = *reinterpret_cast<const bf16x8*>(tile + o1);
+    c2 = *reinterpret_cast<const bf16x8*>(tile + o2);
+    c3 = *reinterpret_cast<const bf16x8*>(tile + o3);
+  };
+  auto fetch_tile = [&](auto slot_c, int j) __attribute__((always_inline)) {
+    if constexpr (decltype(slot_c)::value == 0) fetch_into(a0, a1, a2, a3, j); else fetch_into(b0, b1, b2, b3, j);
+  };
+  auto fetch_word = [&](auto slot_c, int j) __attribute__((always_inline)) {
+    const int key0 = lo + (j < n_tiles ? j : n_tiles - 1) * kTile;
+    const uint64_t w = brow[key0 >> 6];
+    wring[decltype(slot_c)::value] = row_valid ? w : 0ull;
+  };
+  auto stage_k_from = [&](bf16x8 c0, bf16x8 c1, bf16x8 c2, bf16x8 c3, int j) __attribute__((always_inline)) {
+    __bf16* dst = s_k[j % kKBuffers] + lrow * kKsStride + 8 * chunk;
+    *reinterpret_cast<bf16x8*>(dst) = c0;
+    *reinterpret_cast<bf16x8*>(dst + 16 * kKsStride) = c1;
+    *reinterpret_cast<bf16x8*>(dst + 32 * kKsStride) = c2;
+    *reinterpret_cast<bf16x8*>(dst + 48 * kKsStride) = c3;
+  };
+  auto stage_k = [&](auto slot_c, int j) __attribute__((always_inline)) {
+    if constexpr (decltype(slot_c)::value == 0) stage_k_from(a0, a1, a2, a3, j); else stage_k_from(b0, b1, b2, b3, j);
+  };
+  auto stage_v_from = [&](bf16x8 p0, bf16x8 p1, bf16x8 p2, bf16x8 p3, int j) __attribute__((always_inline)) {
+    __bf16* dst = s_vt[j % kVBuffers] + 8 * chunk * kVtStride + vt_col;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      bf16x4 t = {p0[e], p1[e], p2[e], p3[e]};
+      *reinterpret_cast<bf16x4*>(dst + e * kVtStride) = t;
+    }
+  };
+  auto stage_v = [&](auto slot_c, int j) __attribute__((always_inline)) {
+    if constexpr (decltype(slot_c)::value == 0) stage_v_from(a0, a1, a2, a3, j); else stage_v_from(b0, b1, b2, b3, j);
+  };
+
+  // S^T of one unit: 32 keys x 32 queries; accumulator i is key 8*(i/4) + 4*g + i%4 of the unit.
+  // A wave walks through kUnits units per tile: both 32-key halves (KSPLIT 1) or its own half.
+  constexpr int kUnits = kKeys / 32;
+  static_assert((kRing * kUnits) % 2 == 0, "the score registers alternate between two sets per unit");
+  f32x16 s_reg[2];
+  auto k_frag = [&](const __bf16* sk, int key_off, int ks) __attribute__((always_inline)) {
+    return *reinterpret_cast<const bf16x8*>(&sk[(key_off + r) * kKsStride + 16 * ks + 8 * g]);
+  };
+
+  // ---- prologue: K of tiles 0 and 1 and V of tile 0 into LDS, the ring filled behind them --------
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1 % kRing>;
+  uint64_t word = row_valid ? brow[lo >> 6] : 0ull;  // mask word of the tile whose scores are being formed
+  // K runs one tile further ahead than V (K(t+1) is multiplied during step t); both roles keep
+  // the tile that step t stages in ring slot (t + 1) % kRing, so that one piece of code, with
+  // the same registers, serves both.
+  const int ahead = k_loader ? 2 : 1;
+  if (k_loader) {
+    fetch_tile(S0{}, 0);
+    fetch_tile(S1{}, 1);
+    stage_k(S0{}, 0);
+    stage_k(S1{}, 1);
+  } else {
+    fetch_tile(S0{}, 0);
+    stage_v(S0{}, 0);
+  }
+  rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) {
+    constexpr int J = decltype(j)::value;
+    fetch_tile(std::integral_constant<int, (J + 1) % kRing>{}, ahead + J);
+  });
+  rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) {
+    constexpr int J = decltype(j)::value;
+    fetch_word(std::integral_constant<int, (1 + J) % kRing>{}, 1 + J);
+  });
+  __syncthreads();
+  if (wave_active) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s_reg[0][i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+      s_reg[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(s_k[0], kp * kKeys, ks), qf[ks], s_reg[0], 0, 0, 0);
+  }
+
+  // ---- one unit per step -----------------------------------------------------------------------
+  // A step holds S of its unit in registers.  It multiplies the next unit's K by Q on the matrix
+  // pipeline while the vector ALU turns S into P (two scores per MFMA, in source order), then adds
+  // V^T P^T; the last step of a tile stages the tiles that later steps need in between.
+  auto unit_step = [&](auto j_c, auto u_c, int t) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;  // t % kRing
+    constexpr int U = decltype(u_c)::value;  // unit of the tile
+    constexpr int CUR = (J * kUnits + U) & 1;
+    constexpr bool kLast = U == kUnits - 1;
+    f32x16& s_cur = s_reg[CUR];
+    f32x16& s_next = s_reg[CUR ^ 1];
+    const int key_off = kp * kKeys + 32 * U;                       // this unit's keys within the tile
+    const int next_off = kLast ? kp * kKeys : key_off + 32;
+    bf16x8 pf[2];  // P^T of the unit, the B operand of the second product
     if (wave_active) {
-      const __bf16* sk = s_k[buf];
-      const __bf16* sv = s_vt[buf];
-      // S^T tile: 64 keys x 32 queries, two 32x32 blocks
-      f32x16 s[2];
+      // mask, running maximum, lazy rescale: short, not overlapped
+      const uint32_t mine = (uint32_t)(word >> key_off);
+      if (!__all(mine == ~0u)) {
+        const uint32_t w = mine >> (4 * g);
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&sk[(32 * kb + r) * kKsStride + 16 * ks + 8 * g]);
-          s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[ks], s[kb], 0, 0, 0);
+        for (int i = 0; i < 16; ++i) {
+          const bool on = (w >> (8 * (i >> 2) + (i & 3))) & 1u;
+          s_cur[i] = on ? s_cur[i] : -INFINITY;
         }
-      }
-      // accumulator i of block kb is key 32*kb + 8*(i/4) + 4*g + i%4 of the tile
-      if (!__all(word == ~0ull)) {
-        const uint32_t w[2] = {(uint32_t)(word >> (4 * g)), (uint32_t)(word >> (32 + 4 * g))};
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const bool on = (w[kb] >> (8 * (i >> 2) + (i & 3))) & 1u;
-            s[kb][i] = on ? s[kb][i] : -INFINITY;
-          }
       }
       float tmax = -INFINITY;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[kb][i]);
+      for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s_cur[i]);
       tmax = pair_max(tmax) * scale_log2;
       // The running maximum only has to bound the exponents, not equal the true maximum: it is
-      // raised (and O, l rescaled) only when the tile exceeds it by more than kSlack, so most
-      // tiles skip the 64-register rescale.  p <= 2^kSlack stays far inside bf16/fp32 range.
+      // raised (and O, l rescaled) only when a unit exceeds it by more than kSlack, so most units
+      // skip the 64-register rescale.  p <= 2^kSlack stays far inside bf16/fp32 range.
       constexpr float kSlack = 8.f;
       const bool raise = tmax > m + kSlack || m == -INFINITY;
       if (__any(raise)) {
@@ -217,43 +314,111 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
         m = m_new;
       }
       const float m_use = m == -INFINITY ? 0.f : m;
+      // S(next unit) = K Q^T  ||  P = exp2(S * scale - m).  After the last unit the product reads
+      // a stale buffer; its result is never used.
+      const __bf16* sk = s_k[(kLast ? t + 1 : t) % kKBuffers];
       float psum = 0.f;
-      bf16x8 pf[4];
+      constexpr int kDepth = 4;  // K fragments in flight from LDS (a read takes longer than two MFMAs)
+      bf16x8 ka[kDepth];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+      for (int d = 0; d < kDepth; ++d) ka[d] = k_frag(sk, next_off, d);
 #pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          const float p0 = fast_exp2(fmaf(s[kb][i], scale_log2, -m_use));
-          const float p1 = fast_exp2(fmaf(s[kb][i + 1], scale_log2, -m_use));
-          psum += p0 + p1;
-          const f32x2 pp = {p0, p1};
-          const bf16x2 pb = __builtin_convertvector(pp, bf16x2);
-          pf[2 * kb + (i >> 3)][i & 7] = pb[0];
-          pf[2 * kb + (i >> 3)][(i & 7) + 1] = pb[1];
-        }
+      for (int i = 0; i < 16; ++i) s_next[i] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        s_next = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[q % kDepth], qf[q], s_next, 0, 0, 0);
+        if (q + kDepth < 8) ka[q % kDepth] = k_frag(sk, next_off, q + kDepth);
+        const int i = 2 * q;
+        const float p0 = fast_exp2(fmaf(s_cur[i], scale_log2, -m_use));
+        const float p1 = fast_exp2(fmaf(s_cur[i + 1], scale_log2, -m_use));
+        psum += p0 + p1;
+        const f32x2 pp = {p0, p1};
+        const bf16x2 pb = __builtin_convertvector(pp, bf16x2);
+        pf[i >> 3][i & 7] = pb[0];
+        pf[i >> 3][(i & 7) + 1] = pb[1];
+        // the order written here is the order wanted: the vector work of two scores runs while the
+        // matrix pipeline works through the MFMA in front of it
+        __builtin_amdgcn_sched_barrier(0);
+      }
       l += psum;
-      // O^T += V^T P^T ; k-slot j of lane group g is key 16*t + 4*g + (j%4) + 8*(j/4)
+      // P is used only after the staging branches below: pin it here, or its computation is sunk
+      // behind them and out from under the MFMAs
+      asm volatile("" : "+v"(pf[0]), "+v"(pf[1]));
+    }
+    // the first V fragments are requested before the staging code, so that they have arrived when
+    // the second product starts
+    constexpr int kVDepth = 4;
+    bf16x8 va[kVDepth];
+    const __bf16* sv = s_vt[t % kVBuffers] + key_off + 8 * g;
+    auto v_frag = [&](int c) __attribute__((always_inline)) {
+      return *reinterpret_cast<const bf16x8*>(&sv[(32 * (c >> 1) + r) * kVtStride + 16 * (c & 1)]);
+    };
+    if (wave_active) {
 #pragma unroll
-      for (int db = 0; db < 4; ++db) {
+      for (int c = 0; c < kVDepth; ++c) va[c] = v_frag(c);
+    }
+    if (kLast) {
+      // stage and fetch before the second product: the LDS writes and the V transposes run under it
+      using Slot = std::integral_constant<int, (J + 1) % kRing>;
+      if (k_loader) stage_k(Slot{}, t + 2); else stage_v(Slot{}, t + 1);
+      fetch_tile(Slot{}, t + ahead + kRing);
+    }
+    if (wave_active) {
+      // O^T += V^T P^T ; k-slot j of lane group g is key 16*tt + 4*g + (j%4) + 8*(j/4) of the unit,
+      // stored at columns 16*tt + 8*g + j of the V^T row
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-          const __bf16* vp = &sv[(32 * db + r) * kVtStride + 16 * tt + 4 * g];
-          const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(vp);
-          const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(vp + 8);
-          const bf16x8 va = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pf[tt], o[db], 0, 0, 0);
-        }
+      for (int c = 0; c < 8; ++c) {
+        o[c >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[c % kVDepth], pf[c & 1], o[c >> 1], 0, 0, 0);
+        if (c + kVDepth < 8) va[c % kVDepth] = v_frag(c + kVDepth);
       }
     }
-    __syncthreads();
-    if (kBuffers == 1 && t + 1 < n_tiles) {
-      stage(0);  // every wave has left tile t
+    if (kLast) {
+      // mask word of tile t+1, and the word of tile t+1+kRing takes its slot
+      word = wring[(J + 1) % kRing];
+      fetch_word(std::integral_constant<int, (J + 1) % kRing>{}, t + 1 + kRing);
       __syncthreads();
     }
+  };
+  for (int t0 = 0; t0 < n_tiles; t0 += kRing) {
+    rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) {
+      constexpr int J = decltype(j)::value;
+      if (t0 + J < n_tiles)
+        rd_static_for<kUnits>([&](auto u) __attribute__((always_inline)) { unit_step(j, u, t0 + J); });
+    });
   }
 
-  if (!wave_active) return;
   l = pair_sum(l);
+  if (KSPLIT == 2) {
+    // merge the two key parts of every row block: part 1 hands (m, l, o) over through LDS (the tile
+    // buffers are free: every wave has passed the loop's last barrier)
+    float* x_o = reinterpret_cast<float*>(smem);             // [row block][64 accumulators][lane]
+    float* x_ml = x_o + kRowWaves * 64 * 64;                 // [row block][2][lane]
+    static_assert((kWaves / 2) * (64 * 64 + 2 * 64) * 4 <= kKBytes + kVBytes, "merge buffer");
+    if (kp == 1 && wave_active) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x_o[(row_wave * 64 + 16 * db + i) * 64 + lane] = o[db][i];
+      x_ml[(row_wave * 2 + 0) * 64 + lane] = m;
+      x_ml[(row_wave * 2 + 1) * 64 + lane] = l;
+    }
+    __syncthreads();
+    if (kp == 1) return;
+    if (wave_active) {
+      const float m2 = x_ml[(row_wave * 2 + 0) * 64 + lane], l2 = x_ml[(row_wave * 2 + 1) * 64 + lane];
+      const float m_new = fmaxf(m, m2);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float a1 = fast_exp2(m - m_safe), a2 = fast_exp2(m2 - m_safe);  // exp2(-inf) = 0
+      l = a1 * l + a2 * l2;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          o[db][i] = a1 * o[db][i] + a2 * x_o[(row_wave * 64 + 16 * db + i) * 64 + lane];
+      m = m_new;
+    }
+  }
+  if (!wave_active) return;
   if (!row_valid) return;
   // accumulator i of block db is d = 32*db + 8*(i/4) + 4*g + i%4
   if (n_splits == 1) {
@@ -450,10 +615,17 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
     a.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
                                          rd::align_up(slots * n_q * head_dim * sizeof(float), 256));
     const int max_items = batch * a.max_splits;
-    const int q_tiles = (n_q + kRowsPerWG - 1) / kRowsPerWG;
+    const int ksplit = n_q <= rows_per_wg(2) ? 2 : 1;
+    const int q_tiles = (n_q + rows_per_wg(ksplit) - 1) / rows_per_wg(ksplit);
     RD_REQUIRE(max_items <= 65535 && (int64_t)q_tiles * n_heads <= 2147483647LL, RD_ELIMIT,
                "rd_verify_attention: grid too large");
-    { rd::ScopedTiming rd_t("attn_mfma_kernel", s); hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, a); }
+    {
+      rd::ScopedTiming rd_t("attn_mfma_kernel", s);
+      if (ksplit == 2)
+        hipLaunchKernelGGL(attn_mfma_kernel<2>, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, a);
+      else
+        hipLaunchKernelGGL(attn_mfma_kernel<1>, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, a);
+    }
     if (int e = rd::check_launch("rd_verify_attention(mfma)")) return e;
     if (a.max_splits > 1) {
       { rd::ScopedTiming rd_t("attn_combine_kernel", s); hipLaunchKernelGGL(attn_combine_kernel, dim3(n_heads, batch, kCombineSlices), dim3(kD), 0, s, a); }

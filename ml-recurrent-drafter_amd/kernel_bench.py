@@ -90,11 +90,11 @@ def case_tree(rows, reps, replicate=1):
                {x: "GB/s" for x in work}, note=f"whole pack moves {io + work['tree_mask_kernel']} algorithmic bytes")
 
 
-def attention_case(seed=123, full_len=None):
+def attention_case(seed=123, full_len=None, p_copy=0.6):
     rng = np.random.default_rng(seed)
     lens = rng.integers(500, 2549, size=B) if full_len is None else np.full(B, full_len)
     S = int(lens.max())
-    beams = torch.tensor(synthetic_beams(B, W, L, seed=seed), device="cuda")
+    beams = torch.tensor(synthetic_beams(B, W, L, seed=seed, p_copy=p_copy), device="cuda")
     ids_mask = torch.zeros((B, S), dtype=torch.bool, device="cuda")
     for b in range(B):
         ids_mask[b, S - int(lens[b]):] = True
@@ -108,9 +108,11 @@ def attention_case(seed=123, full_len=None):
 
 
 def case_attention(rows, reps):
-    for label, full_len in (("cached length U[500,2548]", None), ("cached length 2548 for every row", 2548),
-                            ("cached length 525 for every row", 525)):
-        lens, n, kv, mask, q, k_, v_ = attention_case(full_len=full_len)
+    for label, full_len, p_copy in (("cached length U[500,2548]", None, 0.6), ("cached length 2548 for every row", 2548, 0.6),
+                                    ("cached length 525 for every row", 525, 0.6),
+                                    ("narrow tree, cached length U[500,2548]", None, 0.93),
+                                    ("narrow tree, cached length 525 for every row", 525, 0.93)):
+        lens, n, kv, mask, q, k_, v_ = attention_case(full_len=full_len, p_copy=p_copy)
         prep = attention.prepare(mask, n_heads=H)
         kt = timed(lambda: attention.masked_attention(q, k_, v_, prep), reps)
         kp = timed(lambda: attention.prepare(mask, n_heads=H), reps)

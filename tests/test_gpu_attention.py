@@ -141,6 +141,7 @@ def test_generic_kernel_random_mask_with_empty_rows():
 @pytest.mark.parametrize("B,H,Hkv,W,L,prev_lens", [
     (1, 1, 1, 2, 3, [40]),            # one tile, one item
     (2, 2, 2, 8, 5, [100, 37]),       # ragged prefix, < 64 queries
+    (2, 2, 2, 24, 5, [300, 150]),     # 64..128 queries: four row blocks, keys of a tile split over wave pairs
     (2, 4, 2, 45, 5, [700, 1300]),    # > 32 queries per wave, split keys, GQA
     (1, 2, 2, 64, 5, [64]),           # > 256 queries: two query tiles
     (3, 2, 2, 16, 4, [2000, 5, 900]),  # several splits and a nearly empty prefix
