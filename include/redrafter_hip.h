@@ -169,6 +169,24 @@ RD_API int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, int6
                          void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Elementwise chains of the decoder layer around the projections, one pass each.
+ *
+ * rd_add_rms_norm: h = x + delta when delta is given (the "hidden_states += ..." of
+ * modeling_llama.py:196, :198; h is written to h_out, which may be x), else h = x;
+ * y = weight * cast(h * rsqrt(mean(h^2) + eps)) with float32 statistics (LlamaRMSNorm.forward,
+ * modeling_llama.py:27-32).  Rows of `cols` contiguous elements, row strides in elements.
+ *
+ * rd_silu_mul: y = silu(gate) * up (LlamaMLP.forward, modeling_llama.py:84-85, for
+ * hidden_act "silu"); gate and up are row-strided views, e.g. the halves of one fused projection.
+ * ------------------------------------------------------------------------------------------ */
+RD_API int rd_add_rms_norm(const void* x, int64_t x_row_stride, const void* delta,
+                           int64_t delta_row_stride, const void* weight, void* y,
+                           int64_t y_row_stride, void* h_out, int64_t h_row_stride, int dtype,
+                           int64_t rows, int cols, float eps, void* stream);
+RD_API int rd_silu_mul(const void* gate, const void* up, int64_t in_row_stride, void* y,
+                       int64_t y_row_stride, int dtype, int64_t rows, int cols, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Rotary position embedding of the new queries and keys, fused with the in-place append of the
  * new keys and values to one layer's cache slabs.  Replaces apply_rotary_pos_emb
  * (modeling_llama.py:87-110) and the two View.cat calls (modeling_llama.py:148-159,

@@ -19,9 +19,34 @@ from transformers.modeling_outputs import CausalLMOutput
 from transformers.modeling_utils import PreTrainedModel
 from transformers.models.llama.configuration_llama import LlamaConfig
 
-from . import attention, kv_cache
+from . import _hip, attention, kv_cache
 
 KeyValue = Tuple[kv_cache.View, kv_cache.View]
+
+
+def _fused_weight(owner: nn.Module, name: str, linears) -> torch.Tensor:
+    """One (sum of out_features, in_features) weight behind several bias-free Linear layers that
+    read the same input.  The layers' own parameters become row slices of it (no second copy,
+    checkpoints load and save under the usual names); rebuilt when a parameter was replaced."""
+    fused = owner.__dict__.get(name)
+    if fused is not None:
+        offset, ok = 0, True
+        for lin in linears:
+            w = lin.weight
+            ok = ok and w.dtype == fused.dtype and w.device == fused.device and \
+                w.data_ptr() == fused.data_ptr() + offset * fused.element_size()
+            offset += w.numel()
+        if ok:
+            return fused
+    assert all(lin.bias is None for lin in linears)
+    fused = torch.cat([lin.weight.data for lin in linears], dim=0)
+    row = 0
+    for lin in linears:
+        n = lin.weight.shape[0]
+        lin.weight.data = fused[row : row + n]
+        row += n
+    owner.__dict__[name] = fused
+    return fused
 
 
 class LlamaRMSNorm(nn.Module):
@@ -30,11 +55,26 @@ class LlamaRMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size))
         self.variance_epsilon = eps
 
-    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
-        # statistics in float32, result rounded to the activations' dtype before the gain
-        x = hidden_states.float()
-        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
-        return self.weight * x.to(hidden_states.dtype)
+    def forward(self, hidden_states: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """weight * cast(x * rsqrt(mean(x^2) + eps)), statistics in float32 (modeling_llama.py:27-32).
+        With `delta`, hidden_states += delta first, in place, in the same pass (the residual update
+        that precedes every norm of a decoder stack)."""
+        x = hidden_states
+        assert x.stride(-1) == 1 and self.weight.dtype == x.dtype and self.weight.is_contiguous()
+        rows = x.numel() // x.shape[-1]
+        x2 = x.view(rows, x.shape[-1]) if x.is_contiguous() else x.reshape(rows, x.shape[-1])
+        in_place = x2.data_ptr() == x.data_ptr()
+        d2 = None
+        if delta is not None:
+            assert delta.shape == x.shape and delta.dtype == x.dtype and in_place
+            d2 = delta.reshape(rows, x.shape[-1])
+            assert d2.stride(-1) == 1
+        y = torch.empty_like(x2)
+        _hip.check(_hip.lib().rd_add_rms_norm(
+            _hip.ptr(x2), x2.stride(0), _hip.ptr(d2), 0 if d2 is None else d2.stride(0), _hip.ptr(self.weight),
+            _hip.ptr(y), y.stride(0), _hip.ptr(x2) if d2 is not None else None, x2.stride(0),
+            _hip.dtype_code(x.dtype), rows, x.shape[-1], float(self.variance_epsilon), _hip.stream()))
+        return y.view(x.shape)
 
 
 class LlamaRotaryEmbedding(nn.Module):
@@ -87,8 +127,21 @@ class LlamaMLP(nn.Module):
         self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
         self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
         self.act_fn = ACT2FN[config.hidden_act]
+        self._silu = config.hidden_act == "silu"
 
     def forward(self, x):
+        if self._silu:
+            # one projection for gate and up, one pass for silu(gate) * up
+            weight = _fused_weight(self, "_gate_up", (self.gate_proj, self.up_proj))
+            gate_up = nn.functional.linear(x, weight)
+            inter = self.gate_proj.out_features
+            rows = gate_up.numel() // (2 * inter)
+            gu = gate_up.view(rows, 2 * inter)
+            act = torch.empty((rows, inter), dtype=x.dtype, device=x.device)
+            _hip.check(_hip.lib().rd_silu_mul(
+                _hip.ptr(gu), _hip.ptr(gu[:, inter:]), gu.stride(0), _hip.ptr(act), act.stride(0),
+                _hip.dtype_code(x.dtype), rows, inter, _hip.stream()))
+            return self.down_proj(act.view(*x.shape[:-1], inter))
         return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
 
 
@@ -120,7 +173,10 @@ class LlamaAttention(nn.Module):
     def forward(self, hidden_states: torch.Tensor, position_ids: torch.LongTensor,
                 past_key_value: KeyValue, attention_mask: attention.PreparedMask) -> torch.Tensor:
         bsz, q_len, _ = hidden_states.size()
-        q, k, v = self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states)
+        # one projection for q, k and v; the three are column slices of its output
+        qkv = nn.functional.linear(hidden_states, _fused_weight(self, "_qkv", (self.q_proj, self.k_proj, self.v_proj)))
+        nq, nk = self.q_proj.out_features, self.k_proj.out_features
+        q, k, v = qkv[..., :nq], qkv[..., nq : nq + nk], qkv[..., nq + nk :]
         cos, sin = self.rotary_emb(v.device, v.dtype, q_len + past_key_value[0].shape[-2])
         # rotation of q (in place) and k, append of k and v to the cache: one kernel
         q, keys, values = kv_cache.rope_append(q, k, v, cos, sin, position_ids, past_key_value)
@@ -137,10 +193,19 @@ class LlamaDecoderLayer(nn.Module):
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
 
     def forward(self, hidden_states, position_ids, past_key_value, attention_mask):
-        hidden_states += self.self_attn(self.input_layernorm(hidden_states), position_ids,
-                                        past_key_value, attention_mask)
-        hidden_states += self.mlp(self.post_attention_layernorm(hidden_states))
+        hidden_states, delta = self.forward_deferred(hidden_states, None, position_ids, past_key_value,
+                                                     attention_mask)
+        hidden_states += delta
         return hidden_states
+
+    def forward_deferred(self, hidden_states, delta, position_ids, past_key_value, attention_mask):
+        """The layer with its last residual update left to the caller: takes the pending update of
+        the layer before (`delta`, or None) and returns (hidden_states, pending update), so that
+        every "hidden_states += ..." (modeling_llama.py:196, :198) runs inside the norm that
+        follows it."""
+        attn = self.self_attn(self.input_layernorm(hidden_states, delta), position_ids, past_key_value,
+                              attention_mask)
+        return hidden_states, self.mlp(self.post_attention_layernorm(hidden_states, attn))
 
 
 class LlamaPreTrainedModel(PreTrainedModel):
@@ -164,10 +229,11 @@ class LlamaModel(LlamaPreTrainedModel):
         if not isinstance(attention_mask, attention.PreparedMask):
             attention_mask = attention.prepare(
                 attention_mask, fix_empty_rows=False, n_heads=self.config.num_attention_heads)
-        hidden_states = self.embed_tokens(input_ids)
+        hidden_states, delta = self.embed_tokens(input_ids), None
         for layer, key_value in zip(self.layers, past_key_values):
-            hidden_states = layer(hidden_states, position_ids, key_value, attention_mask)
-        return self.norm(hidden_states)
+            hidden_states, delta = layer.forward_deferred(hidden_states, delta, position_ids, key_value,
+                                                          attention_mask)
+        return self.norm(hidden_states, delta)
 
 
 class LlamaForCausalLM(LlamaPreTrainedModel):

@@ -1,0 +1,105 @@
+"""rd_add_rms_norm and rd_silu_mul against the torch restatement of the reference's op chains
+(modeling_llama.py:27-32, :84-85, :196-198), and the fused projections against separate ones."""
+
+import pytest
+import torch
+
+from oracle import torch_path
+
+pytestmark = pytest.mark.gpu
+
+# about one unit in the last place of the dtype, relative (a few for float32: two roundings): the mean of squares is summed in another order
+# than torch sums it, so a value may round the other way at a tie
+ULP = {torch.float32: 1e-6, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}
+
+
+def _close(got, want, dtype, max_off_fraction=0.01):
+    got, want = got.float().cpu(), want.float()
+    assert got.shape == want.shape
+    if dtype != torch.float32:  # in 16 bits a float32 ulp of the statistics rarely shows at all
+        off = got != want
+        assert off.float().mean().item() <= max_off_fraction, off.float().mean().item()
+    torch.testing.assert_close(got, want, rtol=ULP[dtype], atol=1e-30)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(1, 8), (5, 128), (7, 344), (33, 4096), (3, 5120), (2, 8192)])
+def test_rms_norm_and_fused_residual(rows, cols, dtype):
+    from recurrent_drafting_amd import modeling_llama
+
+    g = torch.Generator().manual_seed(rows * 1000 + cols)
+    x = (torch.randn(rows, cols, generator=g) * 1.7).to(dtype)
+    delta = torch.randn(rows, cols, generator=g).to(dtype)
+    weight = (1.0 + 0.1 * torch.randn(cols, generator=g)).to(dtype)
+    norm = modeling_llama.LlamaRMSNorm(cols, eps=1e-5).to(dtype).cuda()
+    with torch.no_grad():
+        norm.weight.copy_(weight)
+        got = norm(x.cuda().view(1, rows, cols))
+        _close(got.view(rows, cols), torch_path._rms_norm(x, weight, 1e-5), dtype)
+        hidden = x.cuda().view(1, rows, cols).clone()
+        got2 = norm(hidden, delta.cuda().view(1, rows, cols))
+        summed = x + delta  # rounded to dtype, as "hidden_states += delta" rounds it
+        assert torch.equal(hidden.cpu().view(rows, cols), summed)  # updated in place, bit for bit
+        _close(got2.view(rows, cols), torch_path._rms_norm(summed, weight, 1e-5), dtype)
+
+
+def test_rms_norm_constant_rows_closed_form():
+    """x = c everywhere: mean(x^2) = c^2, y = weight * c / sqrt(c^2 + eps)."""
+    from recurrent_drafting_amd import modeling_llama
+
+    norm = modeling_llama.LlamaRMSNorm(256, eps=0.0).cuda()
+    x = torch.full((4, 256), 3.0, device="cuda")
+    x[1] = -0.5
+    with torch.no_grad():
+        y = norm(x)
+    want = torch.sign(x)
+    torch.testing.assert_close(y, want, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,hidden,inter", [(3, 128, 344), (17, 256, 1024), (9, 512, 11008)])
+def test_mlp_fused_projection_and_silu_mul(rows, hidden, inter, dtype):
+    from recurrent_drafting_amd import modeling_llama
+    from transformers.models.llama.configuration_llama import LlamaConfig
+
+    torch.manual_seed(rows + inter)
+    cfg = LlamaConfig(hidden_size=hidden, intermediate_size=inter, num_hidden_layers=1, num_attention_heads=4,
+                      num_key_value_heads=4, vocab_size=32, hidden_act="silu")
+    mlp = modeling_llama.LlamaMLP(cfg).to(dtype).cuda()
+    with torch.no_grad():
+        for p in mlp.parameters():
+            p.normal_(0.0, 0.05)
+        x = torch.randn(2, rows, hidden, device="cuda").to(dtype)
+        gate, up, down = (w.detach().clone() for w in (mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight))
+        got = mlp(x)
+        # the layers' parameters are now slices of one buffer and still hold their values
+        assert torch.equal(mlp.gate_proj.weight, gate) and torch.equal(mlp.up_proj.weight, up)
+        assert mlp.up_proj.weight.data_ptr() == mlp.gate_proj.weight.data_ptr() + gate.numel() * gate.element_size()
+        g_, u_ = torch.nn.functional.linear(x, gate), torch.nn.functional.linear(x, up)
+        want_act = torch.nn.functional.silu(g_) * u_  # torch's own kernels on the same device
+        want = torch.nn.functional.linear(want_act, down)
+        tol = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 5e-3}[dtype]
+        torch.testing.assert_close(got.float(), want.float(), rtol=tol, atol=tol * want.float().abs().max().item())
+        # the activation kernel alone, on identical inputs, against the CPU op chain
+        gu = torch.cat((g_, u_), dim=-1).view(-1, 2 * inter)
+        act = torch.empty((gu.shape[0], inter), dtype=dtype, device="cuda")
+        from recurrent_drafting_amd import _hip
+        _hip.check(_hip.lib().rd_silu_mul(_hip.ptr(gu), _hip.ptr(gu[:, inter:]), gu.stride(0), _hip.ptr(act), act.stride(0),
+                                          _hip.dtype_code(dtype), gu.shape[0], inter, _hip.stream()))
+        cpu = torch.nn.functional.silu(g_.cpu()) * u_.cpu()
+        _close(act, cpu.view(-1, inter), dtype)
+        # a replaced parameter is noticed
+        mlp.gate_proj.weight = torch.nn.Parameter(gate * 2)
+        torch.testing.assert_close(mlp(x).float(), torch.nn.functional.linear(
+            torch.nn.functional.silu(torch.nn.functional.linear(x, gate * 2)) * u_, down).float(),
+            rtol=tol, atol=tol * want.float().abs().max().item() * 2)
+
+
+def test_argument_errors():
+    from recurrent_drafting_amd import _hip
+
+    x = torch.zeros(2, 12, device="cuda")
+    w = torch.ones(12, device="cuda")
+    rc = _hip.lib().rd_add_rms_norm(_hip.ptr(x), 12, None, 0, _hip.ptr(w), _hip.ptr(x), 12, None, 0,
+                                    _hip.dtype_code(torch.float32), 2, 10, 1e-6, _hip.stream())
+    assert rc != 0 and b"multiple" in _hip.lib().rd_last_error()
