@@ -99,8 +99,11 @@ def gpu_run(steps: int, warmup: int):
         done += 1
     torch.cuda.synchronize()
 
+    # HIP events around every launch of the dominant kernel, live in the timed region (the events
+    # of ALL kernels would cost a few percent of the step; those are taken on the extra steps below)
     shapes = []
     attention.shape_log = shapes
+    _hip.timing_select("attn_mfma_kernel")
     _hip.timing_enable(True)
     elapsed, tokens, timed = 0.0, 0, 0
     first_len = last_len = None
@@ -125,8 +128,9 @@ def gpu_run(steps: int, warmup: int):
             stream = new_stream(ledger)
             for _ in range(warmup):
                 next(stream)
-    kernels = _hip.timing_collect()
+    dominant = _hip.timing_collect()
     _hip.timing_enable(False)
+    _hip.timing_select(None)
     attention.shape_log = None
     accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
     # the generator that is still open has not posted its record yet; close it to flush
@@ -139,8 +143,14 @@ def gpu_run(steps: int, warmup: int):
     # stage breakdown with the reference's synchronised timers, on a few extra steps
     ledger2 = rd.stats.Ledger(sync=True)
     s2 = new_stream(ledger2)
-    for _ in range(6):
+    next(s2)
+    next(s2)
+    _hip.timing_enable(True)  # every kernel of the library, on four steps
+    for _ in range(4):
         next(s2)
+    torch.cuda.synchronize()
+    kernels = _hip.timing_collect()
+    _hip.timing_enable(False)
     s2.close()
     wt = ledger2.records[0]["wall_times"]
     stage = {k: sum(v[2:]) / len(v[2:]) for k, v in wt.items()}
@@ -148,6 +158,7 @@ def gpu_run(steps: int, warmup: int):
 
     result = dict(
         elapsed=elapsed, steps=timed, tokens=tokens, per_seq_tokens=per_seq_tokens, kernels=kernels,
+        dominant=dominant,
         shapes=shapes, stage=stage, ref_style_tokens_per_second=ref_style,
         context=(first_len, last_len), no_pads=no_pads,
     )
@@ -157,29 +168,43 @@ def gpu_run(steps: int, warmup: int):
 
 
 def attention_roofline(run):
-    """Algorithmic FLOPs of every verify-attention launch in the timed region over the summed
-    duration of attn_mfma_kernel: 4 * heads * head_dim * n_q * sum_b(keys_b) per launch."""
+    """The dominant kernel against the roof that binds it.  Per launch, from the shapes the timed
+    region actually ran: algorithmic FLOPs 4 * heads * head_dim * n_q * sum_b(keys_b), algorithmic
+    bytes K and V once (2 * heads * head_dim * 2 B per key) plus Q and O once; duration = HIP events
+    around every launch in the timed region.  Arithmetic intensity below the machine balance
+    (2500 TFLOP/s / 8 TB/s = 312 FLOP/B) means the HBM roof binds, above it the MFMA roof."""
     H, D = LLAMA_7B["num_attention_heads"], LLAMA_7B["hidden_size"] // LLAMA_7B["num_attention_heads"]
-    count, total_ms = run["kernels"].get("attn_mfma_kernel", (0, 0.0))
+    count, total_ms = run["dominant"].get("attn_mfma_kernel", (0, 0.0))
     shapes = run["shapes"][:count] if count else []
-    flops = sum(4.0 * H * D * n_q * B * kv for (B, n_q, kv) in shapes)
     if not count or total_ms <= 0:
         return None
-    achieved = flops / (total_ms * 1e-3) / 1e12
+    flops = sum(4.0 * H * D * n_q * B * kv for (B, n_q, kv) in shapes)
     k_bytes = sum(2.0 * H * D * 2 * B * kv + 2.0 * B * H * n_q * D * 2 for (B, n_q, kv) in shapes)
+    seconds = total_ms * 1e-3
+    tflops, gbs = flops / seconds / 1e12, k_bytes / seconds / 1e9
+    hbm_bound = flops / k_bytes < MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
     traffic = None
     path = os.path.join(ROOT, "profiles", "attn_mfma_kernel_traffic.json")
     if os.path.exists(path):
         with open(path) as f:
             traffic = json.load(f).get("hbm_bytes_per_launch")
-    return dict(
-        kernel="attn_mfma_kernel", bound="mfma", achieved=round(achieved, 2), peak=MFMA_BF16_PEAK_TFLOPS,
-        unit="TFLOP/s", frac=round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), traffic=traffic,
-        launches=count, avg_us=round(total_ms * 1e3 / count, 2),
+    out = dict(kernel="attn_mfma_kernel")
+    if hbm_bound:
+        out.update(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(gbs / HBM_PEAK_GBS, 4))
+    else:
+        out.update(bound="mfma", achieved=round(tflops, 2), peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
+                   frac=round(tflops / MFMA_BF16_PEAK_TFLOPS, 4))
+    out.update(
+        traffic=traffic, launches=count, avg_us=round(total_ms * 1e3 / count, 2),
         algorithmic_gflop_per_launch=round(flops / count / 1e9, 3),
         algorithmic_mb_per_launch=round(k_bytes / count / 1e6, 2),
-        hbm_frac_of_peak=round(k_bytes / (total_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        flop_per_byte=round(flops / k_bytes, 1),
+        mfma_frac_of_peak=round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+        hbm_frac_of_peak=round(gbs / HBM_PEAK_GBS, 4),
+        mean_n_q=round(sum(n for (_, n, _) in shapes) / len(shapes), 1),
+        mean_kv_len=round(sum(kv for (_, _, kv) in shapes) / len(shapes), 1),
     )
+    return out
 
 
 # -------------------------------------------------------------------------------------------------

@@ -49,8 +49,11 @@ RD_API const char* rd_last_error(void);
  * (the one place this library allocates) and makes every entry point bracket each of its kernel
  * launches with two events on the launch stream; rd_timing_collect waits for them and writes one
  * text line per kernel, "<kernel> <launches> <total_ms>", into a HOST buffer, then resets the
- * pool.  rd_timing_enable(0) stops recording. */
+ * pool.  rd_timing_enable(0) stops recording.  rd_timing_select("kernel_name") restricts the
+ * recording to one kernel (the events of every launch cost a few percent of a decode step);
+ * NULL or "" selects all again. */
 RD_API int rd_timing_enable(int on);
+RD_API int rd_timing_select(const char* kernel);
 RD_API int rd_timing_collect(char* out, size_t out_bytes);
 
 /* ------------------------------------------------------------------------------------------

@@ -28,6 +28,7 @@ constexpr int kTimingSlots = 16384;
 struct TimingState {
   std::mutex mu;
   bool enabled = false;
+  std::string only;  // when not empty: the one kernel that is timed
   int used = 0;
   std::vector<hipEvent_t> start, stop;
   std::vector<const char*> name;
@@ -42,6 +43,7 @@ ScopedTiming::ScopedTiming(const char* name, hipStream_t stream) : stream_(strea
   TimingState& t = timing();
   if (!t.enabled) return;
   std::lock_guard<std::mutex> lock(t.mu);
+  if (!t.only.empty() && t.only != name) return;
   if (t.used >= (int)t.start.size()) return;  // pool exhausted: later launches go untimed
   slot_ = t.used++;
   t.name[slot_] = name;
@@ -71,6 +73,13 @@ extern "C" int rd_timing_enable(int on) {
   }
   t.enabled = on != 0;
   t.used = 0;
+  return RD_OK;
+}
+
+extern "C" int rd_timing_select(const char* kernel) {
+  auto& t = rd::timing();
+  std::lock_guard<std::mutex> lock(t.mu);
+  t.only = kernel ? kernel : "";
   return RD_OK;
 }
 

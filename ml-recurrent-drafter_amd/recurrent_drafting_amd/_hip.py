@@ -24,6 +24,7 @@ _PROTOTYPES = {
     "rd_version": (C.c_int, []),
     "rd_last_error": (C.c_char_p, []),
     "rd_timing_enable": (_I, [_I]),
+    "rd_timing_select": (_I, [C.c_char_p]),
     "rd_timing_collect": (_I, [C.c_char_p, _Z]),
     "rd_tree_workspace_bytes": (_Z, [_I, _I, _I]),
     "rd_tree_build": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
@@ -123,6 +124,11 @@ def dtype_code(dt: torch.dtype) -> int:
 def timing_enable(on: bool) -> None:
     """Per-kernel HIP-event timing inside the library (a measurement aid; off by default)."""
     check(lib().rd_timing_enable(int(on)))
+
+
+def timing_select(kernel: str | None) -> None:
+    """Time only the named kernel (None: all kernels)."""
+    check(lib().rd_timing_select(kernel.encode() if kernel else None))
 
 
 def timing_collect() -> dict:
