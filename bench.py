@@ -129,6 +129,7 @@ def gpu_run(steps: int, warmup: int):
             for _ in range(warmup):
                 next(stream)
     dominant = _hip.timing_collect()
+    null_us = _hip.timing_null_kernel_us(64)
     _hip.timing_enable(False)
     _hip.timing_select(None)
     attention.shape_log = None
@@ -158,7 +159,7 @@ def gpu_run(steps: int, warmup: int):
 
     result = dict(
         elapsed=elapsed, steps=timed, tokens=tokens, per_seq_tokens=per_seq_tokens, kernels=kernels,
-        dominant=dominant,
+        dominant=dominant, null_us=null_us,
         shapes=shapes, stage=stage, ref_style_tokens_per_second=ref_style,
         context=(first_len, last_len), no_pads=no_pads,
     )
@@ -201,6 +202,9 @@ def attention_roofline(run):
         flop_per_byte=round(flops / k_bytes, 1),
         mfma_frac_of_peak=round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
         hbm_frac_of_peak=round(gbs / HBM_PEAK_GBS, 4),
+        # HIP events span dispatch and completion signalling too; an empty kernel timed the same way
+        # gives that fixed part (a kernel trace reports about avg_us minus this)
+        null_kernel_event_us=round(run["null_us"], 2),
         mean_n_q=round(sum(n for (_, n, _) in shapes) / len(shapes), 1),
         mean_kv_len=round(sum(kv for (_, _, kv) in shapes) / len(shapes), 1),
     )

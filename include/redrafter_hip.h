@@ -54,6 +54,10 @@ RD_API const char* rd_last_error(void);
  * NULL or "" selects all again. */
 RD_API int rd_timing_enable(int on);
 RD_API int rd_timing_select(const char* kernel);
+/* Average event-to-event time of an EMPTY kernel timed the same way, in microseconds: the fixed
+ * part (dispatch and completion signalling) that the figures of rd_timing_collect include and a
+ * kernel trace does not.  Synchronises the stream. */
+RD_API int rd_timing_null_kernel_us(int launches, void* stream, float* avg_us);
 RD_API int rd_timing_collect(char* out, size_t out_bytes);
 
 /* ------------------------------------------------------------------------------------------

@@ -50,6 +50,19 @@ ScopedTiming::ScopedTiming(const char* name, hipStream_t stream) : stream_(strea
   (void)hipEventRecord(t.start[slot_], stream_);
 }
 
+void timing_events(const char* name, hipEvent_t* start, hipEvent_t* stop) {
+  *start = *stop = nullptr;
+  TimingState& t = timing();
+  if (!t.enabled) return;
+  std::lock_guard<std::mutex> lock(t.mu);
+  if (!t.only.empty() && t.only != name) return;
+  if (t.used >= (int)t.start.size()) return;
+  const int slot = t.used++;
+  t.name[slot] = name;
+  *start = t.start[slot];
+  *stop = t.stop[slot];
+}
+
 ScopedTiming::~ScopedTiming() {
   if (slot_ < 0) return;
   (void)hipEventRecord(timing().stop[slot_], stream_);

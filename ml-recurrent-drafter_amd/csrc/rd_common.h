@@ -37,6 +37,11 @@ struct ScopedTiming {
   int slot_;
 };
 
+// For launches made with hipExtLaunchKernelGGL, which stamps the two events with the kernel's own
+// begin and end (no dispatch latency in between, unlike events recorded around a launch): hands
+// out a pair from the timing pool, or two nulls when this kernel is not being timed.
+void timing_events(const char* name, hipEvent_t* start, hipEvent_t* stop);
+
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 

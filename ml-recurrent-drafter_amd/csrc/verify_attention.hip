@@ -23,6 +23,7 @@
 // Work items come from the plan (attn_plan.h): (batch row, key range) chunks, longest first; rows
 // whose keys are split over several items write fp32 partials that attn_combine_kernel merges.
 #include <hip/hip_bf16.h>
+#include <hip/hip_ext.h>
 #include <hip/hip_fp16.h>
 
 #include <type_traits>
@@ -620,11 +621,13 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
     RD_REQUIRE(max_items <= 65535 && (int64_t)q_tiles * n_heads <= 2147483647LL, RD_ELIMIT,
                "rd_verify_attention: grid too large");
     {
-      rd::ScopedTiming rd_t("attn_mfma_kernel", s);
+      // when timed, the events carry the kernel's own begin and end (what a kernel trace reports)
+      hipEvent_t t0, t1;
+      rd::timing_events("attn_mfma_kernel", &t0, &t1);
       if (ksplit == 2)
-        hipLaunchKernelGGL(attn_mfma_kernel<2>, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, a);
+        hipExtLaunchKernelGGL(attn_mfma_kernel<2>, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, t0, t1, 0, a);
       else
-        hipLaunchKernelGGL(attn_mfma_kernel<1>, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, a);
+        hipExtLaunchKernelGGL(attn_mfma_kernel<1>, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, t0, t1, 0, a);
     }
     if (int e = rd::check_launch("rd_verify_attention(mfma)")) return e;
     if (a.max_splits > 1) {

@@ -209,7 +209,28 @@ def case_rope(rows, reps):
            {"rope_append_kernel": "GB/s"})
 
 
-CASES = dict(rope=case_rope, tree=case_tree, tree_x64=lambda r, n: case_tree(r, n, 64), attention=case_attention, beam=case_beam,
+def case_traffic(rows, reps):
+    """For hardware-counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): a plain copy of known size
+    (256 MiB read, 256 MiB written: the yardstick the counters are scaled by), then the verify
+    attention on the decode-bench shape (narrow tree, cached length 525) and on the ragged
+    configuration-3 shape.  Nothing is timed here."""
+    src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(reps):
+        dst.copy_(src)
+    for full_len, p_copy in ((525, 0.93), (None, 0.6)):
+        lens, n, kv, mask, q, k_, v_ = attention_case(full_len=full_len, p_copy=p_copy)
+        prep = attention.prepare(mask, n_heads=H)
+        for _ in range(reps):
+            attention.masked_attention(q, k_, v_, prep)
+        keys = int(lens.sum()) + B * n
+        rows.append(dict(case=f"traffic: attention n_q={n} sum keys={keys}", kernel="attn_mfma_kernel", launches_per_call=1,
+                         avg_us=0.0, algorithmic_work=2.0 * H * D * 2 * keys + 2.0 * B * H * n * D * 2, achieved=None,
+                         unit=None, frac_of_peak=None, note="algorithmic bytes per launch in algorithmic_work"))
+    torch.cuda.synchronize()
+
+
+CASES = dict(rope=case_rope, traffic=case_traffic, tree=case_tree, tree_x64=lambda r, n: case_tree(r, n, 64), attention=case_attention, beam=case_beam,
              logits=case_logits, kv=case_kv)
 
 
@@ -219,7 +240,7 @@ def main():
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
-    names = [n for n in args.only.split(",") if n] or list(CASES)
+    names = [n for n in args.only.split(",") if n] or [n for n in CASES if n != "traffic"]
     rows = []
     for name in names:
         CASES[name](rows, args.reps)
@@ -227,6 +248,9 @@ def main():
         print(json.dumps(rows))
         return
     for r in rows:
+        if r["unit"] is None and r["algorithmic_work"] is not None:
+            print(f"{r['case']:<72} {r['kernel']:<22} algorithmic bytes per launch {r['algorithmic_work']:.0f}")
+            continue
         rate = "" if r["achieved"] is None else f"{r['achieved']:>9.1f} {r['unit']:<8} {100 * r['frac_of_peak']:6.2f}% of peak"
         print(f"{r['case']:<72} {r['kernel']:<22} x{r['launches_per_call']:<3} {r['avg_us']:>9.2f} us  {rate}")
         if r["note"] and r["kernel"] in ("attn_mfma_kernel", "tree_mask_kernel"):

@@ -25,6 +25,7 @@ _PROTOTYPES = {
     "rd_last_error": (C.c_char_p, []),
     "rd_timing_enable": (_I, [_I]),
     "rd_timing_select": (_I, [C.c_char_p]),
+    "rd_timing_null_kernel_us": (_I, [_I, _P, C.POINTER(C.c_float)]),
     "rd_timing_collect": (_I, [C.c_char_p, _Z]),
     "rd_tree_workspace_bytes": (_Z, [_I, _I, _I]),
     "rd_tree_build": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
@@ -129,6 +130,13 @@ def timing_enable(on: bool) -> None:
 def timing_select(kernel: str | None) -> None:
     """Time only the named kernel (None: all kernels)."""
     check(lib().rd_timing_select(kernel.encode() if kernel else None))
+
+
+def timing_null_kernel_us(launches: int = 64) -> float:
+    """Event-to-event time of an empty kernel: the fixed overhead inside every timed figure."""
+    out = C.c_float(0.0)
+    check(lib().rd_timing_null_kernel_us(launches, stream(), C.byref(out)))
+    return float(out.value)
 
 
 def timing_collect() -> dict:
