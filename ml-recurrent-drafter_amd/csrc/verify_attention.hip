@@ -202,7 +202,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   auto fetch_word = [&](auto slot_c, int j) __attribute__((always_inline)) {
     const int key0 = lo + (j < n_tiles ? j : n_tiles - 1) * kTile;
     const uint64_t w = brow[key0 >> 6];
-    wring[decltype(slot_c)::value] = row_valid ? w : 0ull;
+    wring[decltype(slot_c)::value] = row_valid ? w : ~0ull;  // rows past n_q: no masking work, results unused
   };
   auto stage_k_from = [&](bf16x8 c0, bf16x8 c1, bf16x8 c2, bf16x8 c3, int j) __attribute__((always_inline)) {
     __bf16* dst = s_k[j % kKBuffers] + lrow * kKsStride + 8 * chunk;
@@ -238,7 +238,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // ---- prologue: K of tiles 0 and 1 and V of tile 0 into LDS, the ring filled behind them --------
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1 % kRing>;
-  uint64_t word = row_valid ? brow[lo >> 6] : 0ull;  // mask word of the tile whose scores are being formed
+  uint64_t word = row_valid ? brow[lo >> 6] : ~0ull;  // mask word of the tile whose scores are being formed
   // K runs one tile further ahead than V (K(t+1) is multiplied during step t); both roles keep
   // the tile that step t stages in ring slot (t + 1) % kRing, so that one piece of code, with
   // the same registers, serves both.
@@ -302,7 +302,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       // raised (and O, l rescaled) only when a unit exceeds it by more than kSlack, so most units
       // skip the 64-register rescale.  p <= 2^kSlack stays far inside bf16/fp32 range.
       constexpr float kSlack = 8.f;
-      const bool raise = tmax > m + kSlack || m == -INFINITY;
+      // (rows without a key so far have m = tmax = -inf: nothing to raise, nothing to rescale)
+      const bool raise = tmax > m + kSlack;
       if (__any(raise)) {
         const float m_new = raise ? tmax : m;
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
