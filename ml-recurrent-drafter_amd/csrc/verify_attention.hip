@@ -201,8 +201,9 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   };
   auto fetch_word = [&](auto slot_c, int j) __attribute__((always_inline)) {
     const int key0 = lo + (j < n_tiles ? j : n_tiles - 1) * kTile;
-    const uint64_t w = brow[key0 >> 6];
-    wring[decltype(slot_c)::value] = row_valid ? w : ~0ull;  // rows past n_q: no masking work, results unused
+    // nothing may touch the loaded value here: an operation on it would make the wave wait for
+    // this load, and with it for every tile load issued before it, at this point of every step
+    wring[decltype(slot_c)::value] = brow[key0 >> 6];
   };
   auto stage_k_from = [&](bf16x8 c0, bf16x8 c1, bf16x8 c2, bf16x8 c3, int j) __attribute__((always_inline)) {
     __bf16* dst = s_k[j % kKBuffers] + lrow * kKsStride + 8 * chunk;
@@ -238,7 +239,6 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // ---- prologue: K of tiles 0 and 1 and V of tile 0 into LDS, the ring filled behind them --------
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1 % kRing>;
-  uint64_t word = row_valid ? brow[lo >> 6] : ~0ull;  // mask word of the tile whose scores are being formed
   // K runs one tile further ahead than V (K(t+1) is multiplied during step t); both roles keep
   // the tile that step t stages in ring slot (t + 1) % kRing, so that one piece of code, with
   // the same registers, serves both.
@@ -252,13 +252,15 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     fetch_tile(S0{}, 0);
     stage_v(S0{}, 0);
   }
+  // The ring is filled in the order in which the steps refill it (tile, then mask word, slot by
+  // slot): the loads in flight at the top of the first step are then the same as at the top of
+  // every later one, and the compiler's count of them stays exact around the loop.  The mask word
+  // of tile j sits in wring[j % kRing] from two steps before its tile until the tile's last unit;
+  // it is never copied to another variable (a copy right after the load would be a wait for it).
   rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) {
     constexpr int J = decltype(j)::value;
     fetch_tile(std::integral_constant<int, (J + 1) % kRing>{}, ahead + J);
-  });
-  rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) {
-    constexpr int J = decltype(j)::value;
-    fetch_word(std::integral_constant<int, (1 + J) % kRing>{}, 1 + J);
+    fetch_word(std::integral_constant<int, J>{}, J);
   });
   __syncthreads();
   if (wave_active) {
@@ -285,7 +287,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     bf16x8 pf[2];  // P^T of the unit, the B operand of the second product
     if (wave_active) {
       // mask, running maximum, lazy rescale: short, not overlapped
-      const uint32_t mine = (uint32_t)(word >> key_off);
+      // rows past n_q take an all-ones word: no masking work, and their results are never used
+      const uint32_t mine = row_valid ? (uint32_t)(wring[J] >> key_off) : ~0u;
       if (!__all(mine == ~0u)) {
         const uint32_t w = mine >> (4 * g);
 #pragma unroll
@@ -375,19 +378,23 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       }
     }
     if (kLast) {
-      // mask word of tile t+1, and the word of tile t+1+kRing takes its slot
-      word = wring[(J + 1) % kRing];
-      fetch_word(std::integral_constant<int, (J + 1) % kRing>{}, t + 1 + kRing);
+      // this tile's mask word is done with: the word of tile t+kRing takes its slot
+      fetch_word(std::integral_constant<int, J>{}, t + kRing);
       __syncthreads();
     }
   };
-  for (int t0 = 0; t0 < n_tiles; t0 += kRing) {
+  // Whole rounds of the ring first, then the odd tile.  A round that could skip its second step
+  // would leave two possible sets of loads in flight at the top of the loop, and every wait in
+  // the first step would then have to be a wait for all of them.
+  int t0 = 0;
+  for (; t0 + kRing <= n_tiles; t0 += kRing) {
     rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) {
       constexpr int J = decltype(j)::value;
-      if (t0 + J < n_tiles)
-        rd_static_for<kUnits>([&](auto u) __attribute__((always_inline)) { unit_step(j, u, t0 + J); });
+      rd_static_for<kUnits>([&](auto u) __attribute__((always_inline)) { unit_step(j, u, t0 + J); });
     });
   }
+  if (t0 < n_tiles)
+    rd_static_for<kUnits>([&](auto u) __attribute__((always_inline)) { unit_step(S0{}, u, t0); });
 
   l = pair_sum(l);
   if (KSPLIT == 2) {
