@@ -105,10 +105,17 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   __bf16 (*s_k)[kTile * kKsStride] = reinterpret_cast<__bf16 (*)[kTile * kKsStride]>(smem);
   __bf16 (*s_vt)[kD * kVtStride] = reinterpret_cast<__bf16 (*)[kD * kVtStride]>(smem + kKBytes);
 
+  // The item is requested together with the item count (one trip to memory instead of two; the
+  // item array has a slot for every blockIdx.y), and every kernel argument is fetched up front:
+  // fetched where first used, they cost one more wait each on the way to the first tile load.
   const int item = blockIdx.y;
-  if (item >= a.plan[0]) return;
   const int32_t* it = a.plan + RD_PLAN_HDR + 4 * a.B + 4 * item;
-  const int b = it[0], lo = it[1], hi = it[2], split = it[3];
+  const int n_items = a.plan[0];
+  int b = it[0], lo = it[1], hi = it[2], split = it[3];
+  asm volatile("" : "+s"(b), "+s"(lo), "+s"(hi), "+s"(split));
+  asm volatile("" ::"s"(a.q), "s"(a.q_sb), "s"(a.q_sh), "s"(a.q_ss), "s"(a.k), "s"(a.k_sb), "s"(a.k_sh), "s"(a.k_ss));
+  asm volatile("" ::"s"(a.v), "s"(a.v_sb), "s"(a.v_sh), "s"(a.v_ss), "s"(a.bits), "s"(a.n_q), "s"(a.kv_len), "s"(a.words));
+  if (item >= n_items) return;
   const int n_splits = a.plan[RD_PLAN_HDR + 4 * b + 1];
   // query tiles of one (row, head, key range) are neighbours in dispatch order, so they run
   // together and the second read of the K/V tiles is served by the L2
