@@ -170,8 +170,9 @@ def gpu_run(steps: int, warmup: int):
 
 def attention_roofline(run):
     """The dominant kernel against the roof that binds it.  Per launch, from the shapes the timed
-    region actually ran: algorithmic FLOPs 4 * heads * head_dim * n_q * sum_b(keys_b), algorithmic
-    bytes K and V once (2 * heads * head_dim * 2 B per key) plus Q and O once; duration = HIP events
+    region actually ran: algorithmic FLOPs 4 * heads * head_dim * query rows * keys, algorithmic
+    bytes K and V once (2 * heads * head_dim * 2 B per key) plus Q and O once, query rows = the
+    tree slots that exist (the padding slots of the (batch, n_q) layout are not run); duration = HIP events
     around every launch in the timed region.  Arithmetic intensity below the machine balance
     (2500 TFLOP/s / 8 TB/s = 312 FLOP/B) means the HBM roof binds, above it the MFMA roof."""
     H, D = LLAMA_7B["num_attention_heads"], LLAMA_7B["hidden_size"] // LLAMA_7B["num_attention_heads"]
@@ -179,8 +180,8 @@ def attention_roofline(run):
     shapes = run["shapes"][:count] if count else []
     if not count or total_ms <= 0:
         return None
-    flops = sum(4.0 * H * D * n_q * B * kv for (B, n_q, kv) in shapes)
-    k_bytes = sum(2.0 * H * D * 2 * B * kv + 2.0 * B * H * n_q * D * 2 for (B, n_q, kv) in shapes)
+    flops = sum(4.0 * H * D * rows * kv for (B, n_q, kv, rows) in shapes)
+    k_bytes = sum(2.0 * H * D * 2 * B * kv + 2.0 * rows * H * D * 2 for (B, n_q, kv, rows) in shapes)
     seconds = total_ms * 1e-3
     tflops, gbs = flops / seconds / 1e12, k_bytes / seconds / 1e9
     hbm_bound = flops / k_bytes < MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
@@ -205,8 +206,9 @@ def attention_roofline(run):
         # HIP events span dispatch and completion signalling too; an empty kernel timed the same way
         # gives that fixed part (a kernel trace reports about avg_us minus this)
         null_kernel_event_us=round(run["null_us"], 2),
-        mean_n_q=round(sum(n for (_, n, _) in shapes) / len(shapes), 1),
-        mean_kv_len=round(sum(kv for (_, _, kv) in shapes) / len(shapes), 1),
+        mean_n_q=round(sum(n for (_, n, _, _) in shapes) / len(shapes), 1),
+        mean_query_rows=round(sum(r for (_, _, _, r) in shapes) / len(shapes), 1),
+        mean_kv_len=round(sum(kv for (_, _, kv, _) in shapes) / len(shapes), 1),
     )
     return out
 

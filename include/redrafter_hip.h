@@ -72,13 +72,17 @@ RD_API int rd_timing_collect(char* out, size_t out_bytes);
  * written as a contiguous (batch, max_n) array; slots past a row's own count hold the following
  * rows' entries, clamped to the batch's last entry, exactly as the reference's gather does.
  * prefix_tree may be NULL.
+ * row_start (int32, batch+1) and row_slots (int64, capacity batch*width*length), both optional:
+ * the slots that exist, listed row after row without the padding -- row_start[b] = number of
+ * slots of the rows before b (row_start[batch] = total), row_slots[row_start[b] + t] = b*max_n + t
+ * for t < counts[b].  (No counterpart in the reference, which runs the model on the padding too.)
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_tree_workspace_bytes(int batch, int width, int length);
 RD_API int rd_tree_build(const int64_t* beams, int batch, int width, int length,
                   int64_t* prefix_tree, int64_t* unpacker,
                   int64_t* packed_tokens, int64_t* packed_token_indices,
-                  int64_t* position_offsets, int32_t* counts,
-                  void* workspace, size_t workspace_bytes, void* stream);
+                  int64_t* position_offsets, int32_t* counts, int32_t* row_start,
+                  int64_t* row_slots, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Tree attention mask, rows of the packed tokens only.
@@ -206,6 +210,13 @@ RD_API int rd_silu_mul(const void* gate, const void* up, int64_t in_row_stride, 
  * (may be q itself).  k_cache / v_cache: (batch, n_kv_heads, max_len, head_dim) slabs with element
  * strides cache_strides = {batch, head, row}; rows [row0, row0 + n_new) are written.
  * Every product and the sum are rounded to dtype, as the separate torch kernels round them.
+ *
+ * row_start (batch + 1 int32 on the device, or NULL): packed token rows.  The reference runs the
+ * model on (batch, n_new) slots of which a row's trailing ones are padding whose results nobody
+ * reads (tree_attention.py:70-122 fills them with other rows' tokens).  With row_start, token t of
+ * batch row b is row row_start[b] + t of q, k, v and q_out (token stride; the batch strides are
+ * unused) and exists only for t < row_start[b+1] - row_start[b]; position_ids stay (batch, n_new);
+ * the cache rows of the slots that do not exist are not written.
  * ------------------------------------------------------------------------------------------ */
 RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k,
                           const int64_t* k_strides, const void* v, const int64_t* v_strides,
@@ -214,7 +225,7 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
                           const int64_t* position_ids, int64_t pos_batch_stride, void* q_out,
                           const int64_t* q_out_strides, void* k_cache, void* v_cache,
                           const int64_t* cache_strides, int64_t row0, int64_t max_len,
-                          void* stream);
+                          const int32_t* row_start, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Verification attention.
@@ -237,6 +248,10 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
  * views View.cat returns (kv_cache.py:24-31).  bf16 with head_dim 128 runs on the MFMA kernel
  * (needs 16-byte aligned q/k/v, strides that are multiples of 8 elements, and the workspace);
  * everything else, or force_generic != 0, runs on the generic kernel (head_dim <= 256).
+ * row_start (batch + 1 int32 on the device, or NULL): packed query rows, as in rd_rope_append:
+ * query t of batch row b is row row_start[b] + t of q and of out (sequence stride; their batch
+ * strides are unused), queries t >= row_start[b+1] - row_start[b] are neither read nor written.
+ * The mask bits keep their (batch, n_q) rows.
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_attn_plan_ints(int batch, int n_q, int kv_len);
 RD_API size_t rd_attn_bits_words(int batch, int n_q, int kv_len);
@@ -251,7 +266,7 @@ RD_API int rd_verify_attention(const void* q, const int64_t* q_strides, const vo
                                int n_heads, int n_kv_heads, int n_q, int kv_len, int head_dim,
                                float scale, const uint64_t* bits, const int32_t* plan,
                                void* workspace, size_t workspace_bytes, int force_generic,
-                               void* stream);
+                               const int32_t* row_start, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Causal mask from a padding mask: mask[b,i,j] = (j <= kv_len - query_len + i) && padding[b,j].

@@ -65,6 +65,10 @@ struct RopeArgs {
   void* k_cache; void* v_cache;                 // (B, kv_heads, max_len, D)
   int64_t c_sb, c_sh, c_st;
   int64_t row0;                                 // first cache row written
+  // Packed token rows (or null): token t of batch row b is row row_start[b] + t of q, k, v and
+  // q_out (their batch strides are unused) and exists only for t < row_start[b+1] - row_start[b];
+  // the cache rows of tokens that do not exist are left as they are.
+  const int32_t* row_start;
   int n_new, n_heads, n_kv_heads, head_dim;
 };
 
@@ -84,10 +88,17 @@ __global__ __launch_bounds__(kThreads) void rope_append_kernel(RopeArgs a) {
   pos = pos < 0 ? 0 : (pos >= a.table_rows ? a.table_rows - 1 : pos);  // never read outside the table
   const T* cos_row = reinterpret_cast<const T*>(a.cos) + pos * D;
   const T* sin_row = reinterpret_cast<const T*>(a.sin) + pos * D;
-  const T* q_tok = reinterpret_cast<const T*>(a.q) + b * a.q_sb + t * a.q_st;
-  const T* k_tok = reinterpret_cast<const T*>(a.k) + b * a.k_sb + t * a.k_st;
-  const T* v_tok = reinterpret_cast<const T*>(a.v) + b * a.v_sb + t * a.v_st;
-  T* qo_tok = reinterpret_cast<T*>(a.q_out) + b * a.qo_sb + t * a.qo_st;
+  int64_t tok = t, in_batch = b;  // token row within the batch row's block, and which block
+  if (a.row_start != nullptr) {
+    const int r0 = a.row_start[b];
+    if (t >= a.row_start[b + 1] - r0) return;
+    tok = (int64_t)r0 + t;
+    in_batch = 0;
+  }
+  const T* q_tok = reinterpret_cast<const T*>(a.q) + in_batch * a.q_sb + tok * a.q_st;
+  const T* k_tok = reinterpret_cast<const T*>(a.k) + in_batch * a.k_sb + tok * a.k_st;
+  const T* v_tok = reinterpret_cast<const T*>(a.v) + in_batch * a.v_sb + tok * a.v_st;
+  T* qo_tok = reinterpret_cast<T*>(a.q_out) + in_batch * a.qo_sb + tok * a.qo_st;
   T* kc = reinterpret_cast<T*>(a.k_cache) + b * a.c_sb + (a.row0 + t) * a.c_st;
   T* vc = reinterpret_cast<T*>(a.v_cache) + b * a.c_sb + (a.row0 + t) * a.c_st;
 
@@ -133,7 +144,7 @@ extern "C" int rd_rope_append(const void* q, const int64_t* q_strides, const voi
                               const int64_t* position_ids, int64_t pos_batch_stride, void* q_out,
                               const int64_t* q_out_strides, void* k_cache, void* v_cache,
                               const int64_t* cache_strides, int64_t row0, int64_t max_len,
-                              void* stream) {
+                              const int32_t* row_start, void* stream) {
   RD_REQUIRE(batch > 0 && n_new > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0, RD_EINVAL,
              "rd_rope_append: bad sizes (batch %d n_new %d heads %d kv_heads %d head_dim %d)", batch, n_new,
              n_heads, n_kv_heads, head_dim);
@@ -166,6 +177,7 @@ extern "C" int rd_rope_append(const void* q, const int64_t* q_strides, const voi
   a.k_cache = k_cache; a.v_cache = v_cache;
   a.c_sb = cache_strides[0]; a.c_sh = cache_strides[1]; a.c_st = cache_strides[2];
   a.row0 = row0;
+  a.row_start = row_start;
   a.n_new = n_new; a.n_heads = n_heads; a.n_kv_heads = n_kv_heads; a.head_dim = head_dim;
   hipStream_t s = rd::as_stream(stream);
   const dim3 grid(n_new, batch);

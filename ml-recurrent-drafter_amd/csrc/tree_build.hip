@@ -78,7 +78,8 @@ __global__ __launch_bounds__(kThreads) void tree_rows_kernel(
 __global__ __launch_bounds__(kThreads) void tree_fill_kernel(
     const int64_t* __restrict__ sel_tok, const int32_t* __restrict__ sel_idx, int B, int WL, int L,
     int32_t* __restrict__ counts, int64_t* __restrict__ packed_tokens,
-    int64_t* __restrict__ packed_token_indices, int64_t* __restrict__ position_offsets) {
+    int64_t* __restrict__ packed_token_indices, int64_t* __restrict__ position_offsets,
+    int32_t* __restrict__ row_start, int64_t* __restrict__ row_slots) {
   __shared__ int s_red[3][kThreads / 64];
   const int b = blockIdx.x;
   int before = 0, total = 0, mx = 0;
@@ -110,7 +111,12 @@ __global__ __launch_bounds__(kThreads) void tree_fill_kernel(
   if (b == 0 && threadIdx.x == 0) {
     counts[B] = mx;
     counts[B + 1] = total;
+    if (row_start != nullptr) row_start[B] = total;
   }
+  // the slots that exist, row after row without the padding: where each one sits in (B, max_n)
+  if (row_start != nullptr && threadIdx.x == 0) row_start[b] = before;
+  if (row_slots != nullptr)
+    for (int n = threadIdx.x; n < counts[b]; n += kThreads) row_slots[before + n] = (int64_t)b * mx + n;
   for (int n = threadIdx.x; n < mx; n += kThreads) {
     int g = before + n;
     g = g < total - 1 ? g : total - 1;
@@ -224,8 +230,8 @@ extern "C" size_t rd_tree_workspace_bytes(int batch, int width, int length) {
 extern "C" int rd_tree_build(const int64_t* beams, int batch, int width, int length,
                              int64_t* prefix_tree, int64_t* unpacker, int64_t* packed_tokens,
                              int64_t* packed_token_indices, int64_t* position_offsets,
-                             int32_t* counts, void* workspace, size_t workspace_bytes,
-                             void* stream) {
+                             int32_t* counts, int32_t* row_start, int64_t* row_slots,
+                             void* workspace, size_t workspace_bytes, void* stream) {
   RD_REQUIRE(batch > 0 && width > 0 && length > 0, RD_EINVAL,
              "rd_tree_build: batch/width/length must be positive (%d,%d,%d)", batch, width, length);
   RD_REQUIRE(width <= kMaxWidth && length <= kMaxLength && width * length <= kMaxTokens, RD_ELIMIT,
@@ -249,7 +255,7 @@ extern "C" int rd_tree_build(const int64_t* beams, int batch, int width, int len
   if (int e = rd::check_launch("rd_tree_build(rows)")) return e;
   { rd::ScopedTiming rd_t("tree_fill_kernel", s); hipLaunchKernelGGL(tree_fill_kernel, dim3(batch), dim3(kThreads), 0, s, sel_tok, sel_idx, batch,
                      width * length, length, counts, packed_tokens, packed_token_indices,
-                     position_offsets); }
+                     position_offsets, row_start, row_slots); }
   return rd::check_launch("rd_tree_build(fill)");
 }
 

@@ -46,11 +46,24 @@ struct AttnArgs {
   const int32_t* plan;
   float* part_o;   // [slot][n_q][D]
   float* part_ml;  // [slot][n_q][2]
+  // Packed query rows (or null): row t of batch row b is row row_start[b] + t of q and out (their
+  // batch strides are unused) and exists only for t < row_start[b + 1] - row_start[b].  The mask
+  // rows and the partials keep the padded (batch, n_q) layout.
+  const int32_t* row_start;
   int B, H, Hkv, n_q, kv_len, words, max_splits, D;
   float scale;  // softmax scale; the MFMA kernel works in log2 units (scale * log2 e)
 };
 
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Query rows of batch row b: their count and the element offsets of row 0 in q and out.
+struct RowSpan { int n; int64_t q_off, o_off; };
+__device__ inline RowSpan row_span(const AttnArgs& a, int b) {
+  if (a.row_start == nullptr) return {a.n_q, (int64_t)b * a.q_sb, (int64_t)b * a.o_sb};
+  const int r0 = a.row_start[b], r1 = a.row_start[b + 1];
+  const int n = r1 - r0;
+  return {n < a.n_q ? n : a.n_q, (int64_t)r0 * a.q_ss, (int64_t)r0 * a.o_ss};
+}
 
 // ---------------------------------------------------------------------------------------------
 // MFMA kernel
@@ -126,9 +139,11 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and the compiler knows it
   const int g = lane >> 5, r = lane & 31;
   const int row_wave = wave % kRowWaves, kp = wave / kRowWaves;  // row block and key part of this wave
+  const RowSpan rows = row_span(a, b);
+  if (q_tile * kRowsPerWG >= rows.n) return;  // (every thread of the workgroup: no barrier is skipped)
   const int q_row = q_tile * kRowsPerWG + row_wave * 32 + r;
-  const bool wave_active = q_tile * kRowsPerWG + row_wave * 32 < a.n_q;
-  const bool row_valid = q_row < a.n_q;
+  const bool wave_active = q_tile * kRowsPerWG + row_wave * 32 < rows.n;
+  const bool row_valid = q_row < rows.n;
 
   const __bf16* kbase = reinterpret_cast<const __bf16*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh;
   const __bf16* vbase = reinterpret_cast<const __bf16*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh;
@@ -136,7 +151,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // Q fragments: B operand of S^T = K Q^T; lane (r,g) holds Q[q_row][16*ks + 8*g .. +8)
   bf16x8 qf[8];
   {
-    const __bf16* qp = reinterpret_cast<const __bf16*>(a.q) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh +
+    const __bf16* qp = reinterpret_cast<const __bf16*>(a.q) + rows.q_off + (int64_t)h * a.q_sh +
                        (int64_t)(row_valid ? q_row : 0) * a.q_ss + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
@@ -439,7 +454,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // accumulator i of block db is d = 32*db + 8*(i/4) + 4*g + i%4
   if (n_splits == 1) {
     const float inv = l > 0.f ? 1.f / l : 0.f;
-    __bf16* op = reinterpret_cast<__bf16*>(a.out) + (int64_t)b * a.o_sb + (int64_t)h * a.o_sh +
+    __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh +
                  (int64_t)q_row * a.o_ss + 4 * g;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
@@ -476,7 +491,8 @@ __global__ __launch_bounds__(kD) void attn_combine_kernel(AttnArgs a) {
   if (n_splits <= 1) return;
   const int d = threadIdx.x;
   const int64_t slot0 = ((int64_t)b * a.H + h) * a.max_splits;
-  for (int q = blockIdx.z; q < a.n_q; q += kCombineSlices) {
+  const RowSpan rows = row_span(a, b);
+  for (int q = blockIdx.z; q < rows.n; q += kCombineSlices) {
     float mx = -INFINITY;
     for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, a.part_ml[((slot0 + s) * a.n_q + q) * 2]);
     float acc = 0.f, lsum = 0.f;
@@ -488,7 +504,7 @@ __global__ __launch_bounds__(kD) void attn_combine_kernel(AttnArgs a) {
         acc += w * a.part_o[((slot0 + s) * a.n_q + q) * kD + d];
       }
     }
-    __bf16* op = reinterpret_cast<__bf16*>(a.out) + (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss;
+    __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss;
     op[d] = static_cast<__bf16>(lsum > 0.f ? acc / lsum : 0.f);
   }
 }
@@ -528,7 +544,9 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
   const int q = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int hk = h / (a.H / a.Hkv);
   const int D = a.D, tid = threadIdx.x;
-  const T* qp = reinterpret_cast<const T*>(a.q) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)q * a.q_ss;
+  const RowSpan rows = row_span(a, b);
+  if (q >= rows.n) return;
+  const T* qp = reinterpret_cast<const T*>(a.q) + rows.q_off + (int64_t)h * a.q_sh + (int64_t)q * a.q_ss;
   const T* kb = reinterpret_cast<const T*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh;
   const T* vb = reinterpret_cast<const T*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh;
   if (tid < D) s_q[tid] = ld<T>(qp + tid) * a.scale;
@@ -567,7 +585,7 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
     __syncthreads();
   }
   if (tid < D) {
-    T* op = reinterpret_cast<T*>(a.out) + (int64_t)b * a.o_sb + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss;
+    T* op = reinterpret_cast<T*>(a.out) + rows.o_off + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss;
     st<T>(op + tid, l > 0.f ? acc / l : 0.f);
   }
 }
@@ -597,7 +615,7 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
                                    int dtype, int batch, int n_heads, int n_kv_heads, int n_q,
                                    int kv_len, int head_dim, float scale, const uint64_t* bits,
                                    const int32_t* plan, void* workspace, size_t workspace_bytes,
-                                   int force_generic, void* stream) {
+                                   int force_generic, const int32_t* row_start, void* stream) {
   RD_REQUIRE(batch > 0 && n_heads > 0 && n_kv_heads > 0 && n_q > 0 && kv_len > 0 && head_dim > 0,
              RD_EINVAL, "rd_verify_attention: bad sizes (batch %d heads %d kv_heads %d n_q %d kv %d D %d)",
              batch, n_heads, n_kv_heads, n_q, kv_len, head_dim);
@@ -619,6 +637,7 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
   a.words = (kv_len + 63) / 64; a.max_splits = rd::attn_max_splits(kv_len); a.D = head_dim;
   a.scale = scale;
   a.part_o = nullptr; a.part_ml = nullptr;
+  a.row_start = row_start;
   hipStream_t s = rd::as_stream(stream);
 
   if (!force_generic && mfma_eligible(a, dtype)) {

@@ -28,7 +28,7 @@ _PROTOTYPES = {
     "rd_timing_null_kernel_us": (_I, [_I, _P, C.POINTER(C.c_float)]),
     "rd_timing_collect": (_I, [C.c_char_p, _Z]),
     "rd_tree_workspace_bytes": (_Z, [_I, _I, _I]),
-    "rd_tree_build": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "rd_tree_build": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "rd_tree_mask": (_I, [_P, _P, _P, _P, _I, _L, _L, _I, _I, _I, _P, _P]),
     "rd_unpack_rows": (_I, [_P, _L, _L, _P, _L, _I, _I, _I, _P, _L, _L, _P]),
     "rd_argmax_rows": (_I, [_P, _I, _L, _L, _L, _P, _P]),
@@ -42,7 +42,7 @@ _PROTOTYPES = {
     "rd_silu_mul": (_I, [_P, _P, _L, _P, _L, _I, _L, _I, _P]),
     "rd_rope_append": (
         _I,
-        [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _L, _P],
+        [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _L, _P, _P],
     ),
     "rd_attn_plan_ints": (_Z, [_I, _I, _I]),
     "rd_attn_bits_words": (_Z, [_I, _I, _I]),
@@ -50,7 +50,7 @@ _PROTOTYPES = {
     "rd_attention_workspace_bytes": (_Z, [_I, _I, _I, _I, _I]),
     "rd_verify_attention": (
         _I,
-        [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P, _Z, _I, _P],
+        [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P, _Z, _I, _P, _P],
     ),
     "rd_causal_mask": (_I, [_P, _I, _L, _I, _L, _L, _P, _P]),
     "rd_verify_row_stats": (_I, [_P, _I, _L, _L, _I, _I, _F, _F, _P, _I, _P]),

@@ -16,6 +16,7 @@ from typing import Optional
 import torch
 
 from . import _hip
+from .packed_rows import PackedRows
 
 
 def causal_mask(padding_mask: torch.Tensor, query_len: int, device: torch.device) -> torch.Tensor:
@@ -82,7 +83,7 @@ def prepare(mask: torch.Tensor, fix_empty_rows: bool = True, n_heads: int = 32) 
     return PreparedMask(bits.view(B, n_q, -1), plan, B, n_q, kv_len)
 
 
-# When set to a list, every masked_attention call appends (batch, n_q, kv_len): measurement
+# When set to a list, every masked_attention call appends (batch, n_q, kv_len, query rows): measurement
 # harnesses pair it with the library's per-kernel event timing to price the work that was done.
 shape_log: Optional[list] = None
 
@@ -99,35 +100,49 @@ def masked_attention(
     prepared: PreparedMask,
     scale: Optional[float] = None,
     force_generic: bool = False,
+    rows: Optional[PackedRows] = None,
 ) -> torch.Tensor:
     """q (B, H, n_q, D) [any strides with D contiguous], k/v (B, Hkv, kv_len, D) strided views.
 
-    Returns (B, n_q, H*D), i.e. already in the layout o_proj consumes."""
-    B, H, n_q, D = q.shape
+    Returns (B, n_q, H*D), i.e. already in the layout o_proj consumes.  With `rows`, q is
+    (total, H, D), the query rows that exist, and the result is (total, H*D)."""
     Bk, Hkv, kv_len, Dk = k.shape
+    if rows is None:
+        B, H, n_q, D = q.shape
+    else:
+        T, H, D = q.shape
+        B, n_q = rows.batch, rows.n
+        assert T == rows.total
     assert (Bk, Dk) == (B, D) and v.shape == k.shape and q.dtype == k.dtype == v.dtype
     assert (prepared.batch, prepared.n_q, prepared.kv_len) == (B, n_q, kv_len), "mask/plan mismatch"
-    if q.stride(3) != 1:
+    if q.stride(-1) != 1:
         q = q.contiguous()
     if k.stride(3) != 1:
         k = k.contiguous()
     if v.stride(3) != 1:
         v = v.contiguous()
-    out = torch.empty((B, n_q, H, D), dtype=q.dtype, device=q.device)
-    o_view = out.permute(0, 2, 1, 3)  # (B, H, n_q, D) strides
+    if rows is None:
+        out = torch.empty((B, n_q, H, D), dtype=q.dtype, device=q.device)
+        q_strides = _strides3(q)
+        o_strides = _strides3(out.permute(0, 2, 1, 3))  # (B, H, n_q, D) strides
+    else:
+        out = torch.empty((rows.total, H, D), dtype=q.dtype, device=q.device)
+        q_strides = (C.c_int64 * 3)(0, q.stride(1), q.stride(0))
+        o_strides = (C.c_int64 * 3)(0, out.stride(1), out.stride(0))
     lib = _hip.lib()
     ws_bytes = lib.rd_attention_workspace_bytes(B, H, n_q, kv_len, D)
     if prepared.workspace is None or prepared.workspace.numel() < ws_bytes:
         prepared.workspace = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
     if shape_log is not None:
-        shape_log.append((B, n_q, kv_len))
+        shape_log.append((B, n_q, kv_len, B * n_q if rows is None else rows.total))
     _hip.check(
         lib.rd_verify_attention(
-            _hip.ptr(q), _strides3(q), _hip.ptr(k), _strides3(k), _hip.ptr(v), _strides3(v),
-            _hip.ptr(out), _strides3(o_view), _hip.dtype_code(q.dtype), B, H, Hkv, n_q, kv_len, D,
+            _hip.ptr(q), q_strides, _hip.ptr(k), _strides3(k), _hip.ptr(v), _strides3(v),
+            _hip.ptr(out), o_strides, _hip.dtype_code(q.dtype), B, H, Hkv, n_q, kv_len, D,
             float(scale if scale is not None else 1.0 / math.sqrt(D)), _hip.ptr(prepared.bits),
             _hip.ptr(prepared.plan), _hip.ptr(prepared.workspace), prepared.workspace.numel(),
-            int(force_generic), _hip.stream(),
+            int(force_generic), _hip.ptr(rows.row_start) if rows is not None else None,
+            _hip.stream(),
         )
     )
-    return out.view(B, n_q, H * D)
+    return out.view(B, n_q, H * D) if rows is None else out.view(rows.total, H * D)

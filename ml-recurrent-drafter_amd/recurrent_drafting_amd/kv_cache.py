@@ -8,11 +8,12 @@ generation; `View.cat` appends in place and hands back a strided view, `Cache.un
 from __future__ import annotations
 
 import ctypes
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 
 from . import _hip
+from .packed_rows import PackedRows
 
 
 class View:
@@ -46,22 +47,35 @@ class View:
 
 
 def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
-                position_ids: torch.Tensor, past_key_value: Tuple[View, View]):
+                position_ids: torch.Tensor, past_key_value: Tuple[View, View],
+                rows: Optional[PackedRows] = None):
     """Rotates q and k by their positions and appends the rotated k and v to the cache, one kernel.
 
     q (B, n, heads*D) and k, v (B, n, kv_heads*D) as the projections produce them (token rows may be
     strided, e.g. slices of one fused projection); cos/sin (positions, D) tables in q's dtype;
     position_ids (B, n) int64.  q is rotated in place.  Returns (q as (B, heads, n, D) view, keys,
     values) with keys/values the (B, kv_heads, length, D) views `View.cat` would return
-    (modeling_llama.py:148-159, apply_rotary_pos_emb :87-110)."""
+    (modeling_llama.py:148-159, apply_rotary_pos_emb :87-110).
+
+    With `rows`, q, k and v are (total, heads*D) / (total, kv_heads*D): only the slots that exist.
+    The cache still grows by n rows per batch row (the slots that do not exist keep what the
+    cache held), and q comes back as a (total, heads, D) view."""
     key_view, value_view = past_key_value
     cache = key_view._cache
     _, _, batch, n_kv_heads, max_length, head_dim = cache.shape
-    n_new = q.shape[1]
-    n_heads = q.shape[2] // head_dim
-    assert q.shape == (batch, n_new, n_heads * head_dim) and q.stride(2) == 1
-    assert k.shape == (batch, n_new, n_kv_heads * head_dim) and k.stride(2) == 1
-    assert v.shape == k.shape and v.stride(2) == 1
+    if rows is None:
+        n_new = q.shape[1]
+        lead = (batch, n_new)
+        strides = lambda t: (ctypes.c_int64 * 2)(t.stride(0), t.stride(1))
+    else:
+        assert rows.batch == batch
+        n_new = rows.n
+        lead = (rows.total,)
+        strides = lambda t: (ctypes.c_int64 * 2)(0, t.stride(0))
+    n_heads = q.shape[-1] // head_dim
+    assert q.shape == (*lead, n_heads * head_dim) and q.stride(-1) == 1
+    assert k.shape == (*lead, n_kv_heads * head_dim) and k.stride(-1) == 1
+    assert v.shape == k.shape and v.stride(-1) == 1
     assert q.dtype == k.dtype == v.dtype == cache.dtype == cos.dtype == sin.dtype
     assert cos.shape == sin.shape and cos.shape[1] == head_dim and cos.is_contiguous() and sin.is_contiguous()
     assert position_ids.shape == (batch, n_new) and position_ids.dtype == torch.long and position_ids.stride(1) == 1
@@ -69,21 +83,22 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
     assert value_view._cache is cache and key_view._layer == value_view._layer
     k_slab = cache[key_view._layer, 0]
     v_slab = cache[key_view._layer, 1]
-    two = ctypes.c_int64 * 2
     _hip.check(
         _hip.lib().rd_rope_append(
-            _hip.ptr(q), two(q.stride(0), q.stride(1)), _hip.ptr(k), two(k.stride(0), k.stride(1)),
-            _hip.ptr(v), two(v.stride(0), v.stride(1)), _hip.dtype_code(q.dtype), batch, n_new, n_heads,
+            _hip.ptr(q), strides(q), _hip.ptr(k), strides(k), _hip.ptr(v), strides(v),
+            _hip.dtype_code(q.dtype), batch, n_new, n_heads,
             n_kv_heads, head_dim, _hip.ptr(cos), _hip.ptr(sin), cos.shape[0], _hip.ptr(position_ids),
-            position_ids.stride(0), _hip.ptr(q), two(q.stride(0), q.stride(1)), _hip.ptr(k_slab), _hip.ptr(v_slab),
+            position_ids.stride(0), _hip.ptr(q), strides(q), _hip.ptr(k_slab), _hip.ptr(v_slab),
             (ctypes.c_int64 * 3)(k_slab.stride(0), k_slab.stride(1), k_slab.stride(2)), key_view.length,
-            max_length, _hip.stream(),
+            max_length, _hip.ptr(rows.row_start) if rows is not None else None, _hip.stream(),
         )
     )
     key_view.length += n_new
     value_view.length += n_new
-    q_heads = q.view(batch, n_new, n_heads, head_dim).transpose(1, 2) if q.is_contiguous() else \
-        q.unflatten(2, (n_heads, head_dim)).transpose(1, 2)
+    if rows is None:
+        q_heads = q.unflatten(2, (n_heads, head_dim)).transpose(1, 2)
+    else:
+        q_heads = q.unflatten(1, (n_heads, head_dim))
     return q_heads, k_slab[:, :, : key_view.length, :], v_slab[:, :, : value_view.length, :]
 
 

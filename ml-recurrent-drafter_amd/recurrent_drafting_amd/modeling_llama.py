@@ -20,6 +20,7 @@ from transformers.modeling_utils import PreTrainedModel
 from transformers.models.llama.configuration_llama import LlamaConfig
 
 from . import _hip, attention, kv_cache
+from .packed_rows import PackedRows
 
 KeyValue = Tuple[kv_cache.View, kv_cache.View]
 
@@ -171,16 +172,17 @@ class LlamaAttention(nn.Module):
         self.rotary_emb = LlamaRotaryEmbedding(dim=self.head_dim, base=_rope_theta(config))
 
     def forward(self, hidden_states: torch.Tensor, position_ids: torch.LongTensor,
-                past_key_value: KeyValue, attention_mask: attention.PreparedMask) -> torch.Tensor:
-        bsz, q_len, _ = hidden_states.size()
+                past_key_value: KeyValue, attention_mask: attention.PreparedMask,
+                rows: Optional[PackedRows] = None) -> torch.Tensor:
+        q_len = position_ids.shape[1]
         # one projection for q, k and v; the three are column slices of its output
         qkv = nn.functional.linear(hidden_states, _fused_weight(self, "_qkv", (self.q_proj, self.k_proj, self.v_proj)))
         nq, nk = self.q_proj.out_features, self.k_proj.out_features
         q, k, v = qkv[..., :nq], qkv[..., nq : nq + nk], qkv[..., nq + nk :]
         cos, sin = self.rotary_emb(v.device, v.dtype, q_len + past_key_value[0].shape[-2])
         # rotation of q (in place) and k, append of k and v to the cache: one kernel
-        q, keys, values = kv_cache.rope_append(q, k, v, cos, sin, position_ids, past_key_value)
-        out = attention.masked_attention(q, keys, values, attention_mask)  # (B, q_len, hidden)
+        q, keys, values = kv_cache.rope_append(q, k, v, cos, sin, position_ids, past_key_value, rows)
+        out = attention.masked_attention(q, keys, values, attention_mask, rows=rows)  # (B, q_len, hidden)
         return self.o_proj(out)
 
 
@@ -198,13 +200,14 @@ class LlamaDecoderLayer(nn.Module):
         hidden_states += delta
         return hidden_states
 
-    def forward_deferred(self, hidden_states, delta, position_ids, past_key_value, attention_mask):
+    def forward_deferred(self, hidden_states, delta, position_ids, past_key_value, attention_mask,
+                         rows=None):
         """The layer with its last residual update left to the caller: takes the pending update of
         the layer before (`delta`, or None) and returns (hidden_states, pending update), so that
         every "hidden_states += ..." (modeling_llama.py:196, :198) runs inside the norm that
         follows it."""
         attn = self.self_attn(self.input_layernorm(hidden_states, delta), position_ids, past_key_value,
-                              attention_mask)
+                              attention_mask, rows)
         return hidden_states, self.mlp(self.post_attention_layernorm(hidden_states, attn))
 
 
@@ -224,15 +227,21 @@ class LlamaModel(LlamaPreTrainedModel):
     def get_input_embeddings(self):
         return self.embed_tokens
 
-    def forward(self, input_ids, attention_mask, position_ids, past_key_values) -> torch.Tensor:
-        """attention_mask: (B, q, kv) bool, or an attention.PreparedMask built from one."""
+    def forward(self, input_ids, attention_mask, position_ids, past_key_values,
+                rows: Optional[PackedRows] = None) -> torch.Tensor:
+        """attention_mask: (B, q, kv) bool, or an attention.PreparedMask built from one.
+
+        With `rows`, only the (B, q) slots that exist pass through the layers and the result is
+        (rows.total, hidden); input_ids, attention_mask and position_ids keep their (B, q) shapes."""
         if not isinstance(attention_mask, attention.PreparedMask):
             attention_mask = attention.prepare(
                 attention_mask, fix_empty_rows=False, n_heads=self.config.num_attention_heads)
+        if rows is not None:
+            input_ids = rows.take(input_ids)
         hidden_states, delta = self.embed_tokens(input_ids), None
         for layer, key_value in zip(self.layers, past_key_values):
             hidden_states, delta = layer.forward_deferred(hidden_states, delta, position_ids, key_value,
-                                                          attention_mask)
+                                                          attention_mask, rows)
         return self.norm(hidden_states, delta)
 
 
@@ -251,13 +260,15 @@ class LlamaForCausalLM(LlamaPreTrainedModel):
     def get_output_embeddings(self):
         return self.lm_head
 
-    def hidden_states(self, input_ids, attention_mask, position_ids, past_key_values) -> torch.Tensor:
-        """Final-norm hidden states (B, q, hidden); rows that attend to nothing attend to
-        everything, as the reference arranges on a GPU (modeling_llama.py:264-265)."""
+    def hidden_states(self, input_ids, attention_mask, position_ids, past_key_values,
+                      rows: Optional[PackedRows] = None) -> torch.Tensor:
+        """Final-norm hidden states (B, q, hidden), or (rows.total, hidden) of the slots that
+        exist; rows that attend to nothing attend to everything, as the reference arranges on a
+        GPU (modeling_llama.py:264-265)."""
         prepared = attention.prepare(
             attention_mask, fix_empty_rows=True, n_heads=self.config.num_attention_heads)
         return self.model(input_ids=input_ids, attention_mask=prepared, position_ids=position_ids,
-                          past_key_values=past_key_values)
+                          past_key_values=past_key_values, rows=rows)
 
     def forward(self, input_ids, attention_mask, position_ids, past_key_values) -> CausalLMOutput:
         hidden = self.hidden_states(input_ids, attention_mask, position_ids, past_key_values)

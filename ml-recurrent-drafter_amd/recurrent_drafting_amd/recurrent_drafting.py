@@ -177,11 +177,14 @@ class RecurrentDrafting(torch.nn.Module):
             mask = tree_attention.build_mask(tree, input_ids != pad)
             pads = _count_left_paddings(input_ids, pad)
             position_ids = (prev - pads).unsqueeze(-1) + tree.position_offsets
+            # the slots past a row's own tree are padding (other rows' tokens, tree_attention.py:70-122)
+            # that the reference computes and never reads: the model runs on the slots that exist
+            rows = tree.rows()
             with step_record.time("base_forward"):
-                hidden = llm.hidden_states(tree.packed_beams, mask, position_ids, cache.sliced)
-                logits = llm.lm_head(hidden)  # (B, n, V) in the model's dtype
+                hidden = llm.hidden_states(tree.packed_beams, mask, position_ids, cache.sliced, rows)
+                logits = llm.lm_head(hidden)  # (total, V) in the model's dtype
         with step_record.time("accept_candidate_tokens"):
-            llm_tokens = acceptance.argmax_rows(logits)  # per packed slot
+            llm_tokens = rows.scatter(acceptance.argmax_rows(logits))  # per packed slot
             with step_record.time("choose_from_candidates"):
                 n_tokens, seq_in_beam, next_tokens, last_slot = acceptance.greedy_accept(
                     beams, llm_tokens, tree.unpacker
@@ -191,7 +194,7 @@ class RecurrentDrafting(torch.nn.Module):
                     input_ids, n_tokens, seq_in_beam, beams, cache, pad, unpacker=tree.unpacker
                 )
             with step_record.time("greedy_prepare_next_input"):
-                context = tree_attention.gather_rows(hidden, last_slot.unsqueeze(-1))[:, 0, :]
+                context = hidden.index_select(0, rows.row_of(last_slot))
         return context, input_ids, next_tokens, n_tokens
 
     # -- one speculative-sampling step on the fused path ------------------------------------------
@@ -208,7 +211,12 @@ class RecurrentDrafting(torch.nn.Module):
             pads = _count_left_paddings(input_ids, pad)
             position_ids = (prev - pads).unsqueeze(-1) + tree.position_offsets
             with step_record.time("base_forward"):
-                hidden = llm.hidden_states(tree.packed_beams, mask, position_ids, cache.sliced)
+                # the decoder layers run on the slots that exist (see _greedy_step); the hidden
+                # states go back to their slots before the head, whose rows the kernels below
+                # address as (batch row, slot)
+                rows = tree.rows()
+                hidden = rows.scatter(
+                    llm.hidden_states(tree.packed_beams, mask, position_ids, cache.sliced, rows))
                 logits = llm.lm_head(hidden)
         with step_record.time("accept_candidate_tokens"):
             # four floats per packed row stand in for the filtered, tempered log-softmax tensors
@@ -224,8 +232,8 @@ class RecurrentDrafting(torch.nn.Module):
             with step_record.time("prepare_next_input"):
                 probs = acceptance.residual_probs(log_q, log_p, seq_in_beam, n_tokens)
                 next_tokens = dist.Categorical(probs=probs).sample()
-                rows = torch.arange(B, device=beams.device)
-                last_slot = tree.unpacker[rows, seq_in_beam, n_tokens]
+                batch_rows = torch.arange(B, device=beams.device)
+                last_slot = tree.unpacker[batch_rows, seq_in_beam, n_tokens]
                 context = tree_attention.gather_rows(hidden, last_slot.unsqueeze(-1))[:, 0, :]
         return context, input_ids, next_tokens, n_tokens
 

@@ -14,6 +14,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _hip
+from .packed_rows import PackedRows
 
 
 @dataclass
@@ -27,6 +28,13 @@ class PackedTree:
     prefix_tree: torch.Tensor  # (B, W, L) int64
     counts: torch.Tensor  # (B+2,) int32 on device: per-row count, max, total
     n: int  # packed length (max over rows), host value
+    total: int  # sum of the rows' counts, host value
+    row_start: torch.Tensor  # (B+1,) int32: slots that exist in the rows before each row
+    row_slots: torch.Tensor  # (total,) int64: slot b*n+t of every slot that exists, row after row
+
+    def rows(self) -> PackedRows:
+        """The slots that exist (slot t of row b exists iff t < counts[b])."""
+        return PackedRows(self.row_start, self.row_slots, self.total, self.unpacker.shape[0], self.n)
 
 
 def _check_beams(beams: torch.Tensor) -> Tuple[int, int, int]:
@@ -41,8 +49,9 @@ def build_tree(beams: torch.Tensor) -> PackedTree:
     beams = beams.contiguous()
     dev = beams.device
     n_tok = B * W * L
-    slab = torch.empty((5, n_tok), dtype=torch.long, device=dev)
-    counts = torch.empty(B + 2, dtype=torch.int32, device=dev)
+    slab = torch.empty((6, n_tok), dtype=torch.long, device=dev)
+    counts = torch.empty(2 * B + 3, dtype=torch.int32, device=dev)  # counts (B+2), then row_start (B+1)
+    row_start = counts[B + 2 :]
     lib = _hip.lib()
     ws_bytes = lib.rd_tree_workspace_bytes(B, W, L)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
@@ -50,18 +59,22 @@ def build_tree(beams: torch.Tensor) -> PackedTree:
         lib.rd_tree_build(
             _hip.ptr(beams), B, W, L,
             _hip.ptr(slab[0]), _hip.ptr(slab[1]), _hip.ptr(slab[2]), _hip.ptr(slab[3]),
-            _hip.ptr(slab[4]), _hip.ptr(counts), _hip.ptr(ws), ws_bytes, _hip.stream(),
+            _hip.ptr(slab[4]), _hip.ptr(counts), _hip.ptr(row_start), _hip.ptr(slab[5]),
+            _hip.ptr(ws), ws_bytes, _hip.stream(),
         )
     )
-    n = int(counts[B].item())  # the one host read; shapes below depend on it
+    n, total = counts[B : B + 2].tolist()  # the one host read; shapes below depend on it
     return PackedTree(
         packed_beams=slab[2, : B * n].view(B, n),
         unpacker=slab[1].view(B, W, L),
         packed_token_indices=slab[3, : B * n].view(B, n),
         position_offsets=slab[4, : B * n].view(B, n),
         prefix_tree=slab[0].view(B, W, L),
-        counts=counts,
+        counts=counts[: B + 2],
         n=n,
+        total=total,
+        row_start=row_start,
+        row_slots=slab[5, :total],
     )
 
 
