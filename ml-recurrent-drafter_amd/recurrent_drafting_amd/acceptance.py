@@ -6,6 +6,7 @@ recurrent_drafting/recurrent_drafting.py; that module re-exports them.
 
 from __future__ import annotations
 
+from dataclasses import dataclass
 from typing import Optional, Tuple
 
 import torch
@@ -106,7 +107,26 @@ def _greedy_prepare_next_input(
     return state, next_tokens
 
 
-def realign(
+@dataclass
+class PendingRealign:
+    """The launches of `realign` are queued; the new length (one int32 at `new_len`, on the
+    device) still has to reach the host."""
+
+    ids_buf: torch.Tensor
+    plan: torch.Tensor
+    cache: kv_cache.Cache
+    batch: int
+
+    @property
+    def new_len(self) -> torch.Tensor:
+        return self.plan[:1]
+
+    def finish(self, new_len: int) -> torch.Tensor:
+        self.cache.set_length(new_len)
+        return self.ids_buf[: self.batch * new_len].view(self.batch, new_len)
+
+
+def realign_enqueue(
     input_ids: torch.Tensor,
     n_tokens_in_seq: torch.Tensor,
     seq_in_beam: torch.Tensor,
@@ -114,12 +134,11 @@ def realign(
     cache: kv_cache.Cache,
     pad_token_id: int,
     unpacker: Optional[torch.Tensor] = None,
-) -> torch.Tensor:
-    """Appends the accepted tokens to ids and cache and re-right-aligns both.
+) -> PendingRealign:
+    """Appends the accepted tokens to ids and cache and re-right-aligns both; nothing is read back.
 
     With unpacker=None the cache must already be unpacked (Cache.unpack); with the unpacker given
-    the accepted rows are taken straight from the packed slots and the unpack step is not needed.
-    One host read (the new length)."""
+    the accepted rows are taken straight from the packed slots and the unpack step is not needed."""
     assert input_ids.dtype == torch.long, f"prev_input_ids.dtype {input_ids.dtype} is not long"
     B, W, L = beams.shape
     prev = input_ids.shape[1]
@@ -141,16 +160,28 @@ def realign(
             B, W, L, pad_token_id, _hip.ptr(plan), _hip.ptr(ids_buf), _hip.stream(),
         )
     )
-    # the KV move does not depend on the host read below, so it is enqueued first
     _hip.check(
         lib.rd_kv_compact(
             _hip.ptr(cache._cache), *cache._geometry()[:4], cache._geometry()[4], prev, L,
             _hip.ptr(plan), _hip.stream(),
         )
     )
-    new_len = int(plan[0].item())
-    cache.set_length(new_len)
-    return ids_buf[: B * new_len].view(B, new_len)
+    return PendingRealign(ids_buf, plan, cache, B)
+
+
+def realign(
+    input_ids: torch.Tensor,
+    n_tokens_in_seq: torch.Tensor,
+    seq_in_beam: torch.Tensor,
+    beams: torch.Tensor,
+    cache: kv_cache.Cache,
+    pad_token_id: int,
+    unpacker: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """`realign_enqueue` and the one host read (the new length)."""
+    pending = realign_enqueue(input_ids, n_tokens_in_seq, seq_in_beam, beams, cache, pad_token_id,
+                              unpacker)
+    return pending.finish(int(pending.new_len.item()))
 
 
 def _update_kv_cache_and_input_ids(

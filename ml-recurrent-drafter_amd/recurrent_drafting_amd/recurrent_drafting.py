@@ -14,8 +14,9 @@
 
 Greedy decoding never materialises the (B, W, L, V) logits, never unpacks the KV cache into W*L
 slots and never clones it: argmax commutes with the unpack and with the top-50 filter, and the
-accepted rows are taken straight from their packed slots.  Two host reads per step (packed tree
-length, new sequence length) where the reference has more than ten.
+accepted rows are taken straight from their packed slots.  One host read per step (new sequence
+length, accepted tokens, packed tree length and slots of the coming step) where the reference has
+more than ten.
 
 The module-level helpers of the reference are re-exported with their names for code and tests that
 call them directly.
@@ -23,6 +24,7 @@ call them directly.
 
 from __future__ import annotations
 
+import contextlib
 from dataclasses import dataclass
 from typing import Generator, Optional, Tuple
 
@@ -163,17 +165,30 @@ class RecurrentDrafting(torch.nn.Module):
                     record, input_ids, max_length, beam_shape, sampling_args, special_tokens
                 )
 
-    # -- one greedy step on the fused path ------------------------------------------------------
-    def _greedy_step(self, step_record, input_ids, context, init_tokens, cache, beam_shape, pad):
-        llm = self.llm
-        with step_record.time("generate_candidates"):
-            beams, _ = self.drafter.beam_search_candidates(
-                context, init_tokens, llm.base_model.get_input_embeddings(), beam_shape,
-                return_log_probs=False,
+    # -- the fused path ---------------------------------------------------------------------------
+    # A step is split where its host reads are.  `_draft` queues the beam search and the tree
+    # build of the COMING step; `_verify_and_accept` queues mask, model forward, acceptance and
+    # re-alignment of the current one.  Between two steps the host then needs four integers (new
+    # sequence length, accepted tokens, packed tree length, tree slots) and fetches them in ONE
+    # read, after the next step's draft has been queued: the drafter's many small launches run
+    # behind the model forward instead of in front of an idle GPU.
+    def _draft(self, step_record, context, init_tokens, beam_shape, greedy) -> "_Drafted":
+        # every step times one draft, the one it queues for its successor; the very first draft
+        # (step_record None) is not timed, so that each timer key keeps one entry per step
+        timer = step_record.time("generate_candidates") if step_record is not None else contextlib.nullcontext()
+        with timer:
+            beams, log_q = self.drafter.beam_search_candidates(
+                context, init_tokens, self.llm.base_model.get_input_embeddings(), beam_shape,
+                return_log_probs=not greedy,
             )
+            return _Drafted(beams, log_q, tree_attention.build_tree_enqueue(beams))
+
+    def _verify_and_accept(self, step_record, drafted, tree, input_ids, cache, pad, sampling_args):
+        """-> (context, next_tokens, n_tokens, realignment still to be finished)."""
+        llm, beams = self.llm, drafted.beams
+        greedy = sampling_args.greedy
         with step_record.time("verify_candidates"):
             prev = input_ids.shape[1]
-            tree = tree_attention.build_tree(beams)
             mask = tree_attention.build_mask(tree, input_ids != pad)
             pads = _count_left_paddings(input_ids, pad)
             position_ids = (prev - pads).unsqueeze(-1) + tree.position_offsets
@@ -182,60 +197,44 @@ class RecurrentDrafting(torch.nn.Module):
             rows = tree.rows()
             with step_record.time("base_forward"):
                 hidden = llm.hidden_states(tree.packed_beams, mask, position_ids, cache.sliced, rows)
-                logits = llm.lm_head(hidden)  # (total, V) in the model's dtype
+                if greedy:
+                    logits = llm.lm_head(hidden)  # (total, V) in the model's dtype
+                else:
+                    # the hidden states go back to their slots before the head: the sampling
+                    # kernels address the logits as (batch row, slot)
+                    hidden = rows.scatter(hidden)
+                    logits = llm.lm_head(hidden)
         with step_record.time("accept_candidate_tokens"):
-            llm_tokens = rows.scatter(acceptance.argmax_rows(logits))  # per packed slot
-            with step_record.time("choose_from_candidates"):
-                n_tokens, seq_in_beam, next_tokens, last_slot = acceptance.greedy_accept(
-                    beams, llm_tokens, tree.unpacker
-                )
+            if greedy:
+                llm_tokens = rows.scatter(acceptance.argmax_rows(logits))  # per packed slot
+                with step_record.time("choose_from_candidates"):
+                    n_tokens, seq_in_beam, next_tokens, last_slot = acceptance.greedy_accept(
+                        beams, llm_tokens, tree.unpacker
+                    )
+            else:
+                # four floats per packed row stand in for the filtered, tempered log-softmax tensors
+                temperature = sampling_args.temperature
+                log_p = acceptance.PackedLogP(
+                    logits, acceptance.verify_row_stats(logits, temperature), tree.unpacker, temperature)
+                with step_record.time("choose_from_candidates"):
+                    B, W, L = beams.shape
+                    uniforms = torch.rand((B, W, L - 1), device=beams.device)
+                    n_tokens, seq_in_beam = acceptance.sample_accept(beams, log_p, drafted.log_q, uniforms)
             with step_record.time("update_kv_cache_and_input_ids"):
-                input_ids = acceptance.realign(
+                realignment = acceptance.realign_enqueue(
                     input_ids, n_tokens, seq_in_beam, beams, cache, pad, unpacker=tree.unpacker
                 )
-            with step_record.time("greedy_prepare_next_input"):
-                context = hidden.index_select(0, rows.row_of(last_slot))
-        return context, input_ids, next_tokens, n_tokens
-
-    # -- one speculative-sampling step on the fused path ------------------------------------------
-    def _sampling_step(self, step_record, input_ids, context, init_tokens, cache, beam_shape, pad,
-                       temperature):
-        llm = self.llm
-        with step_record.time("generate_candidates"):
-            beams, log_q = self.drafter.beam_search_candidates(
-                context, init_tokens, llm.base_model.get_input_embeddings(), beam_shape)
-        with step_record.time("verify_candidates"):
-            prev = input_ids.shape[1]
-            tree = tree_attention.build_tree(beams)
-            mask = tree_attention.build_mask(tree, input_ids != pad)
-            pads = _count_left_paddings(input_ids, pad)
-            position_ids = (prev - pads).unsqueeze(-1) + tree.position_offsets
-            with step_record.time("base_forward"):
-                # the decoder layers run on the slots that exist (see _greedy_step); the hidden
-                # states go back to their slots before the head, whose rows the kernels below
-                # address as (batch row, slot)
-                rows = tree.rows()
-                hidden = rows.scatter(
-                    llm.hidden_states(tree.packed_beams, mask, position_ids, cache.sliced, rows))
-                logits = llm.lm_head(hidden)
-        with step_record.time("accept_candidate_tokens"):
-            # four floats per packed row stand in for the filtered, tempered log-softmax tensors
-            log_p = acceptance.PackedLogP(
-                logits, acceptance.verify_row_stats(logits, temperature), tree.unpacker, temperature)
-            with step_record.time("choose_from_candidates"):
-                B, W, L = beams.shape
-                uniforms = torch.rand((B, W, L - 1), device=beams.device)
-                n_tokens, seq_in_beam = acceptance.sample_accept(beams, log_p, log_q, uniforms)
-            with step_record.time("update_kv_cache_and_input_ids"):
-                input_ids = acceptance.realign(
-                    input_ids, n_tokens, seq_in_beam, beams, cache, pad, unpacker=tree.unpacker)
-            with step_record.time("prepare_next_input"):
-                probs = acceptance.residual_probs(log_q, log_p, seq_in_beam, n_tokens)
-                next_tokens = dist.Categorical(probs=probs).sample()
-                batch_rows = torch.arange(B, device=beams.device)
-                last_slot = tree.unpacker[batch_rows, seq_in_beam, n_tokens]
-                context = tree_attention.gather_rows(hidden, last_slot.unsqueeze(-1))[:, 0, :]
-        return context, input_ids, next_tokens, n_tokens
+            if greedy:
+                with step_record.time("greedy_prepare_next_input"):
+                    context = hidden.index_select(0, rows.row_of(last_slot))
+            else:
+                with step_record.time("prepare_next_input"):
+                    probs = acceptance.residual_probs(drafted.log_q, log_p, seq_in_beam, n_tokens)
+                    next_tokens = dist.Categorical(probs=probs).sample()
+                    batch_rows = torch.arange(B, device=beams.device)
+                    last_slot = tree.unpacker[batch_rows, seq_in_beam, n_tokens]
+                    context = tree_attention.gather_rows(hidden, last_slot.unsqueeze(-1))[:, 0, :]
+        return context, next_tokens, n_tokens, realignment
 
     def _generate(self, text_generation, input_ids, max_length, beam_shape, sampling_args,
                   special_tokens) -> Generator[torch.Tensor, None, None]:
@@ -255,24 +254,27 @@ class RecurrentDrafting(torch.nn.Module):
         context, init_tokens = _comprehend_prompt(
             self.llm, input_ids, cache, sampling_args, special_tokens.pad
         )
+        drafted, tree = None, None  # what has been drafted for the coming step
         while seq_len < max_length:
             with text_generation.step() as step_record:
-                if sampling_args.greedy:
-                    context, input_ids, init_tokens, n_tokens = self._greedy_step(
-                        step_record, input_ids, context, init_tokens, cache, beam_shape,
-                        special_tokens.pad,
-                    )
-                else:
-                    context, input_ids, init_tokens, n_tokens = self._sampling_step(
-                        step_record, input_ids, context, init_tokens, cache, beam_shape,
-                        special_tokens.pad, sampling_args.temperature,
-                    )
+                if drafted is None:  # first step: nothing was drafted ahead
+                    drafted = self._draft(None, context, init_tokens, beam_shape, sampling_args.greedy)
+                    tree = drafted.tree.finish(*drafted.tree.sizes.tolist())
+                context, init_tokens, n_tokens, realignment = self._verify_and_accept(
+                    step_record, drafted, tree, input_ids, cache, special_tokens.pad, sampling_args)
+                drafted = self._draft(step_record, context, init_tokens, beam_shape, sampling_args.greedy)
+                # the one host read of the step
+                new_len, n_accepted, tree_n, tree_total = torch.cat(
+                    (realignment.new_len, n_tokens.sum(dtype=torch.int32).view(1), drafted.tree.sizes)
+                ).tolist()
+                input_ids = realignment.finish(new_len)
+                tree = drafted.tree.finish(tree_n, tree_total)
                 output_tokens = torch.cat((input_ids, init_tokens.unsqueeze(-1)), dim=-1)
                 seq_len = output_tokens.shape[1]
                 step_record.set(
                     {
                         "input_id_length": seq_len,
-                        "avg_num_accepted": torch.sum(n_tokens).item() / batch_size,
+                        "avg_num_accepted": n_accepted / batch_size,
                     }
                 )
                 yield output_tokens[:, :max_length] if seq_len > max_length else output_tokens
@@ -280,3 +282,10 @@ class RecurrentDrafting(torch.nn.Module):
                     ended = (output_tokens[:, init_seq_len:] == special_tokens.eos).any(dim=-1)
                     if bool(ended.all()):
                         break
+
+
+@dataclass
+class _Drafted:
+    beams: torch.Tensor  # (B, W, L) int64
+    log_q: Optional[torch.Tensor]  # (B, W, L-1, V) float32, sampling only
+    tree: tree_attention.PendingTree

@@ -43,15 +43,46 @@ def _check_beams(beams: torch.Tensor) -> Tuple[int, int, int]:
     return tuple(beams.shape)  # type: ignore[return-value]
 
 
-def build_tree(beams: torch.Tensor) -> PackedTree:
-    """Dedup + unpacker + pack + position offsets in two launches (tree_attention.py:331-335)."""
+@dataclass
+class PendingTree:
+    """The launches of `build_tree` are queued; the packed length and the total (two int32 at
+    `sizes`, on the device) still have to reach the host before the outputs can be shaped."""
+
+    slab: torch.Tensor  # (6, B*W*L) int64
+    counts: torch.Tensor  # (2B+3,) int32: counts (B), max, total, row_start (B+1)
+    shape: Tuple[int, int, int]
+
+    @property
+    def sizes(self) -> torch.Tensor:
+        B = self.shape[0]
+        return self.counts[B : B + 2]
+
+    def finish(self, n: int, total: int) -> PackedTree:
+        B, W, L = self.shape
+        slab, counts = self.slab, self.counts
+        return PackedTree(
+            packed_beams=slab[2, : B * n].view(B, n),
+            unpacker=slab[1].view(B, W, L),
+            packed_token_indices=slab[3, : B * n].view(B, n),
+            position_offsets=slab[4, : B * n].view(B, n),
+            prefix_tree=slab[0].view(B, W, L),
+            counts=counts[: B + 2],
+            n=n,
+            total=total,
+            row_start=counts[B + 2 :],
+            row_slots=slab[5, :total],
+        )
+
+
+def build_tree_enqueue(beams: torch.Tensor) -> PendingTree:
+    """Dedup + unpacker + pack + position offsets in two launches (tree_attention.py:331-335);
+    nothing is read back."""
     B, W, L = _check_beams(beams)
     beams = beams.contiguous()
     dev = beams.device
     n_tok = B * W * L
     slab = torch.empty((6, n_tok), dtype=torch.long, device=dev)
     counts = torch.empty(2 * B + 3, dtype=torch.int32, device=dev)  # counts (B+2), then row_start (B+1)
-    row_start = counts[B + 2 :]
     lib = _hip.lib()
     ws_bytes = lib.rd_tree_workspace_bytes(B, W, L)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
@@ -59,23 +90,18 @@ def build_tree(beams: torch.Tensor) -> PackedTree:
         lib.rd_tree_build(
             _hip.ptr(beams), B, W, L,
             _hip.ptr(slab[0]), _hip.ptr(slab[1]), _hip.ptr(slab[2]), _hip.ptr(slab[3]),
-            _hip.ptr(slab[4]), _hip.ptr(counts), _hip.ptr(row_start), _hip.ptr(slab[5]),
+            _hip.ptr(slab[4]), _hip.ptr(counts), _hip.ptr(counts[B + 2 :]), _hip.ptr(slab[5]),
             _hip.ptr(ws), ws_bytes, _hip.stream(),
         )
     )
-    n, total = counts[B : B + 2].tolist()  # the one host read; shapes below depend on it
-    return PackedTree(
-        packed_beams=slab[2, : B * n].view(B, n),
-        unpacker=slab[1].view(B, W, L),
-        packed_token_indices=slab[3, : B * n].view(B, n),
-        position_offsets=slab[4, : B * n].view(B, n),
-        prefix_tree=slab[0].view(B, W, L),
-        counts=counts[: B + 2],
-        n=n,
-        total=total,
-        row_start=row_start,
-        row_slots=slab[5, :total],
-    )
+    return PendingTree(slab, counts, (B, W, L))
+
+
+def build_tree(beams: torch.Tensor) -> PackedTree:
+    """`build_tree_enqueue` and the one host read that the output shapes depend on."""
+    pending = build_tree_enqueue(beams)
+    n, total = pending.sizes.tolist()
+    return pending.finish(n, total)
 
 
 def build_mask(tree: PackedTree, padding_mask: torch.Tensor) -> torch.Tensor:
