@@ -264,8 +264,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
-        log("bench.py: this build runs on ONE GPU (the decode step shards by batch row with no "
-            "exchange; see DESIGN.md); --gpus must be 1")
+        log("bench.py: this build runs on ONE GPU (the decode step would shard by batch row with no "
+            "exchange between the GPUs); --gpus must be 1")
         sys.exit(2)
     if not torch.cuda.is_available():
         log("bench.py: no GPU visible; the HIP path has no CPU fallback")
