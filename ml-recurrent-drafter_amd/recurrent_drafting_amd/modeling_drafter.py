@@ -81,7 +81,10 @@ def beam_topk_step(
     B, W, V = logits.shape
     assert log_p_beam.dtype == torch.float32 and log_p_beam.shape == (B, W)
     assert beams.dtype == torch.long and beams.shape[:2] == (B, W)
-    x = _hip.aligned_rows(logits.reshape(B * W, V))
+    x = logits.reshape(B * W, V)
+    if x.stride(0) < V:  # rows shown several times (an expanded view): the kernel wants real rows
+        x = x.contiguous()
+    x = _hip.aligned_rows(x)
     beams = beams.contiguous()
     log_p_beam = log_p_beam.contiguous()
     t = beams.shape[2]
@@ -106,6 +109,8 @@ def beam_topk_step(
 
 class Drafter(transformers.PreTrainedModel):
     config_class = configuration_drafter.DrafterConfig
+    # False computes the first beam-search iteration for all W (identical) beams, as upstream does
+    first_iteration_once = True
 
     def __init__(self, cfg: configuration_drafter.DrafterConfig):
         super().__init__(cfg)
@@ -158,13 +163,20 @@ class Drafter(transformers.PreTrainedModel):
         step_log_probs: List[torch.Tensor] = []
         step_parents: List[torch.Tensor] = []
 
-        for _ in range(L - 1):
-            last = embeddings(beams[..., -1])
+        for it in range(L - 1):
+            # In the first iteration every beam of a row holds the same token, state and context
+            # (modeling_drafter.py:170-189), so the W rows of logits are W copies of one row:
+            # that row is computed once per batch row and shown W times.
+            rows = 1 if it == 0 and self.first_iteration_once else W
+            last = embeddings(beams[:, :rows, -1])
             if self.config.rnn:
-                state = torch.nn.functional.silu(self.rnn_w(last) + self.rnn_u(state))
+                state = torch.nn.functional.silu(self.rnn_w(last) + self.rnn_u(state[:, :rows]))
             else:
-                state = last + state
-            logits = self.raw_logits(torch.cat([context, state], dim=-1))
+                state = last + state[:, :rows]
+            logits = self.raw_logits(torch.cat([context[:, :rows], state], dim=-1))
+            if rows != W:
+                logits = logits.expand(B, W, V)
+                state = state.expand(B, W, hidden)
             log_p_beam, _, parents, beams, logp = beam_topk_step(
                 logits, log_p_beam, beams, want_log_probs=return_log_probs
             )
