@@ -226,7 +226,7 @@ def cpu_baseline(per_seq_tokens: float):
     t = time.perf_counter()
     torch.nn.functional.linear(a, w)
     gflops = 2 * 1448 * 4096 * 4096 / (time.perf_counter() - t) / 1e9
-    layers = (2, 4) if gflops > 300 else (1, 2)
+    layers = (4, 12) if gflops > 300 else (1, 2)
     log(f"[bench] cpu baseline: {threads} threads, bf16 GEMM {gflops:.0f} GFLOP/s, sample layers {layers}")
     gen = torch.Generator().manual_seed(SEED)
     times = []
@@ -239,9 +239,13 @@ def cpu_baseline(per_seq_tokens: float):
         ctx = torch.randn(BATCH, 4096, generator=gen).bfloat16()
         tok = torch.randint(1, 32000, (BATCH,), generator=gen)
         with torch.inference_mode():
-            t = time.perf_counter()
-            P.greedy_step(llm, drafter, ids, ctx, tok, cache, WIDTH, LENGTH, 0, tie="topk")
-            times.append(time.perf_counter() - t)
+            step_times = []
+            for _ in range(2):  # the first pass pays one-time costs (allocator, kernel selection)
+                cache.set_length(PROMPT)
+                t = time.perf_counter()
+                P.greedy_step(llm, drafter, ids, ctx, tok, cache, WIDTH, LENGTH, 0, tie="topk")
+                step_times.append(time.perf_counter() - t)
+            times.append(min(step_times))
         log(f"[bench] cpu step with {n_layers} layers: {times[-1]:.2f}s")
         del llm, drafter, cache
     per_layer = (times[1] - times[0]) / (layers[1] - layers[0])
@@ -250,7 +254,7 @@ def cpu_baseline(per_seq_tokens: float):
         value=round(per_seq_tokens * BATCH / full, 3), unit="tokens/s", cores=threads, kind="port",
         sample=(f"one decode step of the same workload (batch {BATCH}, context {PROMPT}, beam {WIDTH}x{LENGTH}, bf16) "
                 f"through the torch restatement with {layers[0]} and {layers[1]} of 32 layers "
-                f"({times[0]:.2f}s, {times[1]:.2f}s), extrapolated linearly to 32 layers = {full:.2f}s/step; "
+                f"({times[0]:.2f}s, {times[1]:.2f}s; faster of two passes each), extrapolated linearly to 32 layers = {full:.2f}s/step; "
                 f"tokens per step taken from the GPU run"),
         seconds_per_step=round(full, 3),
     )
