@@ -75,7 +75,9 @@ RD_API int rd_timing_collect(char* out, size_t out_bytes);
  * row_start (int32, batch+1) and row_slots (int64, capacity batch*width*length), both optional:
  * the slots that exist, listed row after row without the padding -- row_start[b] = number of
  * slots of the rows before b (row_start[batch] = total), row_slots[row_start[b] + t] = b*max_n + t
- * for t < counts[b].  (No counterpart in the reference, which runs the model on the padding too.)
+ * for t < counts[b]; the entries from total up to the next multiple of 32 (or the capacity) are 0,
+ * so that a caller may round its row count up.  (No counterpart in the reference, which runs the
+ * model on the padding too.)
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_tree_workspace_bytes(int batch, int width, int length);
 RD_API int rd_tree_build(const int64_t* beams, int batch, int width, int length,

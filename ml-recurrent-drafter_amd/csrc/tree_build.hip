@@ -72,6 +72,8 @@ __global__ __launch_bounds__(kThreads) void tree_rows_kernel(
   if (threadIdx.x == 0) counts[b] = s_start[W - 1] + s_nown[W - 1];
 }
 
+constexpr int kRowSlotsPad = 32;  // row_slots is zero-filled up to the next multiple of this
+
 // ---------------------------------------------------------------------------------------------
 // Per batch row: slot n of row b reads entry min(offset_b + n, total-1) of the batch-wide list.
 // ---------------------------------------------------------------------------------------------
@@ -115,8 +117,16 @@ __global__ __launch_bounds__(kThreads) void tree_fill_kernel(
   }
   // the slots that exist, row after row without the padding: where each one sits in (B, max_n)
   if (row_start != nullptr && threadIdx.x == 0) row_start[b] = before;
-  if (row_slots != nullptr)
+  if (row_slots != nullptr) {
     for (int n = threadIdx.x; n < counts[b]; n += kThreads) row_slots[before + n] = (int64_t)b * mx + n;
+    // a caller may round the number of rows up to a multiple of kRowSlotsPad (slot 0 stands in)
+    if (b == 0) {
+      const int64_t cap = (int64_t)B * WL;
+      int64_t end = ((int64_t)total + kRowSlotsPad - 1) / kRowSlotsPad * kRowSlotsPad;
+      end = end < cap ? end : cap;
+      for (int64_t n = total + threadIdx.x; n < end; n += kThreads) row_slots[n] = 0;
+    }
+  }
   for (int n = threadIdx.x; n < mx; n += kThreads) {
     int g = before + n;
     g = g < total - 1 ? g : total - 1;

@@ -105,14 +105,15 @@ def masked_attention(
     """q (B, H, n_q, D) [any strides with D contiguous], k/v (B, Hkv, kv_len, D) strided views.
 
     Returns (B, n_q, H*D), i.e. already in the layout o_proj consumes.  With `rows`, q is
-    (total, H, D), the query rows that exist, and the result is (total, H*D)."""
+    (rows.rows, H, D), the query rows that exist (and the stand-in rows behind them, which are
+    neither read nor written), and the result is (rows.rows, H*D)."""
     Bk, Hkv, kv_len, Dk = k.shape
     if rows is None:
         B, H, n_q, D = q.shape
     else:
         T, H, D = q.shape
         B, n_q = rows.batch, rows.n
-        assert T == rows.total
+        assert T == rows.rows
     assert (Bk, Dk) == (B, D) and v.shape == k.shape and q.dtype == k.dtype == v.dtype
     assert (prepared.batch, prepared.n_q, prepared.kv_len) == (B, n_q, kv_len), "mask/plan mismatch"
     if q.stride(-1) != 1:
@@ -126,7 +127,7 @@ def masked_attention(
         q_strides = _strides3(q)
         o_strides = _strides3(out.permute(0, 2, 1, 3))  # (B, H, n_q, D) strides
     else:
-        out = torch.empty((rows.total, H, D), dtype=q.dtype, device=q.device)
+        out = torch.empty((rows.rows, H, D), dtype=q.dtype, device=q.device)
         q_strides = (C.c_int64 * 3)(0, q.stride(1), q.stride(0))
         o_strides = (C.c_int64 * 3)(0, out.stride(1), out.stride(0))
     lib = _hip.lib()
@@ -145,4 +146,4 @@ def masked_attention(
             _hip.stream(),
         )
     )
-    return out.view(B, n_q, H * D) if rows is None else out.view(rows.total, H * D)
+    return out.view(B, n_q, H * D) if rows is None else out.view(rows.rows, H * D)

@@ -70,7 +70,7 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
     else:
         assert rows.batch == batch
         n_new = rows.n
-        lead = (rows.total,)
+        lead = (rows.rows,)
         strides = lambda t: (ctypes.c_int64 * 2)(0, t.stride(0))
     n_heads = q.shape[-1] // head_dim
     assert q.shape == (*lead, n_heads * head_dim) and q.stride(-1) == 1

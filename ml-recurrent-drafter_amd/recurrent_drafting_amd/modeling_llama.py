@@ -232,7 +232,7 @@ class LlamaModel(LlamaPreTrainedModel):
         """attention_mask: (B, q, kv) bool, or an attention.PreparedMask built from one.
 
         With `rows`, only the (B, q) slots that exist pass through the layers and the result is
-        (rows.total, hidden); input_ids, attention_mask and position_ids keep their (B, q) shapes."""
+        (rows.rows, hidden); input_ids, attention_mask and position_ids keep their (B, q) shapes."""
         if not isinstance(attention_mask, attention.PreparedMask):
             attention_mask = attention.prepare(
                 attention_mask, fix_empty_rows=False, n_heads=self.config.num_attention_heads)
@@ -262,7 +262,7 @@ class LlamaForCausalLM(LlamaPreTrainedModel):
 
     def hidden_states(self, input_ids, attention_mask, position_ids, past_key_values,
                       rows: Optional[PackedRows] = None) -> torch.Tensor:
-        """Final-norm hidden states (B, q, hidden), or (rows.total, hidden) of the slots that
+        """Final-norm hidden states (B, q, hidden), or (rows.rows, hidden) of the slots that
         exist; rows that attend to nothing attend to everything, as the reference arranges on a
         GPU (modeling_llama.py:264-265)."""
         prepared = attention.prepare(

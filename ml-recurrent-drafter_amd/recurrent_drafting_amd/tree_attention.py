@@ -14,7 +14,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _hip
-from .packed_rows import PackedRows
+from .packed_rows import PackedRows, round_up_rows
 
 
 @dataclass
@@ -30,11 +30,12 @@ class PackedTree:
     n: int  # packed length (max over rows), host value
     total: int  # sum of the rows' counts, host value
     row_start: torch.Tensor  # (B+1,) int32: slots that exist in the rows before each row
-    row_slots: torch.Tensor  # (total,) int64: slot b*n+t of every slot that exists, row after row
+    row_slots: torch.Tensor  # (total rounded up,) int64: slot b*n+t of every slot that exists, row after row, then zeros
 
     def rows(self) -> PackedRows:
         """The slots that exist (slot t of row b exists iff t < counts[b])."""
-        return PackedRows(self.row_start, self.row_slots, self.total, self.unpacker.shape[0], self.n)
+        return PackedRows(self.row_start, self.row_slots, self.total, self.unpacker.shape[0], self.n,
+                          self.row_slots.shape[0])
 
 
 def _check_beams(beams: torch.Tensor) -> Tuple[int, int, int]:
@@ -70,7 +71,7 @@ class PendingTree:
             n=n,
             total=total,
             row_start=counts[B + 2 :],
-            row_slots=slab[5, :total],
+            row_slots=slab[5, : round_up_rows(total, B * W * L)],
         )
 
 

@@ -40,11 +40,11 @@ def test_attention_packed_equals_padded(dtype, H, D, n, counts, kv_prev, generic
     padded = attention.masked_attention(q.transpose(1, 2), k, v, prep, force_generic=generic)  # (B, n, H*D)
     q_packed = rows.take(q)  # (T, H, D)
     packed = attention.masked_attention(q_packed, k, v, prep, force_generic=generic, rows=rows)
-    assert packed.shape == (rows.total, H * D)
-    assert torch.equal(packed, rows.take(padded))
+    assert packed.shape == (rows.rows, H * D) and rows.rows % 32 == 0 and rows.rows >= rows.total
+    assert torch.equal(packed[: rows.total], rows.take(padded)[: rows.total])
     # the packed call writes nothing outside its rows: run it into a poisoned neighbourhood
     again = attention.masked_attention(q_packed, k, v, prep, force_generic=generic, rows=rows)
-    assert torch.equal(again, packed)
+    assert torch.equal(again[: rows.total], packed[: rows.total])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
@@ -77,8 +77,10 @@ def test_rope_append_packed_equals_padded(dtype):
 
     q_pad, cache_pad = run(False)   # (B, heads, n, dim)
     q_pack, cache_pack = run(True)  # (T, heads, dim)
-    assert q_pack.shape == (rows.total, heads, dim)
-    assert torch.equal(q_pack, rows.take(q_pad.transpose(1, 2)))
+    assert q_pack.shape == (rows.rows, heads, dim)
+    assert torch.equal(q_pack[: rows.total], rows.take(q_pad.transpose(1, 2))[: rows.total])
+    # the stand-in rows behind the last row that exists are not rotated
+    assert torch.equal(q_pack[rows.total :], rows.take(qkv)[rows.total :, :nq].view(-1, heads, dim))
     for b, c in enumerate(counts):
         assert torch.equal(cache_pack[:, b, :, : prev + c], cache_pad[:, b, :, : prev + c])
         assert torch.equal(cache_pack[:, b, :, prev + c :], old[:, b, :, prev + c :])  # untouched
@@ -110,10 +112,10 @@ def test_model_on_packed_rows_matches_padded():
         with torch.inference_mode():
             outs.append(llm.hidden_states(ids, mask, pos, cache.sliced, rows if packed else None))
     padded, packed = outs
-    assert packed.shape == (rows.total, 64)
+    assert packed.shape == (rows.rows, 64)
     # a slot that exists attends only to slots that exist (causal within the row), so the values
     # of the padding slots cannot reach it
-    torch.testing.assert_close(packed, rows.take(padded), rtol=2e-5, atol=2e-5)
+    torch.testing.assert_close(packed[: rows.total], rows.take(padded)[: rows.total], rtol=2e-5, atol=2e-5)
 
 
 def test_tree_build_lists_the_slots_that_exist():
@@ -126,8 +128,8 @@ def test_tree_build_lists_the_slots_that_exist():
         tree = tree_attention.build_tree(beams)
         counts = tree.counts[:B]
         assert tree.total == int(counts.sum()) and tree.n == int(counts.max())
-        want = PackedRows.from_counts(counts, tree.total, tree.n)
+        want = PackedRows.from_counts(counts, tree.total, tree.n, capacity=B * W * L)
         got = tree.rows()
         assert torch.equal(got.row_start, want.row_start) and got.row_start.dtype == torch.int32
         assert torch.equal(got.index, want.index) and got.index.dtype == torch.long
-        assert (got.total, got.batch, got.n) == (want.total, B, tree.n)
+        assert (got.total, got.batch, got.n, got.rows) == (want.total, B, tree.n, want.rows)
