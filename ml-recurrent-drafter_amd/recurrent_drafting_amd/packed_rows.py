@@ -67,6 +67,16 @@ class PackedRows:
         out.index_copy_(0, self.index[: self.total], rows[: self.total])
         return out.view(self.batch, self.n, *rows.shape[1:])
 
+    def spread(self, rows: torch.Tensor) -> torch.Tensor:
+        """(rows, ...) -> (batch, n, ...) with a copy of packed row 0 in the slots that do not
+        exist: ordinary values for code that goes on to process every slot (a constant fill would
+        hand it rows of equal numbers, the worst case of the top-k selection kernels)."""
+        assert rows.shape[0] == self.rows
+        where = torch.zeros(self.batch * self.n, dtype=torch.long, device=rows.device)
+        where.index_copy_(0, self.index[: self.total],
+                          torch.arange(self.total, dtype=torch.long, device=rows.device))
+        return rows.index_select(0, where).view(self.batch, self.n, *rows.shape[1:])
+
     def row_of(self, slot: torch.Tensor) -> torch.Tensor:
         """(batch,) slot numbers -> their packed rows."""
         return self.row_start[:-1].long() + slot

@@ -202,7 +202,7 @@ class RecurrentDrafting(torch.nn.Module):
                 else:
                     # the hidden states go back to their slots before the head: the sampling
                     # kernels address the logits as (batch row, slot)
-                    hidden = rows.scatter(hidden)
+                    hidden = rows.spread(hidden)
                     logits = llm.lm_head(hidden)
         with step_record.time("accept_candidate_tokens"):
             if greedy:

@@ -18,6 +18,9 @@ def test_index_take_scatter_roundtrip():
     for b, c in enumerate(counts.tolist()):
         assert torch.equal(back[b, :c], padded[b, :c]) and (back[b, c:] == -1).all()
     assert rows.row_of(torch.tensor([2, 0, 3, 1])).tolist() == [2, 3, 7, 9]
+    spread = rows.spread(taken)
+    for b, c in enumerate(counts.tolist()):
+        assert torch.equal(spread[b, :c], padded[b, :c]) and (spread[b, c:] == padded[0, 0]).all()
 
 
 def test_full_rows_are_the_identity():
