@@ -72,12 +72,34 @@ constexpr int kD = 128;
 constexpr int kTile = 64;                  // keys per tile
 constexpr int kWaves = 8;
 constexpr int kMfmaThreads = kWaves * 64;  // 512
-// The 8 waves split into kWaves / KSPLIT row blocks of 32 query rows and KSPLIT key parts: with
-// KSPLIT = 2 (at most 128 query rows per workgroup) waves 0-3 take the first 32 keys of every tile
-// and waves 4-7 the last 32, each with its own running maximum, sum and accumulators, merged
-// through LDS at the end -- otherwise half of the waves would have no rows and the other half would
-// serialise their MFMA and softmax phases alone on their SIMDs.
-constexpr int rows_per_wg(int ksplit) { return (kWaves / ksplit) * 32; }
+// How the 8 waves of a workgroup share its query rows (blocks of 32) and the 64 keys of a tile.
+// A wave is either FULL (it takes both 32-key units of every tile for its row block) or a HALF (it
+// takes one unit; two halves share a row block, each with its own running maximum, sum and
+// accumulators, merged through LDS at the end).  Wave w runs on SIMD w % 4, so the layouts spread
+// the units of a tile evenly over the SIMDs:
+//   kSplit  <= 128 rows  4 blocks, all halves (w, w+4)                      2 units per SIMD
+//   kMix5   <= 160 rows  blocks 0,1 full (w0,w1); 2,3,4 halves (w2+w6, w3+w7, w4+w5)   3,3,2,2
+//   kMix6   <= 192 rows  blocks 0-3 full (w0-w3); 4,5 halves (w4+w5, w6+w7)            3 each
+//   kFull   <= 256 rows  8 blocks, all full                                 4 units per SIMD
+// Without halves, a workgroup with few rows would leave waves idle and let the others serialise
+// their MFMA and softmax phases alone on their SIMDs.
+enum Layout { kSplit = 0, kMix5 = 1, kMix6 = 2, kFull = 3 };
+constexpr int rows_per_wg(int layout) { return layout == kSplit ? 128 : layout == kMix5 ? 160 : layout == kMix6 ? 192 : 256; }
+constexpr int layout_for(int n_q) { return n_q <= 128 ? kSplit : n_q <= 160 ? kMix5 : n_q <= 192 ? kMix6 : kFull; }
+struct WaveRole { int block, part, pair; };  // part: 0/1 = that half of the keys, 2 = full; pair: merge slot of a half
+__device__ inline WaveRole wave_role(int layout, int w) {
+  switch (layout) {
+    case kSplit: return {w & 3, w >> 2, w & 3};
+    case kMix5: {
+      if (w < 2) return {w, 2, 0};
+      if (w == 2 || w == 6) return {2, w == 6, 0};
+      if (w == 3 || w == 7) return {3, w == 7, 1};
+      return {4, w == 5, 2};
+    }
+    case kMix6: return w < 4 ? WaveRole{w, 2, 0} : WaveRole{4 + ((w - 4) >> 1), (w - 4) & 1, (w - 4) >> 1};
+    default: return {w, 2, 0};
+  }
+}
 constexpr int kKBuffers = 3;               // K tiles in LDS: K(t+1) is multiplied while K(t+2) is staged
 constexpr int kVBuffers = 2;               // V tiles in LDS: V(t) is multiplied while V(t+1) is staged
 constexpr int kRing = 2;                   // register stages of tiles on their way from memory
@@ -107,12 +129,10 @@ __device__ inline float pair_sum(float v) {
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-template <int KSPLIT>
+template <int LAYOUT>
 __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
-  constexpr int kRowWaves = kWaves / KSPLIT;  // row blocks per workgroup
-  constexpr int kRowsPerWG = kRowWaves * 32;
-  constexpr int kKeys = kTile / KSPLIT;       // keys of a tile that one wave handles
-  constexpr int kKeyBlocks = kKeys / 32, kKeySteps = kKeys / 16;
+  constexpr int kRowsPerWG = rows_per_wg(LAYOUT);
+  constexpr bool kHasFull = LAYOUT != kSplit, kHasHalf = LAYOUT != kFull;
   constexpr int kKBytes = kKBuffers * kTile * kKsStride * 2, kVBytes = kVBuffers * kD * kVtStride * 2;
   __shared__ __attribute__((aligned(16))) char smem[kKBytes + kVBytes];
   __bf16 (*s_k)[kTile * kKsStride] = reinterpret_cast<__bf16 (*)[kTile * kKsStride]>(smem);
@@ -138,7 +158,10 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, and the compiler knows it
   const int g = lane >> 5, r = lane & 31;
-  const int row_wave = wave % kRowWaves, kp = wave / kRowWaves;  // row block and key part of this wave
+  const WaveRole role = wave_role(LAYOUT, wave);
+  const int row_wave = role.block;                     // row block of this wave
+  const bool full = kHasFull && (!kHasHalf || role.part == 2);  // wave-uniform
+  const int kp = full ? 0 : role.part;                 // key half of a half wave
   const RowSpan rows = row_span(a, b);
   if (q_tile * kRowsPerWG >= rows.n) return;  // (every thread of the workgroup: no barrier is skipped)
   const int q_row = q_tile * kRowsPerWG + row_wave * 32 + r;
@@ -250,9 +273,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   };
 
   // S^T of one unit: 32 keys x 32 queries; accumulator i is key 8*(i/4) + 4*g + i%4 of the unit.
-  // A wave walks through kUnits units per tile: both 32-key halves (KSPLIT 1) or its own half.
-  constexpr int kUnits = kKeys / 32;
-  static_assert((kRing * kUnits) % 2 == 0, "the score registers alternate between two sets per unit");
+  // A wave walks through one or two units per tile: both 32-key halves (a full wave) or its own.
+  static_assert(kRing % 2 == 0, "the score registers alternate between two sets per unit");
   f32x16 s_reg[2];
   auto k_frag = [&](const __bf16* sk, int key_off, int ks) __attribute__((always_inline)) {
     return *reinterpret_cast<const bf16x8*>(&sk[(key_off + r) * kKsStride + 16 * ks + 8 * g]);
@@ -290,24 +312,27 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     for (int i = 0; i < 16; ++i) s_reg[0][i] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks)
-      s_reg[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(s_k[0], kp * kKeys, ks), qf[ks], s_reg[0], 0, 0, 0);
+      s_reg[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(s_k[0], kp * 32, ks), qf[ks], s_reg[0], 0, 0, 0);
   }
 
   // ---- one unit per step -----------------------------------------------------------------------
   // A step holds S of its unit in registers.  It multiplies the next unit's K by Q on the matrix
   // pipeline while the vector ALU turns S into P (two scores per MFMA, in source order), then adds
   // V^T P^T; the last step of a tile stages the tiles that later steps need in between.
-  auto unit_step = [&](auto j_c, auto u_c, int t) __attribute__((always_inline)) {
-    constexpr int J = decltype(j_c)::value;  // t % kRing
-    constexpr int U = decltype(u_c)::value;  // unit of the tile
-    constexpr int CUR = (J * kUnits + U) & 1;
-    constexpr bool kLast = U == kUnits - 1;
+  // j_c: t % kRing; cur_c: which score register set holds this unit's S; last_c: the tile's last
+  // step (staging, fetches and barrier belong to it); run: this wave has a unit in this step
+  // (wave-uniform); key_off: the unit's keys within the tile; next_t, next_off: tile and key offset
+  // of the unit whose scores this step forms for the wave's next turn.
+  auto unit_step = [&](auto j_c, auto cur_c, auto last_c, int t, bool run, int key_off, int next_t,
+                       int next_off) __attribute__((always_inline)) {
+    constexpr int J = decltype(j_c)::value;
+    constexpr int CUR = decltype(cur_c)::value;
+    constexpr bool kLast = decltype(last_c)::value;
     f32x16& s_cur = s_reg[CUR];
     f32x16& s_next = s_reg[CUR ^ 1];
-    const int key_off = kp * kKeys + 32 * U;                       // this unit's keys within the tile
-    const int next_off = kLast ? kp * kKeys : key_off + 32;
+    const bool busy = wave_active && run;
     bf16x8 pf[2];  // P^T of the unit, the B operand of the second product
-    if (wave_active) {
+    if (busy) {
       // mask, running maximum, lazy rescale: short, not overlapped
       // rows past n_q take an all-ones word: no masking work, and their results are never used
       const uint32_t mine = row_valid ? (uint32_t)(wring[J] >> key_off) : ~0u;
@@ -343,7 +368,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       const float m_use = m == -INFINITY ? 0.f : m;
       // S(next unit) = K Q^T  ||  P = exp2(S * scale - m).  After the last unit the product reads
       // a stale buffer; its result is never used.
-      const __bf16* sk = s_k[(kLast ? t + 1 : t) % kKBuffers];
+      const __bf16* sk = s_k[next_t % kKBuffers];
       float psum = 0.f;
       constexpr int kDepth = 4;  // K fragments in flight from LDS (a read takes longer than two MFMAs)
       bf16x8 ka[kDepth];
@@ -380,7 +405,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     auto v_frag = [&](int c) __attribute__((always_inline)) {
       return *reinterpret_cast<const bf16x8*>(&sv[(32 * (c >> 1) + r) * kVtStride + 16 * (c & 1)]);
     };
-    if (wave_active) {
+    if (busy) {
 #pragma unroll
       for (int c = 0; c < kVDepth; ++c) va[c] = v_frag(c);
     }
@@ -390,7 +415,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       if (k_loader) stage_k(Slot{}, t + 2); else stage_v(Slot{}, t + 1);
       fetch_tile(Slot{}, t + ahead + kRing);
     }
-    if (wave_active) {
+    if (busy) {
       // O^T += V^T P^T ; k-slot j of lane group g is key 16*tt + 4*g + (j%4) + 8*(j/4) of the unit,
       // stored at columns 16*tt + 8*g + j of the V^T row
 #pragma unroll
@@ -408,35 +433,58 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // Whole rounds of the ring first, then the odd tile.  A round that could skip its second step
   // would leave two possible sets of loads in flight at the top of the loop, and every wait in
   // the first step would then have to be a wait for all of them.
+  // One tile.  A full wave takes both units of the tile, in score sets 0 and 1.  A half wave takes
+  // its unit (keys kp*32..) and alternates between the score sets from tile to tile, which is one
+  // unit per tile of the two-tile ring round: its turn is the first step of even tiles and the
+  // second step of odd ones.  In a layout that has both kinds, both run the same two steps per
+  // tile, a half wave idling through the step that is not its turn (wave-uniform branches): two
+  // separate loops in one kernel keep the registers of both alive and spill.
+  using Yes = std::true_type;
+  using No = std::false_type;
+  using One = std::integral_constant<int, 1>;
+  auto tile_step = [&](auto j, int t) __attribute__((always_inline)) {
+    constexpr int J = decltype(j)::value;
+    if constexpr (kHasFull && kHasHalf) {
+      const int off = kp * 32;  // kp is 0 for a full wave
+      unit_step(j, S0{}, No{}, t, full || J == 0, off, full ? t : t + 1, full ? 32 : off);
+      unit_step(j, One{}, Yes{}, t, full || J == 1, full ? 32 : off, t + 1, full ? 0 : off);
+    } else if constexpr (kHasFull) {
+      unit_step(j, S0{}, No{}, t, true, 0, t, 32);
+      unit_step(j, One{}, Yes{}, t, true, 32, t + 1, 0);
+    } else {
+      unit_step(j, std::integral_constant<int, J & 1>{}, Yes{}, t, true, kp * 32, t + 1, kp * 32);
+    }
+  };
+  // Whole rounds of the ring first, then the odd tile.  A round that could skip its second step
+  // would leave two possible sets of loads in flight at the top of the loop, and every wait in
+  // the first step would then have to be a wait for all of them.
   int t0 = 0;
   for (; t0 + kRing <= n_tiles; t0 += kRing) {
-    rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) {
-      constexpr int J = decltype(j)::value;
-      rd_static_for<kUnits>([&](auto u) __attribute__((always_inline)) { unit_step(j, u, t0 + J); });
-    });
+    rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) { tile_step(j, t0 + decltype(j)::value); });
   }
-  if (t0 < n_tiles)
-    rd_static_for<kUnits>([&](auto u) __attribute__((always_inline)) { unit_step(S0{}, u, t0); });
+  if (t0 < n_tiles) tile_step(S0{}, t0);
 
   l = pair_sum(l);
-  if (KSPLIT == 2) {
+  if (kHasHalf) {
     // merge the two key parts of every row block: part 1 hands (m, l, o) over through LDS (the tile
     // buffers are free: every wave has passed the loop's last barrier)
-    float* x_o = reinterpret_cast<float*>(smem);             // [row block][64 accumulators][lane]
-    float* x_ml = x_o + kRowWaves * 64 * 64;                 // [row block][2][lane]
+    float* x_o = reinterpret_cast<float*>(smem);             // [pair][64 accumulators][lane]
+    float* x_ml = x_o + (kWaves / 2) * 64 * 64;              // [pair][2][lane]
     static_assert((kWaves / 2) * (64 * 64 + 2 * 64) * 4 <= kKBytes + kVBytes, "merge buffer");
-    if (kp == 1 && wave_active) {
+    const int pair = role.pair;
+    const bool second = !full && kp == 1;
+    if (second && wave_active) {
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) x_o[(row_wave * 64 + 16 * db + i) * 64 + lane] = o[db][i];
-      x_ml[(row_wave * 2 + 0) * 64 + lane] = m;
-      x_ml[(row_wave * 2 + 1) * 64 + lane] = l;
+        for (int i = 0; i < 16; ++i) x_o[(pair * 64 + 16 * db + i) * 64 + lane] = o[db][i];
+      x_ml[(pair * 2 + 0) * 64 + lane] = m;
+      x_ml[(pair * 2 + 1) * 64 + lane] = l;
     }
     __syncthreads();
-    if (kp == 1) return;
-    if (wave_active) {
-      const float m2 = x_ml[(row_wave * 2 + 0) * 64 + lane], l2 = x_ml[(row_wave * 2 + 1) * 64 + lane];
+    if (second) return;
+    if (wave_active && !full) {
+      const float m2 = x_ml[(pair * 2 + 0) * 64 + lane], l2 = x_ml[(pair * 2 + 1) * 64 + lane];
       const float m_new = fmaxf(m, m2);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       const float a1 = fast_exp2(m - m_safe), a2 = fast_exp2(m2 - m_safe);  // exp2(-inf) = 0
@@ -445,7 +493,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-          o[db][i] = a1 * o[db][i] + a2 * x_o[(row_wave * 64 + 16 * db + i) * 64 + lane];
+          o[db][i] = a1 * o[db][i] + a2 * x_o[(pair * 64 + 16 * db + i) * 64 + lane];
       m = m_new;
     }
   }
@@ -650,18 +698,21 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
     a.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
                                          rd::align_up(slots * n_q * head_dim * sizeof(float), 256));
     const int max_items = batch * a.max_splits;
-    const int ksplit = n_q <= rows_per_wg(2) ? 2 : 1;
-    const int q_tiles = (n_q + rows_per_wg(ksplit) - 1) / rows_per_wg(ksplit);
+    const int layout = layout_for(n_q);
+    const int q_tiles = (n_q + rows_per_wg(layout) - 1) / rows_per_wg(layout);
     RD_REQUIRE(max_items <= 65535 && (int64_t)q_tiles * n_heads <= 2147483647LL, RD_ELIMIT,
                "rd_verify_attention: grid too large");
     {
       // when timed, the events carry the kernel's own begin and end (what a kernel trace reports)
       hipEvent_t t0, t1;
       rd::timing_events("attn_mfma_kernel", &t0, &t1);
-      if (ksplit == 2)
-        hipExtLaunchKernelGGL(attn_mfma_kernel<2>, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, t0, t1, 0, a);
-      else
-        hipExtLaunchKernelGGL(attn_mfma_kernel<1>, dim3(n_heads * q_tiles, max_items), dim3(kMfmaThreads), 0, s, t0, t1, 0, a);
+      const dim3 grid(n_heads * q_tiles, max_items), block(kMfmaThreads);
+      switch (layout) {
+        case kSplit: hipExtLaunchKernelGGL(attn_mfma_kernel<kSplit>, grid, block, 0, s, t0, t1, 0, a); break;
+        case kMix5: hipExtLaunchKernelGGL(attn_mfma_kernel<kMix5>, grid, block, 0, s, t0, t1, 0, a); break;
+        case kMix6: hipExtLaunchKernelGGL(attn_mfma_kernel<kMix6>, grid, block, 0, s, t0, t1, 0, a); break;
+        default: hipExtLaunchKernelGGL(attn_mfma_kernel<kFull>, grid, block, 0, s, t0, t1, 0, a); break;
+      }
     }
     if (int e = rd::check_launch("rd_verify_attention(mfma)")) return e;
     if (a.max_splits > 1) {

@@ -161,6 +161,23 @@ def test_mfma_kernel(B, H, Hkv, W, L, prev_lens):
     _assert_close(got2, ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("nq", [127, 128, 129, 150, 160, 161, 192, 193, 256, 257])
+def test_mfma_kernel_every_wave_layout(nq):
+    """Query counts on both sides of every boundary between the ways the waves of a workgroup share
+    rows and keys (128, 160, 192, 256 rows per workgroup), odd and even numbers of key tiles."""
+    rng = np.random.default_rng(nq)
+    B, H = 2, 2
+    for kv_prev in (70, 200):
+        kv = kv_prev + nq
+        mask = rng.random((B, nq, kv)) > 0.35
+        mask[:, :, kv_prev:] &= np.tril(np.ones((nq, nq), dtype=bool))  # causal over the new tokens
+        mask[0, :, : kv_prev // 2] = False  # row 0 starts later: its first tiles are skipped
+        mask[1, nq // 2, :] = False  # a query with no key at all
+        q = rng.standard_normal((B, H, nq, 128)); k = rng.standard_normal((B, H, kv, 128)); v = rng.standard_normal((B, H, kv, 128))
+        got, ref = _run(q, k, v, mask, torch.bfloat16, force_generic=False, cache_like=True)
+        _assert_close(got, ref, torch.bfloat16)
+
+
 def test_mfma_kernel_pad_tokens_inside_the_prefix_and_empty_rows():
     """Keys masked by VALUE in the middle of the prefix, and a query row with no key at all."""
     rng = np.random.default_rng(11)

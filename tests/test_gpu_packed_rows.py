@@ -19,6 +19,8 @@ def _rows(counts, n):
 @pytest.mark.parametrize("dtype,H,D,n,counts,kv_prev,generic", [
     (torch.bfloat16, 4, 128, 100, [100, 37, 64, 1], 300, False),     # two waves per row block
     (torch.bfloat16, 2, 128, 200, [130, 200, 33], 500, False),       # one wave per row block
+    (torch.bfloat16, 2, 128, 150, [150, 20, 97], 260, False),        # two full row blocks, three split ones
+    (torch.bfloat16, 2, 128, 180, [64, 180, 161], 333, False),       # four full row blocks, two split ones
     (torch.bfloat16, 1, 128, 300, [290, 10], 700, False),            # two query tiles; a tile with no rows
     (torch.bfloat16, 2, 128, 90, [90, 45], 2400, False),             # long rows: keys split over work items
     (torch.float32, 3, 64, 20, [20, 7, 1], 50, True),
