@@ -249,7 +249,9 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
  * {batch, head, sequence}; the last dimension is contiguous.  k and v are normally the strided
  * views View.cat returns (kv_cache.py:24-31).  bf16 with head_dim 128 runs on the MFMA kernel
  * (needs 16-byte aligned q/k/v, strides that are multiples of 8 elements, and the workspace);
- * everything else, or force_generic != 0, runs on the generic kernel (head_dim <= 256).
+ * everything else (more than 128 heads included), or force_generic != 0, runs on the generic
+ * kernel (head_dim <= 256).  The plan's arrival counters (its tail) are counted up and left at
+ * zero by every call; calls that share a plan must not overlap in time.
  * row_start (batch + 1 int32 on the device, or NULL): packed query rows, as in rd_rope_append:
  * query t of batch row b is row row_start[b] + t of q and of out (sequence stride; their batch
  * strides are unused), queries t >= row_start[b+1] - row_start[b] are neither read nor written.

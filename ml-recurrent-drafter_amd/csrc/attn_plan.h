@@ -5,6 +5,8 @@
 //   per batch row b, 4 ints at RD_PLAN_HDR + 4*b:  {kv_begin, n_splits, first_item, 0}
 //   items, 4 ints each at RD_PLAN_HDR + 4*batch:   {b, kv_lo, kv_hi, split}  (longest first)
 //   scratch: first attended key of every (b, q) row
+//   arrival counters, one per (b, head, query tile), zero between launches: the work items of a
+//   split row count themselves in, and the last one to arrive merges the partials of all
 #pragma once
 
 #include "rd_common.h"
@@ -16,6 +18,16 @@ namespace rd {
 constexpr int kAttnChunk = 512;       // target keys per work item
 constexpr int kAttnSortLimit = 2048;  // more items than this are dispatched unsorted
 
+constexpr int kAttnMaxHeads = 128;    // heads the arrival counters are laid out for
+constexpr int kAttnRowsPerTile = 256; // query rows of the largest workgroup layout
+
 inline int attn_max_splits(int kv_len) { return (kv_len + kAttnChunk - 1) / kAttnChunk; }
+inline int attn_max_q_tiles(int n_q) { return (n_q + kAttnRowsPerTile - 1) / kAttnRowsPerTile; }
+inline size_t attn_counter_offset(int batch, int n_q, int kv_len) {
+  return RD_PLAN_HDR + 4 * (size_t)batch + 4 * (size_t)batch * attn_max_splits(kv_len) + (size_t)batch * n_q;
+}
+inline size_t attn_counter_ints(int batch, int n_q) {
+  return (size_t)batch * kAttnMaxHeads * attn_max_q_tiles(n_q);
+}
 
 }  // namespace rd

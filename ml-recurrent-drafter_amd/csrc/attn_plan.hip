@@ -49,9 +49,12 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
                                                              int B, int n_q, int kv_len, int words,
                                                              int min_chunk, int max_splits,
                                                              int n_heads, int n_cu,
-                                                             int32_t* __restrict__ plan) {
+                                                             int32_t* __restrict__ plan,
+                                                             int32_t* __restrict__ counters,
+                                                             int n_counters) {
   __shared__ int s_n_items;
   __shared__ int s_chunk;
+  for (int i = threadIdx.x; i < n_counters; i += kThreads) counters[i] = 0;
   int32_t* per_row = plan + RD_PLAN_HDR;
   int32_t* items = plan + RD_PLAN_HDR + 4 * B;
   // pass 1: per batch row, first attended key and number of splits
@@ -143,7 +146,8 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
 extern "C" size_t rd_attn_plan_ints(int batch, int n_q, int kv_len) {
   if (batch <= 0 || n_q <= 0 || kv_len <= 0) return 0;
   const int max_splits = rd::attn_max_splits(kv_len);
-  return RD_PLAN_HDR + 4 * (size_t)batch + 4 * (size_t)batch * max_splits + (size_t)batch * n_q;
+  (void)max_splits;
+  return rd::attn_counter_offset(batch, n_q, kv_len) + rd::attn_counter_ints(batch, n_q);
 }
 
 extern "C" size_t rd_attn_bits_words(int batch, int n_q, int kv_len) {
@@ -184,6 +188,7 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
                      mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first); }
   if (int e = rd::check_launch("rd_attn_prepare(bits)")) return e;
   { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 0, s, row_first, batch, n_q, kv_len,
-                     words, rd::kAttnChunk, max_splits, n_heads, compute_units(), plan); }
+                     words, rd::kAttnChunk, max_splits, n_heads, compute_units(), plan,
+                     plan + rd::attn_counter_offset(batch, n_q, kv_len), (int)rd::attn_counter_ints(batch, n_q)); }
   return rd::check_launch("rd_attn_prepare(plan)");
 }

@@ -21,7 +21,8 @@
 //   attn_generic_kernel   any dtype, head_dim <= 256, one workgroup per (row, head, query); the
 //                         correctness path for shapes the MFMA kernel does not cover.
 // Work items come from the plan (attn_plan.h): (batch row, key range) chunks, longest first; rows
-// whose keys are split over several items write fp32 partials that attn_combine_kernel merges.
+// whose keys are split over several items write fp32 partials, and the item that finishes last
+// merges them (an arrival counter per (row, head, query tile) in the plan).
 #include <hip/hip_bf16.h>
 #include <hip/hip_ext.h>
 #include <hip/hip_fp16.h>
@@ -50,6 +51,7 @@ struct AttnArgs {
   // batch strides are unused) and exists only for t < row_start[b + 1] - row_start[b].  The mask
   // rows and the partials keep the padded (batch, n_q) layout.
   const int32_t* row_start;
+  int32_t* counters;  // arrival counters of the plan: [batch][kAttnMaxHeads][query tiles], zero between launches
   int B, H, Hkv, n_q, kv_len, words, max_splits, D;
   float scale;  // softmax scale; the MFMA kernel works in log2 units (scale * log2 e)
 };
@@ -482,8 +484,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       x_ml[(pair * 2 + 1) * 64 + lane] = l;
     }
     __syncthreads();
-    if (second) return;
-    if (wave_active && !full) {
+    if (wave_active && !full && !second) {
       const float m2 = x_ml[(pair * 2 + 0) * 64 + lane], l2 = x_ml[(pair * 2 + 1) * 64 + lane];
       const float m_new = fmaxf(m, m2);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
@@ -497,10 +498,11 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       m = m_new;
     }
   }
-  if (!wave_active) return;
-  if (!row_valid) return;
+  const bool second_half = kHasHalf && !full && kp == 1;  // has handed its part to its partner
+  const bool writer = wave_active && row_valid && !second_half;
   // accumulator i of block db is d = 32*db + 8*(i/4) + 4*g + i%4
   if (n_splits == 1) {
+    if (!writer) return;
     const float inv = l > 0.f ? 1.f / l : 0.f;
     __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh +
                  (int64_t)q_row * a.o_ss + 4 * g;
@@ -512,9 +514,15 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
                     static_cast<__bf16>(o[db][4 * i4 + 2] * inv), static_cast<__bf16>(o[db][4 * i4 + 3] * inv)};
         *reinterpret_cast<bf16x4*>(op + 32 * db + 8 * i4) = w;
       }
-  } else {
-    const int64_t slot = ((int64_t)b * a.H + h) * a.max_splits + split;
-    float* po = a.part_o + (slot * a.n_q + q_row) * kD + 4 * g;
+    return;
+  }
+  // The keys of this batch row are split over n_splits work items: each leaves (m, l, O) of its
+  // key range as fp32 partials, counts itself in, and the last one to arrive merges the partials
+  // of all of them (m in log2 units).  Nobody returns before the count: the barriers below are
+  // reached by every wave of the workgroup.
+  const int64_t slot0 = ((int64_t)b * a.H + h) * a.max_splits;
+  if (writer) {
+    float* po = a.part_o + ((slot0 + split) * a.n_q + q_row) * kD + 4 * g;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -523,38 +531,74 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
         *reinterpret_cast<f32x4*>(po + 32 * db + 8 * i4) = w;
       }
     if (g == 0) {
-      float* pm = a.part_ml + (slot * a.n_q + q_row) * 2;
+      float* pm = a.part_ml + ((slot0 + split) * a.n_q + q_row) * 2;
       pm[0] = m;
       pm[1] = l;
     }
   }
-}
-
-// Merges the partials of rows whose keys were split (m in log2 units).  One workgroup per
-// (head, batch row, query slice); rows that were not split cost one early exit per workgroup.
-constexpr int kCombineSlices = 32;
-__global__ __launch_bounds__(kD) void attn_combine_kernel(AttnArgs a) {
-  const int h = blockIdx.x, b = blockIdx.y;
-  const int n_splits = a.plan[RD_PLAN_HDR + 4 * b + 1];
-  if (n_splits <= 1) return;
-  const int d = threadIdx.x;
-  const int64_t slot0 = ((int64_t)b * a.H + h) * a.max_splits;
-  const RowSpan rows = row_span(a, b);
-  for (int q = blockIdx.z; q < rows.n; q += kCombineSlices) {
-    float mx = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, a.part_ml[((slot0 + s) * a.n_q + q) * 2]);
-    float acc = 0.f, lsum = 0.f;
-    if (mx > -INFINITY) {
-      for (int s = 0; s < n_splits; ++s) {
-        const float* pm = a.part_ml + ((slot0 + s) * a.n_q + q) * 2;
-        const float w = fast_exp2(pm[0] - mx);
-        lsum += w * pm[1];
-        acc += w * a.part_o[((slot0 + s) * a.n_q + q) * kD + d];
+  // The barrier waits until the partial stores of every wave have left the compute unit; one
+  // wave then does the device-wide part for the whole workgroup: it makes the partials visible
+  // before the item is counted and, if the item is the last, drops stale lines before the others'
+  // partials are read.  (The fences work on the whole L2 of this XCD, so one per workgroup it is,
+  // not one per wave.)
+  __syncthreads();
+  int* s_last = reinterpret_cast<int*>(smem);  // (the tile buffers are free by now)
+  int32_t* counter = a.counters + ((int64_t)b * rd::kAttnMaxHeads + h) * q_tiles + q_tile;
+  if (wave == 0) {
+    __threadfence();
+    int last = 0;
+    if (lane == 0) last = atomicAdd(counter, 1) == n_splits - 1;
+    last = __builtin_amdgcn_readfirstlane(last);
+    if (last) __threadfence();
+    if (lane == 0) *s_last = last;
+  }
+  __syncthreads();
+  if (*s_last == 0) return;
+  // 16 row groups x 32 lanes of four dims; eight rows per pass and thread, so that the loads of
+  // a pass (two per row and split) are in flight together: the merge is bound by their latency
+  const int q_end = (q_tile + 1) * kRowsPerWG < rows.n ? (q_tile + 1) * kRowsPerWG : rows.n;
+  constexpr int kGroups = kMfmaThreads / 32, kPass = 8;
+  const int rg = tid >> 5, dq = (tid & 31) * 4;
+  for (int q0 = q_tile * kRowsPerWG + rg; q0 < q_end; q0 += kGroups * kPass) {
+    float mx[kPass], ls[kPass];
+    f32x4 acc[kPass];
+#pragma unroll
+    for (int j = 0; j < kPass; ++j) {
+      mx[j] = -INFINITY; ls[j] = 0.f; acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int s = 0; s < n_splits; ++s) {
+      f32x2 ml[kPass];
+      f32x4 po[kPass];
+#pragma unroll
+      for (int j = 0; j < kPass; ++j) {
+        const int q = q0 + kGroups * j < q_end ? q0 + kGroups * j : q_end - 1;  // clamped: loads stay unconditional
+        const int64_t row = (slot0 + s) * a.n_q + q;
+        ml[j] = *reinterpret_cast<const f32x2*>(a.part_ml + row * 2);
+        po[j] = *reinterpret_cast<const f32x4*>(a.part_o + row * kD + dq);
+      }
+#pragma unroll
+      for (int j = 0; j < kPass; ++j) {
+        const float m_new = fmaxf(mx[j], ml[j][0]);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float a1 = fast_exp2(mx[j] - m_safe), a2 = fast_exp2(ml[j][0] - m_safe);  // exp2(-inf) = 0
+        ls[j] = a1 * ls[j] + a2 * ml[j][1];
+        acc[j] = a1 * acc[j] + a2 * po[j];
+        mx[j] = m_new;
       }
     }
-    __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss;
-    op[d] = static_cast<__bf16>(lsum > 0.f ? acc / lsum : 0.f);
+#pragma unroll
+    for (int j = 0; j < kPass; ++j) {
+      const int q = q0 + kGroups * j;
+      if (q < q_end) {
+        const float inv = ls[j] > 0.f ? 1.f / ls[j] : 0.f;
+        __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss + dq;
+        bf16x4 w = {static_cast<__bf16>(acc[j][0] * inv), static_cast<__bf16>(acc[j][1] * inv),
+                    static_cast<__bf16>(acc[j][2] * inv), static_cast<__bf16>(acc[j][3] * inv)};
+        *reinterpret_cast<bf16x4*>(op) = w;
+      }
+    }
   }
+  if (tid == 0) *counter = 0;  // ready for the next launch on this plan
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -641,7 +685,7 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
 bool mfma_eligible(const AttnArgs& a, int dtype) {
   auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
   auto m8 = [](int64_t s) { return (s % 8) == 0; };
-  return dtype == RD_BF16 && a.D == kD && al(a.q) && al(a.k) && al(a.v) && ((uintptr_t)a.out & 7) == 0 &&
+  return dtype == RD_BF16 && a.D == kD && a.H <= rd::kAttnMaxHeads && al(a.q) && al(a.k) && al(a.v) && ((uintptr_t)a.out & 7) == 0 &&
          m8(a.q_sb) && m8(a.q_sh) && m8(a.q_ss) && m8(a.k_sb) && m8(a.k_sh) && m8(a.k_ss) &&
          m8(a.v_sb) && m8(a.v_sh) && m8(a.v_ss) && (a.o_sb % 4) == 0 && (a.o_sh % 4) == 0 &&
          (a.o_ss % 4) == 0;
@@ -686,6 +730,7 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
   a.scale = scale;
   a.part_o = nullptr; a.part_ml = nullptr;
   a.row_start = row_start;
+  a.counters = const_cast<int32_t*>(plan) + rd::attn_counter_offset(batch, n_q, kv_len);
   hipStream_t s = rd::as_stream(stream);
 
   if (!force_generic && mfma_eligible(a, dtype)) {
@@ -714,12 +759,7 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
         default: hipExtLaunchKernelGGL(attn_mfma_kernel<kFull>, grid, block, 0, s, t0, t1, 0, a); break;
       }
     }
-    if (int e = rd::check_launch("rd_verify_attention(mfma)")) return e;
-    if (a.max_splits > 1) {
-      { rd::ScopedTiming rd_t("attn_combine_kernel", s); hipLaunchKernelGGL(attn_combine_kernel, dim3(n_heads, batch, kCombineSlices), dim3(kD), 0, s, a); }
-      return rd::check_launch("rd_verify_attention(combine)");
-    }
-    return RD_OK;
+    return rd::check_launch("rd_verify_attention(mfma)");
   }
   const dim3 grid(n_q, n_heads, batch);
   switch (dtype) {
