@@ -119,11 +119,10 @@ def case_attention(rows, reps):
         keys = int(lens.sum()) + B * n
         flops = 4.0 * H * D * n * keys
         byts = 2.0 * H * D * 2 * keys + 2.0 * B * H * n * D * 2
-        both = dict(kt)
         total_us = sum(us * c for c, us in kt.values())
         report(rows, f"verify_attention {label} (n_q={n}, sum keys={keys})", kt,
                {"attn_mfma_kernel": flops}, {"attn_mfma_kernel": "TFLOP/s"},
-               note=f"{flops / 1e9:.1f} GFLOP, {byts / 1e6:.0f} MB algorithmic; mfma+combine {total_us:.1f} us = "
+               note=f"{flops / 1e9:.1f} GFLOP, {byts / 1e6:.0f} MB algorithmic; {total_us:.1f} us = "
                     f"{flops / total_us / 1e6:.0f} TFLOP/s, {byts / total_us / 1e3:.0f} GB/s "
                     f"({byts / total_us / 1e3 / HBM:.3f} of HBM peak)")
         report(rows, f"attn_prepare {label}", kp, {"mask_bits_kernel": B * n * kv + B * n * ((kv + 63) // 64) * 8},
