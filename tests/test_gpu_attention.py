@@ -51,7 +51,7 @@ def test_mask_bits_and_plan():
     mask[1, 3, :] = False  # an empty row gets all keys
     mask[2, :, :64] = False
     mask[2, 5, 70] = True
-    prep = attention.prepare(_dev(mask, torch.bool), n_heads=4096)  # many heads: minimum-size items
+    prep = attention.prepare(_dev(mask, torch.bool), n_heads=1)  # one head: minimum-size items
     words = prep.bits.cpu().numpy().view(np.uint64)
     fixed = T.fully_masked_rows_to_true(mask)
     for b in range(B):
@@ -154,7 +154,8 @@ def test_mfma_kernel(B, H, Hkv, W, L, prev_lens):
     q = rng.standard_normal((B, H, nq, D)); k = rng.standard_normal((B, Hkv, kv, D)); v = rng.standard_normal((B, Hkv, kv, D))
     got, ref = _run(q, k, v, mask, torch.bfloat16, force_generic=False, cache_like=True)
     _assert_close(got, ref, torch.bfloat16)
-    # a plan made for many heads cuts every row into minimum-size items: exercises the partials
+    # (with few heads the plan above cuts long rows into minimum-size items and merges partials)
+    # a plan made for many heads leaves every row whole: one work item per row, no partials
     got3, _ = _run(q, k, v, mask, torch.bfloat16, force_generic=False, cache_like=True, n_heads_for_plan=4096)
     _assert_close(got3, ref, torch.bfloat16)
     got2, _ = _run(q, k, v, mask, torch.bfloat16, force_generic=True, cache_like=True)
@@ -176,6 +177,33 @@ def test_mfma_kernel_every_wave_layout(nq):
         q = rng.standard_normal((B, H, nq, 128)); k = rng.standard_normal((B, H, kv, 128)); v = rng.standard_normal((B, H, kv, 128))
         got, ref = _run(q, k, v, mask, torch.bfloat16, force_generic=False, cache_like=True)
         _assert_close(got, ref, torch.bfloat16)
+
+
+def test_split_rows_merge_is_repeatable_on_one_plan():
+    """Every row split into many work items (a plan made for one head: minimum-size items): the item that arrives last
+    merges the partials and leaves the plan's arrival counters at zero, so launch after launch on
+    the same plan (one per layer in the model) must give the same bits, equal to the unsplit result
+    up to the rounding of the merge."""
+    from recurrent_drafting_amd import attention
+
+    torch.manual_seed(3)
+    B, H, D, nq, kv = 3, 6, 128, 150, 1900
+    q = torch.randn(B, nq, H, D, device="cuda", dtype=torch.bfloat16).permute(0, 2, 1, 3)
+    k = torch.randn(B, H, kv, D, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(B, H, kv, D, device="cuda", dtype=torch.bfloat16)
+    mask = torch.rand(B, nq, kv, device="cuda") > 0.4
+    whole_plan = attention.prepare(mask, n_heads=4096)  # a share of many heads: nothing is split
+    assert int(whole_plan.plan[0]) == B
+    whole = attention.masked_attention(q, k, v, whole_plan)
+    prep = attention.prepare(mask, n_heads=1)
+    assert int(prep.plan[0]) >= 3 * B  # really split
+    first = attention.masked_attention(q, k, v, prep).clone()
+    for _ in range(40):
+        again = attention.masked_attention(q, k, v, prep)
+        assert torch.equal(again, first)
+    counters = prep.plan[-(B * 128 * 1):]
+    assert not counters.any()
+    assert (first.float() - whole.float()).abs().max() <= 2e-2 * whole.float().abs().max()
 
 
 def test_mfma_kernel_pad_tokens_inside_the_prefix_and_empty_rows():
