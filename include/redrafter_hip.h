@@ -198,6 +198,16 @@ RD_API int rd_add_rms_norm(const void* x, int64_t x_row_stride, const void* delt
                            int64_t rows, int cols, float eps, void* stream);
 RD_API int rd_silu_mul(const void* gate, const void* up, int64_t in_row_stride, void* y,
                        int64_t y_row_stride, int dtype, int64_t rows, int cols, void* stream);
+/* The elementwise steps between the GEMMs of the drafter head, one launch each.
+ * mode 0: y = x + silu(z), ResBlock.forward (modeling_drafter.py:38-39);
+ * mode 1: y = silu(x + z), the recurrent state update (modeling_drafter.py:192-197).
+ * y2 (optional) receives the same values, e.g. the state's half of the [context, state] tensor
+ * that upstream builds with torch.cat (modeling_drafter.py:199).  (rows, cols) with element row
+ * strides, cols contiguous; every intermediate is rounded to dtype as the separate torch kernels
+ * round it. */
+RD_API int rd_silu_add(const void* x, int64_t x_row_stride, const void* z, int64_t z_row_stride,
+                       void* y, int64_t y_row_stride, void* y2, int64_t y2_row_stride, int mode,
+                       int dtype, int64_t rows, int cols, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Rotary position embedding of the new queries and keys, fused with the in-place append of the

@@ -6,6 +6,11 @@
 //                     modeling_llama.py:27-32 (LlamaRMSNorm.forward), :196, :198 (the += updates)
 //   rd_silu_mul       y = silu(gate) * up, gate and up the two halves of one fused projection
 //                     modeling_llama.py:84-85 (LlamaMLP.forward)
+//   rd_silu_add       the two elementwise steps of the drafter head, one launch each:
+//                     mode 0  y = x + silu(z)   ResBlock.forward (modeling_drafter.py:38-39)
+//                     mode 1  y = silu(x + z)   the recurrent state update (modeling_drafter.py:192-197),
+//                             written to up to two places (the state, and its half of the
+//                             [context, state] input of the head, modeling_drafter.py:199)
 //
 // Rounding follows the tensors' dtype at the points where upstream materialises a tensor: the sum
 // h, the normalised value before the gain, the activation before the product.  The mean of squares
@@ -126,6 +131,34 @@ __global__ __launch_bounds__(kThreads) void silu_mul_kernel(
   *reinterpret_cast<V*>(y + row * y_stride + (int64_t)vi * N) = o;
 }
 
+template <typename T, int MODE>
+__global__ __launch_bounds__(kThreads) void silu_add_kernel(
+    const T* __restrict__ x, int64_t x_stride, const T* __restrict__ z, int64_t z_stride, T* __restrict__ y,
+    int64_t y_stride, T* __restrict__ y2, int64_t y2_stride, int cols) {
+#pragma clang fp contract(off)
+  using V = Vec<T>;
+  constexpr int N = V::N;
+  const int64_t row = blockIdx.y;
+  const int vi = blockIdx.x * kThreads + threadIdx.x;
+  if (vi >= cols / N) return;
+  const V a = *reinterpret_cast<const V*>(x + row * x_stride + (int64_t)vi * N);
+  const V b = *reinterpret_cast<const V*>(z + row * z_stride + (int64_t)vi * N);
+  V o;
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    const float av = Cvt<T>::up(a.v[e]), bv = Cvt<T>::up(b.v[e]);
+    if (MODE == 0) {
+      const float act = Cvt<T>::up(Cvt<T>::down(bv / (1.0f + expf(-bv))));
+      o.v[e] = Cvt<T>::down(av + act);
+    } else {
+      const float s = Cvt<T>::up(Cvt<T>::down(av + bv));
+      o.v[e] = Cvt<T>::down(s / (1.0f + expf(-s)));
+    }
+  }
+  *reinterpret_cast<V*>(y + row * y_stride + (int64_t)vi * N) = o;
+  if (y2 != nullptr) *reinterpret_cast<V*>(y2 + row * y2_stride + (int64_t)vi * N) = o;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <typename T>
@@ -197,4 +230,44 @@ extern "C" int rd_silu_mul(const void* gate, const void* up, int64_t in_row_stri
     }
   }
   return rd::check_launch("rd_silu_mul");
+}
+
+extern "C" int rd_silu_add(const void* x, int64_t x_row_stride, const void* z, int64_t z_row_stride,
+                           void* y, int64_t y_row_stride, void* y2, int64_t y2_row_stride, int mode,
+                           int dtype, int64_t rows, int cols, void* stream) {
+  RD_REQUIRE(rows > 0 && cols > 0 && rows <= 65535, RD_EINVAL, "rd_silu_add: bad sizes (rows %lld cols %d)",
+             (long long)rows, cols);
+  RD_REQUIRE(mode == 0 || mode == 1, RD_EINVAL, "rd_silu_add: unknown mode %d", mode);
+  RD_REQUIRE(dtype == RD_F32 || dtype == RD_BF16 || dtype == RD_F16, RD_EINVAL, "rd_silu_add: unknown dtype %d", dtype);
+  const int vec = dtype == RD_F32 ? 4 : 8;
+  RD_REQUIRE(cols % vec == 0, RD_ELIMIT, "rd_silu_add: cols %d must be a multiple of %d", cols, vec);
+  RD_REQUIRE(x && z && y, RD_EINVAL, "rd_silu_add: null pointer");
+  RD_REQUIRE(aligned16(x) && aligned16(z) && aligned16(y) && aligned16(y2) && x_row_stride % vec == 0 &&
+                 z_row_stride % vec == 0 && y_row_stride % vec == 0 && (!y2 || y2_row_stride % vec == 0) &&
+                 x_row_stride >= cols && z_row_stride >= cols && y_row_stride >= cols && (!y2 || y2_row_stride >= cols),
+             RD_EINVAL, "rd_silu_add: alignment or strides");
+  hipStream_t s = rd::as_stream(stream);
+  const dim3 grid((cols / vec + kThreads - 1) / kThreads, (unsigned)rows);
+#define RD_SA(T, MODE)                                                                                   \
+  hipLaunchKernelGGL((silu_add_kernel<T, MODE>), grid, dim3(kThreads), 0, s, reinterpret_cast<const T*>(x), \
+                     x_row_stride, reinterpret_cast<const T*>(z), z_row_stride, reinterpret_cast<T*>(y),  \
+                     y_row_stride, reinterpret_cast<T*>(y2), y2_row_stride, cols)
+  {
+    rd::ScopedTiming rd_t("silu_add_kernel", s);
+    if (mode == 0) {
+      switch (dtype) {
+        case RD_F32: RD_SA(float, 0); break;
+        case RD_BF16: RD_SA(__hip_bfloat16, 0); break;
+        default: RD_SA(__half, 0); break;
+      }
+    } else {
+      switch (dtype) {
+        case RD_F32: RD_SA(float, 1); break;
+        case RD_BF16: RD_SA(__hip_bfloat16, 1); break;
+        default: RD_SA(__half, 1); break;
+      }
+    }
+  }
+#undef RD_SA
+  return rd::check_launch("rd_silu_add");
 }

@@ -40,6 +40,7 @@ _PROTOTYPES = {
     "rd_kv_compact": (_I, [_P, _I, _I, _I, _L, _L, _L, _I, _P, _P]),
     "rd_add_rms_norm": (_I, [_P, _L, _P, _L, _P, _P, _L, _P, _L, _I, _L, _I, _F, _P]),
     "rd_silu_mul": (_I, [_P, _P, _L, _P, _L, _I, _L, _I, _P]),
+    "rd_silu_add": (_I, [_P, _L, _P, _L, _P, _L, _P, _L, _I, _I, _L, _I, _P]),
     "rd_rope_append": (
         _I,
         [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _L, _P, _P],

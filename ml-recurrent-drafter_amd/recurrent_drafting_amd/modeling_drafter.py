@@ -42,6 +42,26 @@ class ResBlock(torch.nn.Module):
         return x + torch.nn.functional.silu(self.linear(x))
 
 
+def silu_add(x: torch.Tensor, z: torch.Tensor, mode: int, also: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """mode 0: x + silu(z); mode 1: silu(x + z).  x and z (..., cols) of one dtype with contiguous
+    columns and a common row layout; `also`, a (..., cols) view of the same leading shape whose
+    rows may be strided, receives a second copy of the result."""
+    cols = x.shape[-1]
+    assert x.shape == z.shape and x.dtype == z.dtype
+    x2, z2 = x.reshape(-1, cols), z.reshape(-1, cols)
+    assert x2.stride(1) == 1 and z2.stride(1) == 1
+    out = torch.empty((x2.shape[0], cols), dtype=x.dtype, device=x.device)
+    y2 = None
+    if also is not None:
+        assert also.shape == x.shape and also.dtype == x.dtype and also.stride(-1) == 1
+        y2 = also.view(-1, cols)  # (a view: the rows of `also` must be evenly strided)
+    _hip.check(_hip.lib().rd_silu_add(
+        _hip.ptr(x2), x2.stride(0), _hip.ptr(z2), z2.stride(0), _hip.ptr(out), out.stride(0),
+        _hip.ptr(y2), 0 if y2 is None else y2.stride(0), mode, _hip.dtype_code(x.dtype),
+        x2.shape[0], cols, _hip.stream()))
+    return out.view(x.shape)
+
+
 def _gather_beams(x: torch.Tensor, selected_beams: torch.Tensor) -> torch.Tensor:
     """x (B, W, ...) re-ordered along dim 1 by selected_beams (B, W) (modeling_drafter.py:42-53)."""
     B, W = x.shape[0], x.shape[1]
@@ -126,8 +146,13 @@ class Drafter(transformers.PreTrainedModel):
             self.rnn_w = torch.nn.Linear(cfg.hidden_size, cfg.hidden_size, bias=False)
 
     def raw_logits(self, x: torch.Tensor) -> torch.Tensor:
-        """Vocabulary logits of [context, state] before any normalisation."""
-        return self.lm_head(self.input_proj(x) if hasattr(self, "input_proj") else x)
+        """Vocabulary logits of [context, state] before any normalisation: `self.lm_head`, with
+        the sum and the activation of every ResBlock (modeling_drafter.py:38-39) in one kernel."""
+        x = self.input_proj(x) if hasattr(self, "input_proj") else x
+        *blocks, head = self.lm_head
+        for block in blocks:
+            x = silu_add(x, block.linear(x), mode=0)
+        return head(x)
 
     def compute_logits(self, x: torch.Tensor) -> torch.Tensor:
         """Logits with the row maximum at zero and everything below the top 50 at LOG_0
@@ -160,6 +185,10 @@ class Drafter(transformers.PreTrainedModel):
         context = prompt_state.unsqueeze(1).expand(B, W, hidden)
         beams = init_token.view(B, 1, 1).expand(B, W, 1).contiguous()
         state = torch.zeros(B, W, hidden, device=dev, dtype=prompt_state.dtype)
+        # [context, state], the input of the head (modeling_drafter.py:199): the context half is
+        # written once, the state half by the kernel that forms the state
+        head_in = torch.empty(B, W, 2 * hidden, device=dev, dtype=prompt_state.dtype)
+        head_in[..., :hidden] = context
         step_log_probs: List[torch.Tensor] = []
         step_parents: List[torch.Tensor] = []
 
@@ -170,10 +199,12 @@ class Drafter(transformers.PreTrainedModel):
             rows = 1 if it == 0 and self.first_iteration_once else W
             last = embeddings(beams[:, :rows, -1])
             if self.config.rnn:
-                state = torch.nn.functional.silu(self.rnn_w(last) + self.rnn_u(state[:, :rows]))
+                state = silu_add(self.rnn_w(last), self.rnn_u(state[:, :rows]), mode=1,
+                                 also=head_in[:, :rows, hidden:])
             else:
                 state = last + state[:, :rows]
-            logits = self.raw_logits(torch.cat([context[:, :rows], state], dim=-1))
+                head_in[:, :rows, hidden:] = state
+            logits = self.raw_logits(head_in[:, :rows])
             if rows != W:
                 logits = logits.expand(B, W, V)
                 state = state.expand(B, W, hidden)

@@ -103,3 +103,35 @@ def test_argument_errors():
     rc = _hip.lib().rd_add_rms_norm(_hip.ptr(x), 12, None, 0, _hip.ptr(w), _hip.ptr(x), 12, None, 0,
                                     _hip.dtype_code(torch.float32), 2, 10, 1e-6, _hip.stream())
     assert rc != 0 and b"multiple" in _hip.lib().rd_last_error()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_silu_add_matches_the_torch_ops_bit_for_bit(dtype):
+    """x + silu(z) and silu(x + z) as torch computes them with separate kernels
+    (modeling_drafter.py:38-39, 192-197), strided rows and the second output included."""
+    from recurrent_drafting_amd import modeling_drafter as md
+
+    torch.manual_seed(1)
+    B, W, cols = 3, 5, 256
+    wide = (torch.randn(B, W, 2 * cols, device="cuda") * 3).to(dtype)
+    x = wide[..., :cols]  # strided rows
+    z = (torch.randn(B, W, cols, device="cuda") * 3).to(dtype)
+    got0 = md.silu_add(x, z, mode=0)
+    assert torch.equal(got0, x + torch.nn.functional.silu(z))
+    also = torch.zeros(B, W, 2 * cols, device="cuda", dtype=dtype)
+    got1 = md.silu_add(x, z, mode=1, also=also[..., cols:])
+    want1 = torch.nn.functional.silu(x + z)
+    assert torch.equal(got1, want1) and torch.equal(also[..., cols:], want1) and not also[..., :cols].any()
+    one = md.silu_add(x[:, :1], z[:, :1], mode=1, also=also[:, :1, :cols])  # one row per batch row
+    assert torch.equal(one, want1[:, :1]) and torch.equal(also[:, :1, :cols], want1[:, :1])
+
+
+def test_raw_logits_equals_the_module_stack():
+    import recurrent_drafting_amd as rd
+
+    torch.manual_seed(2)
+    cfg = rd.configuration_drafter.DrafterConfig(vocab_size=320, hidden_size=64, exit_dim=128, num_draft_layers=2, rnn=True)
+    drafter = rd.modeling_drafter.Drafter(cfg).cuda().to(torch.bfloat16).eval()
+    x = torch.randn(4, 7, 128, device="cuda").to(torch.bfloat16)
+    with torch.inference_mode():
+        assert torch.equal(drafter.raw_logits(x), drafter.lm_head(x))
