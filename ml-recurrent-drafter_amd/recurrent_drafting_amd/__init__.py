@@ -12,9 +12,11 @@ from . import (  # noqa: F401
     acceptance,
     attention,
     configuration_drafter,
+    gemm_tuning,
     kv_cache,
     modeling_drafter,
     modeling_llama,
+    packed_rows,
     recurrent_drafting,
     rng,
     stats,

@@ -32,7 +32,7 @@ import torch
 import torch.distributions as dist
 import transformers
 
-from . import acceptance, attention, kv_cache, modeling_drafter, modeling_llama, stats, tree_attention
+from . import acceptance, attention, gemm_tuning, kv_cache, modeling_drafter, modeling_llama, stats, tree_attention
 from .acceptance import (  # noqa: F401  (re-exported: the reference's helper names)
     _choose_from_candidates,
     _count_left_paddings,
@@ -144,6 +144,7 @@ class RecurrentDrafting(torch.nn.Module):
         super().__init__()
         self.llm = llm
         self.drafter = drafter
+        gemm_tuning.load()  # kernel selection table for the dense layers' GEMMs (no-op without one)
 
     def llm_n_kv_heads(self) -> int:
         if isinstance(self.llm, modeling_llama.LlamaForCausalLM):
