@@ -16,6 +16,7 @@ namespace {
 
 constexpr int kMaxRowWaves = 16;
 constexpr int kCap = 2048;  // LDS candidate list
+constexpr int kPivotMargin = 16;  // thread maxima taken beyond k when the pivot is chosen
 
 template <typename T> struct Num;
 template <> struct Num<float> {
