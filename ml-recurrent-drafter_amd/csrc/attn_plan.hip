@@ -58,14 +58,21 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
   int32_t* per_row = plan + RD_PLAN_HDR;
   int32_t* items = plan + RD_PLAN_HDR + 4 * B;
   // pass 1: per batch row, first attended key and number of splits
-  for (int b = threadIdx.x; b < B; b += kThreads) {
+  // (one wave per batch row at a time: the minimum over its query rows)
+  for (int b = threadIdx.x >> 6; b < B; b += kThreads / 64) {
     int first = kv_len;
-    for (int q = 0; q < n_q; ++q) {
+    for (int q = threadIdx.x & 63; q < n_q; q += 64) {
       const int f = row_first[(int64_t)b * n_q + q];
       first = f < first ? f : first;
     }
-    per_row[4 * b + 0] = (first / 64) * 64;
-    per_row[4 * b + 3] = 0;
+    for (int off = 32; off > 0; off >>= 1) {
+      const int o = __shfl_xor(first, off);
+      first = o < first ? o : first;
+    }
+    if ((threadIdx.x & 63) == 0) {
+      per_row[4 * b + 0] = (first / 64) * 64;
+      per_row[4 * b + 3] = 0;
+    }
   }
   __syncthreads();
   if (threadIdx.x == 0) {
