@@ -23,7 +23,7 @@ __global__ __launch_bounds__(kThreads) void tree_rows_kernel(
     int64_t* __restrict__ unpacker, int64_t* __restrict__ sel_tok, int32_t* __restrict__ sel_idx,
     int32_t* __restrict__ counts) {
   __shared__ int64_t s_tok[kMaxTokens];
-  __shared__ int16_t s_owner[kMaxTokens];
+  __shared__ int32_t s_owner[kMaxTokens];
   __shared__ int16_t s_nown[kMaxWidth];
   __shared__ int32_t s_start[kMaxWidth];
 
@@ -33,17 +33,21 @@ __global__ __launch_bounds__(kThreads) void tree_rows_kernel(
   for (int t = threadIdx.x; t < WL; t += kThreads) s_tok[t] = row[t];
   __syncthreads();
 
-  // owner[i][k] = smallest j whose first k+1 tokens equal beam i's.
-  for (int i = threadIdx.x; i < W; i += kThreads) {
+  // owner[i][k] = smallest j whose first k+1 tokens equal beam i's.  Every pair (i, j < i) is
+  // looked at by some thread: the length of the common prefix, then a minimum per position.
+  for (int t = threadIdx.x; t < WL; t += kThreads) s_owner[t] = t / L;  // a beam matches itself
+  __syncthreads();
+  for (int pr = threadIdx.x; pr < W * W; pr += kThreads) {
+    const int i = pr / W, j = pr - i * W;
+    if (j >= i) continue;
     const int64_t* mine = s_tok + i * L;
-    int best = 0;  // positions [0,best) already have their owner
-    for (int j = 0; j <= i && best < L; ++j) {
-      const int64_t* other = s_tok + j * L;
-      int m = 0;
-      while (m < L && other[m] == mine[m]) ++m;
-      for (int k = best; k < m; ++k) s_owner[i * L + k] = (int16_t)j;
-      best = m > best ? m : best;
-    }
+    const int64_t* other = s_tok + j * L;
+    int m = 0;
+    while (m < L && other[m] == mine[m]) ++m;
+    for (int k = 0; k < m; ++k) atomicMin(&s_owner[i * L + k], j);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < W; i += kThreads) {
     int n = 0;
     for (int k = 0; k < L; ++k) n += (s_owner[i * L + k] == i);
     s_nown[i] = (int16_t)n;
