@@ -179,6 +179,24 @@ def test_mfma_kernel_every_wave_layout(nq):
         _assert_close(got, ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("nq,kv_prev", [(300, 1500), (150, 2100), (96, 1300)])
+def test_mfma_kernel_split_rows_in_every_layout_against_the_oracle(nq, kv_prev):
+    """Long rows with few heads: the plan cuts every row into 512-key items, so several work items
+    (and, at 300 queries, two query tiles each) meet at the arrival counters and one of them merges."""
+    from recurrent_drafting_amd import attention
+
+    rng = np.random.default_rng(nq + kv_prev)
+    B, H = 2, 2
+    kv = kv_prev + nq
+    mask = rng.random((B, nq, kv)) > 0.5
+    mask[1, :, : kv_prev - 200] = False  # a row that starts late: fewer items than row 0
+    q = rng.standard_normal((B, H, nq, 128)); k = rng.standard_normal((B, H, kv, 128)); v = rng.standard_normal((B, H, kv, 128))
+    prep = attention.prepare(_dev(mask, torch.bool), n_heads=H)
+    assert int(prep.plan[0]) >= 4  # split
+    got, ref = _run(q, k, v, mask, torch.bfloat16, force_generic=False, cache_like=True)
+    _assert_close(got, ref, torch.bfloat16)
+
+
 def test_split_rows_merge_is_repeatable_on_one_plan():
     """Every row split into many work items (a plan made for one head: minimum-size items): the item that arrives last
     merges the partials and leaves the plan's arrival counters at zero, so launch after launch on
