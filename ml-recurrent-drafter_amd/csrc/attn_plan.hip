@@ -152,8 +152,6 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
 
 extern "C" size_t rd_attn_plan_ints(int batch, int n_q, int kv_len) {
   if (batch <= 0 || n_q <= 0 || kv_len <= 0) return 0;
-  const int max_splits = rd::attn_max_splits(kv_len);
-  (void)max_splits;
   return rd::attn_counter_offset(batch, n_q, kv_len) + rd::attn_counter_ints(batch, n_q);
 }
 
