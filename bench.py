@@ -1,6 +1,7 @@
 """Benchmark of the ReDrafter decode step on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py --cpu-kernels      (per-kernel CPU baselines only; no GPU needed)
 
 Workload (the configuration the headline metric is quoted on): random-init Vicuna-7B-shaped Llama
 in bf16 (32 layers, hidden 4096, 32 heads, FFN 11008, vocab 32000) with a ReDrafter head (hidden
@@ -260,13 +261,121 @@ def cpu_baseline(per_seq_tokens: float):
     )
 
 
+def cpu_kernel_baselines(reps: int = 3):
+    """Per-kernel CPU baselines: the torch restatement of each stage on the host cores, on the shapes
+    of the kernel micro-benchmarks (ml-recurrent-drafter_amd/kernel_bench.py).  Needs no GPU.  Prints one
+    line per case: best of `reps` passes after one warm-up pass."""
+    import numpy as np
+    from oracle import torch_path as P
+    from oracle import tree_oracle as T
+
+    threads = torch.get_num_threads()
+    log(f"[bench] per-kernel cpu baselines: {threads} threads, best of {reps} after one warm-up pass")
+    rows = []
+
+    def case(name, fn, n=reps):
+        with torch.inference_mode():
+            fn()
+            best = float("inf")
+            for _ in range(n):
+                t = time.perf_counter()
+                fn()
+                best = min(best, time.perf_counter() - t)
+        rows.append((name, best))
+        print(f"{name:<78} cpu {best * 1e3:11.3f} ms   ({threads} threads)", flush=True)
+
+    B, W, L, V, H, D = BATCH, WIDTH, LENGTH, 32000, 32, 128
+    g = torch.Generator().manual_seed(SEED)
+    beams = torch.from_numpy(T.synthetic_beams(B, W, L, seed=SEED))
+    for prev in (0, 2548):
+        pm = torch.ones(B, prev, dtype=torch.int64)
+        case(f"tree_pack batch {B} prev {prev} (dedup, unpacker, pack, mask)", lambda: P.pack(beams, pm))
+
+    # verification attention: additive bias + SDPA as the decoder layer issues them (one layer)
+    rng = np.random.default_rng(SEED)
+    for label, lens in (("cached length U[500,2548]", rng.integers(500, 2549, size=B)), ("cached length 525 for every row", np.full(B, 525))):
+        S = int(lens.max())
+        pm = torch.zeros(B, S, dtype=torch.int64)
+        for b in range(B):
+            pm[b, S - int(lens[b]):] = 1
+        tok, _, mask, _ = P.pack(beams, pm)
+        n = tok.shape[1]
+        q = torch.randn(B, H, n, D, generator=g).bfloat16()
+        k = torch.randn(B, H, S + n, D, generator=g).bfloat16()
+        v = torch.randn(B, H, S + n, D, generator=g).bfloat16()
+
+        def attn():
+            m = P.rows_without_keys_to_true(mask)
+            return torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=P.bias(m.unsqueeze(1), q.dtype))
+        case(f"verify_attention {label} (n_q={n}, sum keys={int(lens.sum()) + B * n}), one layer", attn)
+
+    # one beam-search step after the drafter's GEMMs: the chain of modeling_drafter.py:201-215
+    logits = torch.randn(B, W, V, generator=g).bfloat16()
+    log_p_beam = torch.randn(B, W, generator=g)
+
+    def beam_step():
+        x = logits - logits.max(dim=-1, keepdim=True).values
+        x = P.top_k_filter(x)
+        logp = torch.log_softmax(x, dim=-1)
+        score = (logp + log_p_beam.unsqueeze(-1)).reshape(B, W * V)
+        top, idx = torch.topk(score, W, dim=-1)
+        return top, idx % V, idx // V
+    case(f"beam_topk step, logits ({B},{W},{V}) bf16", beam_step)
+
+    packed_logits = torch.randn(1448, V, generator=g).bfloat16()
+    case("argmax packed bf16 logits (rows 1448)", lambda: packed_logits.argmax(dim=-1))
+    case("verify_row_stats: top-50 filter + log_softmax of packed logits (rows 1448, fp32)",
+         lambda: torch.log_softmax(P.top_k_filter(packed_logits.float()), dim=-1))
+    hidden = torch.randn(B, 181, 4096, generator=g).bfloat16()
+    unpacker = torch.randint(0, 181, (B, W, L), generator=g)
+    case("unpack hidden (B,n,4096) bf16", lambda: P.unpack(hidden, unpacker))
+
+    # KV cache: append of the tree rows' K (one layer), Cache.unpack and the re-alignment (32 layers)
+    prev, n = 1500, 168
+    cache = P.Cache(B, prev + n + 64, 32, H, D, torch.bfloat16, "cpu")
+    cache.set_length(prev)
+    new_k = torch.randn(B, H, n, D, generator=g).bfloat16()
+    cos_t, sin_t = P._rope_tables(D, 10000.0, 2048, "cpu", torch.bfloat16)
+    pos = torch.randint(prev, prev + L, (B, n), generator=g)
+
+    def rope_append():
+        cache.set_length(prev)
+        c, s_ = cos_t[pos].unsqueeze(1), sin_t[pos].unsqueeze(1)
+        cache.append(0, 0, P._rope(new_k, c, s_))
+        cache.append(0, 1, new_k)
+        cache.set_length(prev)
+    case(f"rope + append prev {prev} n {n} (K rotated, V plain), one layer", rope_append)
+    unp = torch.randint(0, n, (B, W, L), generator=g)
+
+    def kv_unpack():
+        cache.set_length(prev + n)
+        cache.unpack(prev, unp)
+        cache.set_length(prev)
+    case(f"Cache.unpack prev {prev} n {n}, 32 layers", kv_unpack, n=2)
+    ids = torch.randint(1, V, (B, prev), generator=g)
+    n_tokens = torch.tensor([0, 1, 2, 3, 4, 4, 2, 1])[:B]
+    seq_in_beam = torch.randint(0, W, (B,), generator=g)
+
+    def realign():
+        cache.set_length(prev + W * L)
+        P.realign(ids, n_tokens, seq_in_beam, beams, cache, 0)
+        cache.set_length(prev)
+    case(f"realign ids + KV prev {prev}, accepted lengths differ, 32 layers", realign, n=2)
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-kernels", action="store_true",
+                    help="only time the CPU restatement of each stage on the micro-benchmark shapes (no GPU needed)")
     args = ap.parse_args()
+    if args.cpu_kernels:
+        cpu_kernel_baselines()
+        return
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (the decode step would shard by batch row with no "
             "exchange between the GPUs); --gpus must be 1")
