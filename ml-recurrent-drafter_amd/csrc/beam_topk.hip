@@ -314,7 +314,9 @@ int launch_rows(const void* logits, int64_t row_stride, int rows, int V, const f
                        force_fallback); } while (0)
   switch (row_geometry(V)) {
     case 0: RD_ROWS(32, 256); break;
-    case 1: RD_ROWS(128, 256); break;
+    // few rows (batch*width below two per compute unit): twice the threads per row hide more of the
+    // per-row latency (360 rows of 32000: 22.5 -> 18.7 us); with many rows the smaller workgroup wins
+    case 1: if (rows <= 512) RD_ROWS(64, 512); else RD_ROWS(128, 256); break;
     default: RD_ROWS(64, 1024); break;
   }
 #undef RD_ROWS

@@ -9,7 +9,8 @@ namespace {
 
 constexpr int kThreads = 256;
 
-using vec16 = uint4;
+// (a plain vector type: arrays of HIP's uint4 class were placed in scratch memory by the compiler)
+typedef unsigned int vec16 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(kThreads) void gather_rows_kernel(
     const char* __restrict__ src, int64_t src_batch_stride, int64_t row_bytes,
@@ -43,21 +44,21 @@ __global__ __launch_bounds__(kThreads) void kv_unpack_kernel(
   const int b = (int)((slab / H) % B);
   char* base = cache + slab * max_len * row_bytes + prev * row_bytes;
   const int64_t* idx = index + (int64_t)b * T;
-  for (int64_t c0 = 0; c0 < row_bytes; c0 += chunk_bytes) {
-    const int cb = (int)((row_bytes - c0) < chunk_bytes ? (row_bytes - c0) : chunk_bytes);
-    const int vpr = cb >> 4;  // 16-byte vectors per row in this chunk
-    for (int v = threadIdx.x; v < n_src * vpr; v += kThreads) {
-      const int r = v / vpr, c = v - r * vpr;
-      s_rows[v] = *reinterpret_cast<const vec16*>(base + (int64_t)r * row_bytes + c0 + (c << 4));
-    }
-    __syncthreads();
-    for (int v = threadIdx.x; v < T * vpr; v += kThreads) {
-      const int t = v / vpr, c = v - t * vpr;
-      const int64_t r = idx[t];
-      if (r >= 0 && r < n_src)
-        *reinterpret_cast<vec16*>(base + (int64_t)t * row_bytes + c0 + (c << 4)) = s_rows[r * vpr + c];
-    }
-    __syncthreads();
+  // one column chunk of the slab per workgroup (blockIdx.y): narrow chunks keep the LDS share
+  // small, so that several workgroups are resident and their read and write phases overlap
+  const int64_t c0 = (int64_t)blockIdx.y * chunk_bytes;
+  const int cb = (int)((row_bytes - c0) < chunk_bytes ? (row_bytes - c0) : chunk_bytes);
+  const int vpr = cb >> 4;  // 16-byte vectors per row in this chunk
+  for (int v = threadIdx.x; v < n_src * vpr; v += kThreads) {
+    const int r = v / vpr, c = v - r * vpr;
+    s_rows[v] = *reinterpret_cast<const vec16*>(base + (int64_t)r * row_bytes + c0 + (c << 4));
+  }
+  __syncthreads();
+  for (int v = threadIdx.x; v < T * vpr; v += kThreads) {
+    const int t = v / vpr, c = v - t * vpr;
+    const int64_t r = idx[t];
+    if (r >= 0 && r < n_src)
+      *reinterpret_cast<vec16*>(base + (int64_t)t * row_bytes + c0 + (c << 4)) = s_rows[r * vpr + c];
   }
 }
 
@@ -98,11 +99,13 @@ __global__ __launch_bounds__(kThreads) void kv_compact_kernel(
     for (int64_t it = 0; it < n_chunks; ++it) {
       // moving right: highest chunk first; moving left: lowest chunk first
       const int64_t ch = new_pads > old_pads ? n_chunks - 1 - it : it;
+      // (loads past the end are clamped, not skipped: an element left unset on some path would
+      // send the whole array through scratch memory, i.e. through HBM a second time)
       vec16 r[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int64_t i = ch * kChunk + (int64_t)u * kThreads + threadIdx.x;
-        if (i < nvec) r[u] = src[i];
+        r[u] = src[i < nvec ? i : nvec - 1];
       }
       __syncthreads();  // the whole chunk is in registers before any of it is overwritten
 #pragma unroll
@@ -173,11 +176,15 @@ extern "C" int rd_kv_unpack(void* cache, int n_layers, int batch, int n_heads, i
              (long long)prev, n_out, n_src, (long long)max_len);
   constexpr int kLds = 64 * 1024;
   RD_REQUIRE((int64_t)n_src * 16 <= kLds, RD_ELIMIT, "rd_kv_unpack: n_src %d > %d", n_src, kLds / 16);
-  int64_t chunk = (kLds / n_src) / 16 * 16;
+  // column chunk: one 128-byte line per row (whole 256-byte rows left too few workgroups resident:
+  // 450 us against 352 us for the 7B cache at 1500 tokens; 64-byte pieces took 624 us)
+  int64_t chunk = (int64_t)n_src * 128 <= kLds ? 128 : (kLds / n_src) / 16 * 16;
   if (chunk > row_bytes) chunk = row_bytes;
   const size_t lds = (size_t)n_src * chunk;
   const int64_t slabs = (int64_t)n_layers * 2 * batch * n_heads;
-  { rd::ScopedTiming rd_t("kv_unpack_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(kv_unpack_kernel, dim3(slabs), dim3(kThreads), lds, rd::as_stream(stream),
+  const int col_chunks = (int)((row_bytes + chunk - 1) / chunk);
+  RD_REQUIRE(col_chunks <= 65535, RD_ELIMIT, "rd_kv_unpack: row_bytes %lld needs %d column chunks", (long long)row_bytes, col_chunks);
+  { rd::ScopedTiming rd_t("kv_unpack_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(kv_unpack_kernel, dim3(slabs, col_chunks), dim3(kThreads), lds, rd::as_stream(stream),
                      reinterpret_cast<char*>(cache), batch, n_heads, max_len, row_bytes, prev, index,
                      n_out, n_src, (int)chunk); }
   return rd::check_launch("rd_kv_unpack");

@@ -315,7 +315,8 @@ __device__ inline float row_kth_radix(const T* __restrict__ x_row, int V, float 
 // Launch geometry for a vocabulary of V elements: threads per row x values per thread (a multiple
 // of the 16-byte vector for every dtype).  -1 when V is beyond the compiled limit.
 //   V <= 8192        256 threads x 32
-//   V <= 32768       256 threads x 128   (two workgroups per compute unit)
+//   V <= 32768       256 threads x 128   (two workgroups per compute unit); the beam search uses
+//                    512 threads x 64 when it has at most 512 rows
 //   V <= 65536      1024 threads x 64
 inline int row_geometry(int V) { return V <= 8192 ? 0 : (V <= 32768 ? 1 : (V <= 65536 ? 2 : -1)); }
 
