@@ -154,13 +154,20 @@ RD_API int rd_count_left_paddings(const int64_t* input_ids, int64_t ids_row_stri
  * src_row[j] is the cache row holding accepted token j: prev + seq*length + j when unpacker is
  * NULL (cache already unpacked by rd_kv_unpack), prev + unpacker[b,seq,j] otherwise.
  * new_ids: capacity batch*(prev+length), written as a contiguous (batch, M) array.
+ * kv_row_shift (batch int32 on the device, read and written, or NULL): with it the cache is not
+ * re-aligned.  Token column c of row b is taken to live in cache row c - kv_row_shift[b]; the plan
+ * is written in cache rows with old_pads == new_pads (rd_kv_compact then only appends the accepted
+ * rows behind the live ones) and kv_row_shift[b] grows by new_pads - old_pads.  The reference moves
+ * the whole live cache on every step (recurrent_drafting.py:200-209); the same array is handed to
+ * rd_rope_append and rd_attn_prepare, and rd_kv_materialize moves the rows once when the
+ * reference's layout is wanted.
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_realign_plan_ints(int batch, int length);
 RD_API int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride, int64_t prev,
                            const int64_t* n_tokens_in_seq, const int64_t* seq_in_beam,
                            const int64_t* beams, const int64_t* unpacker, int batch, int width,
                            int length, int64_t pad_token_id, int32_t* plan, int64_t* new_ids,
-                           void* stream);
+                           int32_t* kv_row_shift, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * KV cache, shape (n_layers, 2, batch, n_heads, max_len, head_dim), rows of row_bytes bytes.
@@ -177,6 +184,14 @@ RD_API int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride, int
 RD_API int rd_kv_unpack(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
                         int64_t row_bytes, int64_t prev, const int64_t* index, int n_out, int n_src,
                         void* stream);
+/* rd_kv_materialize: undoes kv_row_shift (see rd_realign_plan): every row's cache rows move to
+ * the place where column and cache row agree (columns [0, length)), and the shifts are cleared.
+ * plan: rd_kv_materialize_plan_ints(batch) int32 of workspace.  No counterpart in the reference,
+ * which keeps that layout at all times. */
+RD_API size_t rd_kv_materialize_plan_ints(int batch);
+RD_API int rd_kv_materialize(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
+                             int64_t row_bytes, int64_t length, int32_t* kv_row_shift,
+                             int32_t* plan, void* stream);
 RD_API int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
                          int64_t row_bytes, int64_t prev, int length, const int32_t* plan,
                          void* stream);
@@ -229,6 +244,8 @@ RD_API int rd_silu_add(const void* x, int64_t x_row_stride, const void* z, int64
  * batch row b is row row_start[b] + t of q, k, v and q_out (token stride; the batch strides are
  * unused) and exists only for t < row_start[b+1] - row_start[b]; position_ids stay (batch, n_new);
  * the cache rows of the slots that do not exist are not written.
+ * kv_row_shift (batch int32 on the device, or NULL): token t of row b goes to cache row
+ * row0 + t - kv_row_shift[b] (see rd_realign_plan); a row outside [0, max_len) is not written.
  * ------------------------------------------------------------------------------------------ */
 RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k,
                           const int64_t* k_strides, const void* v, const int64_t* v_strides,
@@ -237,7 +254,7 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
                           const int64_t* position_ids, int64_t pos_batch_stride, void* q_out,
                           const int64_t* q_out_strides, void* k_cache, void* v_cache,
                           const int64_t* cache_strides, int64_t row0, int64_t max_len,
-                          const int32_t* row_start, void* stream);
+                          const int32_t* row_start, const int32_t* kv_row_shift, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Verification attention.
@@ -266,12 +283,17 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
  * query t of batch row b is row row_start[b] + t of q and of out (sequence stride; their batch
  * strides are unused), queries t >= row_start[b+1] - row_start[b] are neither read nor written.
  * The mask bits keep their (batch, n_q) rows.
+ * kv_row_shift (rd_attn_prepare; batch int32 on the device, or NULL): recorded in the plan; the
+ * attention then reads key column c of row b from cache row c - kv_row_shift[b] of k and v (see
+ * rd_realign_plan).  Whole 64-key tiles are loaded, so up to 63 rows below a row's first key are
+ * touched: the caller keeps 64 rows of readable memory in front of the first slab.
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_attn_plan_ints(int batch, int n_q, int kv_len);
 RD_API size_t rd_attn_bits_words(int batch, int n_q, int kv_len);
 RD_API int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64_t mask_stride_q,
                            int batch, int n_q, int kv_len, int n_heads, int fix_empty_rows,
-                           uint64_t* bits, int32_t* plan, void* stream);
+                           uint64_t* bits, int32_t* plan, const int32_t* kv_row_shift,
+                           void* stream);
 RD_API size_t rd_attention_workspace_bytes(int batch, int n_heads, int n_q, int kv_len,
                                            int head_dim);
 RD_API int rd_verify_attention(const void* q, const int64_t* q_strides, const void* k,

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kThreads) void realign_plan_kernel(
     const int64_t* __restrict__ n_tokens_in_seq, const int64_t* __restrict__ seq_in_beam,
     const int64_t* __restrict__ beams, const int64_t* __restrict__ unpacker, int B, int W, int L,
     int64_t pad, const int32_t* __restrict__ pads, int32_t* __restrict__ plan,
-    int64_t* __restrict__ new_ids) {
+    int64_t* __restrict__ new_ids, int32_t* __restrict__ kv_shift) {
   const int b = blockIdx.x;
   int m = 0;
   for (int r = threadIdx.x; r < B; r += kThreads) {
@@ -158,12 +158,20 @@ __global__ __launch_bounds__(kThreads) void realign_plan_kernel(
   const int new_pads = m - live - n_new;
   const int s = clampi((int)seq_in_beam[b], 0, W - 1);
   int32_t* row_plan = plan + 4 + (int64_t)b * (4 + L);
+  // With kv_shift the cache rows stay where they are: token column c of this row lives in cache row
+  // c - kv_shift[b], the plan is written in cache rows (nothing moves, the accepted rows are appended
+  // behind the live ones) and the shift takes up the change of the left padding instead.
+  const int shift = kv_shift ? kv_shift[b] : 0;
   if (threadIdx.x == 0) {
     if (b == 0) { plan[0] = m; plan[1] = (int)prev; plan[2] = L; plan[3] = 0; }
-    row_plan[0] = old_pads; row_plan[1] = new_pads; row_plan[2] = n_new; row_plan[3] = live;
+    row_plan[0] = old_pads - shift;
+    row_plan[1] = (kv_shift ? old_pads : new_pads) - shift;
+    row_plan[2] = n_new; row_plan[3] = live;
   }
   for (int j = threadIdx.x; j < L; j += kThreads)
-    row_plan[4 + j] = (int)prev + (unpacker ? (int)unpacker[((int64_t)b * W + s) * L + j] : s * L + j);
+    row_plan[4 + j] = (int)prev - shift + (unpacker ? (int)unpacker[((int64_t)b * W + s) * L + j] : s * L + j);
+  __syncthreads();  // every thread has read the old shift
+  if (kv_shift && threadIdx.x == 0) kv_shift[b] = shift + new_pads - old_pads;
 
   int64_t* out = new_ids + (int64_t)b * m;
   const int64_t* in = ids + (int64_t)b * ids_row_stride;
@@ -235,7 +243,7 @@ extern "C" int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride,
                                const int64_t* n_tokens_in_seq, const int64_t* seq_in_beam,
                                const int64_t* beams, const int64_t* unpacker, int batch, int width,
                                int length, int64_t pad_token_id, int32_t* plan, int64_t* new_ids,
-                               void* stream) {
+                               int32_t* kv_row_shift, void* stream) {
   RD_REQUIRE(batch > 0 && width > 0 && length > 0 && prev >= 0, RD_EINVAL,
              "rd_realign_plan: bad sizes (batch %d width %d length %d prev %lld)", batch, width,
              length, (long long)prev);
@@ -250,7 +258,7 @@ extern "C" int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride,
   if (int e = rd::check_launch("rd_realign_plan(pads)")) return e;
   { rd::ScopedTiming rd_t("realign_plan_kernel", s); hipLaunchKernelGGL(realign_plan_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
                      ids_row_stride, prev, n_tokens_in_seq, seq_in_beam, beams, unpacker, batch,
-                     width, length, pad_token_id, pads, plan, new_ids); }
+                     width, length, pad_token_id, pads, plan, new_ids, kv_row_shift); }
   return rd::check_launch("rd_realign_plan");
 }
 

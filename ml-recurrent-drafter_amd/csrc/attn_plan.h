@@ -2,7 +2,9 @@
 //
 // plan (int32):
 //   [0] n_items  [1] n_q  [2] kv_len  [3] words per mask row  [4] max_splits  [5] chunk  [6..7] 0
-//   per batch row b, 4 ints at RD_PLAN_HDR + 4*b:  {kv_begin, n_splits, first_item, 0}
+//   per batch row b, 4 ints at RD_PLAN_HDR + 4*b:  {kv_begin, n_splits, first_item, kv_shift}
+//     (kv_shift: key column c of this row lives in cache row c - kv_shift; 0 unless the cache is
+//      kept in place when the token ids are re-aligned)
 //   items, 4 ints each at RD_PLAN_HDR + 4*batch:   {b, kv_lo, kv_hi, split}  (longest first)
 //   scratch: first attended key of every (b, q) row
 //   arrival counters, one per (b, head, query tile), zero between launches: the work items of a

@@ -49,6 +49,7 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
                                                              int B, int n_q, int kv_len, int words,
                                                              int min_chunk, int max_splits,
                                                              int n_heads, int n_cu,
+                                                             const int32_t* __restrict__ kv_shift,
                                                              int32_t* __restrict__ plan,
                                                              int32_t* __restrict__ counters,
                                                              int n_counters) {
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
     }
     if ((threadIdx.x & 63) == 0) {
       per_row[4 * b + 0] = (first / 64) * 64;
-      per_row[4 * b + 3] = 0;
+      per_row[4 * b + 3] = kv_shift ? kv_shift[b] : 0;  // cache row of key c is c - shift
     }
   }
   __syncthreads();
@@ -176,7 +177,8 @@ int compute_units() {
 
 extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64_t mask_stride_q,
                                int batch, int n_q, int kv_len, int n_heads, int fix_empty_rows,
-                               uint64_t* bits, int32_t* plan, void* stream) {
+                               uint64_t* bits, int32_t* plan, const int32_t* kv_row_shift,
+                               void* stream) {
   RD_REQUIRE(batch > 0 && n_q > 0 && kv_len > 0 && n_heads > 0, RD_EINVAL,
              "rd_attn_prepare: bad sizes (batch %d n_q %d kv_len %d n_heads %d)", batch, n_q, kv_len,
              n_heads);
@@ -193,7 +195,7 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
                      mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first); }
   if (int e = rd::check_launch("rd_attn_prepare(bits)")) return e;
   { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 0, s, row_first, batch, n_q, kv_len,
-                     words, rd::kAttnChunk, max_splits, n_heads, compute_units(), plan,
+                     words, rd::kAttnChunk, max_splits, n_heads, compute_units(), kv_row_shift, plan,
                      plan + rd::attn_counter_offset(batch, n_q, kv_len), (int)rd::attn_counter_ints(batch, n_q)); }
   return rd::check_launch("rd_attn_prepare(plan)");
 }

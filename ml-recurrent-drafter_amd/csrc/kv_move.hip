@@ -119,6 +119,24 @@ __global__ __launch_bounds__(kThreads) void kv_compact_kernel(
   for (int v = threadIdx.x; v < n_new * vpr; v += kThreads) tail[v] = s_acc[v];
 }
 
+// Plan that moves every row of the cache from where it physically is (token column c in cache row
+// c - shift[b]) to the layout in which column and cache row agree; the shifts are cleared.
+__global__ void materialize_plan_kernel(int32_t* __restrict__ shift, int B, int64_t length,
+                                        int64_t max_len, int32_t* __restrict__ plan) {
+  for (int b = threadIdx.x; b < B; b += blockDim.x) {
+    const int64_t s = shift[b];
+    int64_t p0 = s < 0 ? -s : 0;                 // first cache row whose column is not negative
+    int64_t p1 = length - s;                     // cache row of column `length`
+    p1 = p1 > max_len ? max_len : p1;
+    if (p1 + s > max_len) p1 = max_len - s;
+    const int64_t live = p1 > p0 ? p1 - p0 : 0;
+    int32_t* rp = plan + 4 + (int64_t)b * 5;
+    rp[0] = (int32_t)p0; rp[1] = (int32_t)(p0 + s); rp[2] = 0; rp[3] = (int32_t)live; rp[4] = 0;
+    shift[b] = 0;
+  }
+  if (threadIdx.x == 0) { plan[0] = (int32_t)length; plan[1] = (int32_t)length; plan[2] = 1; plan[3] = 0; }
+}
+
 int check_cache_args(const char* who, const void* cache, int n_layers, int B, int H,
                      int64_t max_len, int64_t row_bytes) {
   RD_REQUIRE(cache, RD_EINVAL, "%s: null cache", who);
@@ -205,4 +223,24 @@ extern "C" int rd_kv_compact(void* cache, int n_layers, int batch, int n_heads, 
   { rd::ScopedTiming rd_t("kv_compact_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(kv_compact_kernel, dim3(slabs), dim3(kThreads), lds, rd::as_stream(stream),
                      reinterpret_cast<char*>(cache), batch, n_heads, max_len, row_bytes, plan, length); }
   return rd::check_launch("rd_kv_compact");
+}
+
+extern "C" size_t rd_kv_materialize_plan_ints(int batch) { return batch > 0 ? 4 + (size_t)batch * 5 : 0; }
+
+extern "C" int rd_kv_materialize(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
+                                 int64_t row_bytes, int64_t length, int32_t* kv_row_shift,
+                                 int32_t* plan, void* stream) {
+  if (int e = check_cache_args("rd_kv_materialize", cache, n_layers, batch, n_heads, max_len, row_bytes))
+    return e;
+  RD_REQUIRE(kv_row_shift && plan && length >= 0 && length <= max_len, RD_EINVAL,
+             "rd_kv_materialize: null pointer or length %lld outside [0, %lld]", (long long)length,
+             (long long)max_len);
+  RD_REQUIRE(row_bytes <= 64 * 1024, RD_ELIMIT, "rd_kv_materialize: row_bytes %lld > 65536", (long long)row_bytes);
+  hipStream_t s = rd::as_stream(stream);
+  hipLaunchKernelGGL(materialize_plan_kernel, dim3(1), dim3(kThreads), 0, s, kv_row_shift, batch, length, max_len, plan);
+  if (int e = rd::check_launch("rd_kv_materialize(plan)")) return e;
+  const int64_t slabs = (int64_t)n_layers * 2 * batch * n_heads;
+  { rd::ScopedTiming rd_t("kv_compact_kernel", s); hipLaunchKernelGGL(kv_compact_kernel, dim3(slabs), dim3(kThreads), (size_t)row_bytes, s,
+                     reinterpret_cast<char*>(cache), batch, n_heads, max_len, row_bytes, plan, 1); }
+  return rd::check_launch("rd_kv_materialize");
 }

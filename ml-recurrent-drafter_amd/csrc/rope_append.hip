@@ -64,7 +64,10 @@ struct RopeArgs {
   void* q_out; int64_t qo_sb, qo_st;            // (B, n, heads, D); may be q itself
   void* k_cache; void* v_cache;                 // (B, kv_heads, max_len, D)
   int64_t c_sb, c_sh, c_st;
-  int64_t row0;                                 // first cache row written
+  int64_t row0;                                 // first cache row written (before the row's shift)
+  int64_t max_len;
+  // Per batch row (or null): token column c of row b lives in cache row c - kv_shift[b].
+  const int32_t* kv_shift;
   // Packed token rows (or null): token t of batch row b is row row_start[b] + t of q, k, v and
   // q_out (their batch strides are unused) and exists only for t < row_start[b+1] - row_start[b];
   // the cache rows of tokens that do not exist are left as they are.
@@ -99,10 +102,15 @@ __global__ __launch_bounds__(kThreads) void rope_append_kernel(RopeArgs a) {
   const T* k_tok = reinterpret_cast<const T*>(a.k) + in_batch * a.k_sb + tok * a.k_st;
   const T* v_tok = reinterpret_cast<const T*>(a.v) + in_batch * a.v_sb + tok * a.v_st;
   T* qo_tok = reinterpret_cast<T*>(a.q_out) + in_batch * a.qo_sb + tok * a.qo_st;
-  T* kc = reinterpret_cast<T*>(a.k_cache) + b * a.c_sb + (a.row0 + t) * a.c_st;
-  T* vc = reinterpret_cast<T*>(a.v_cache) + b * a.c_sb + (a.row0 + t) * a.c_st;
+  int64_t cache_row = a.row0 + t - (a.kv_shift ? a.kv_shift[b] : 0);
+  // a shift that leaves the slab is never followed: q is still rotated, k and v are dropped
+  const bool in_cache = cache_row >= 0 && cache_row < a.max_len;
+  cache_row = in_cache ? cache_row : 0;
+  T* kc = reinterpret_cast<T*>(a.k_cache) + b * a.c_sb + cache_row * a.c_st;
+  T* vc = reinterpret_cast<T*>(a.v_cache) + b * a.c_sb + cache_row * a.c_st;
+  const int n_tasks = in_cache ? q_tasks + k_tasks + v_tasks : q_tasks;
 
-  for (int task = threadIdx.x; task < q_tasks + k_tasks + v_tasks; task += kThreads) {
+  for (int task = threadIdx.x; task < n_tasks; task += kThreads) {
     if (task >= q_tasks + k_tasks) {
       const int c = task - q_tasks - k_tasks;
       const int h = c / (D / N), d = (c % (D / N)) * N;
@@ -144,7 +152,7 @@ extern "C" int rd_rope_append(const void* q, const int64_t* q_strides, const voi
                               const int64_t* position_ids, int64_t pos_batch_stride, void* q_out,
                               const int64_t* q_out_strides, void* k_cache, void* v_cache,
                               const int64_t* cache_strides, int64_t row0, int64_t max_len,
-                              const int32_t* row_start, void* stream) {
+                              const int32_t* row_start, const int32_t* kv_row_shift, void* stream) {
   RD_REQUIRE(batch > 0 && n_new > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0, RD_EINVAL,
              "rd_rope_append: bad sizes (batch %d n_new %d heads %d kv_heads %d head_dim %d)", batch, n_new,
              n_heads, n_kv_heads, head_dim);
@@ -177,6 +185,8 @@ extern "C" int rd_rope_append(const void* q, const int64_t* q_strides, const voi
   a.k_cache = k_cache; a.v_cache = v_cache;
   a.c_sb = cache_strides[0]; a.c_sh = cache_strides[1]; a.c_st = cache_strides[2];
   a.row0 = row0;
+  a.max_len = max_len;
+  a.kv_shift = kv_row_shift;
   a.row_start = row_start;
   a.n_new = n_new; a.n_heads = n_heads; a.n_kv_heads = n_kv_heads; a.head_dim = head_dim;
   hipStream_t s = rd::as_stream(stream);

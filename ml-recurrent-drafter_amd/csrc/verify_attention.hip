@@ -152,6 +152,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   asm volatile("" ::"s"(a.v), "s"(a.v_sb), "s"(a.v_sh), "s"(a.v_ss), "s"(a.bits), "s"(a.n_q), "s"(a.kv_len), "s"(a.words));
   if (item >= n_items) return;
   const int n_splits = a.plan[RD_PLAN_HDR + 4 * b + 1];
+  const int kv_shift = a.plan[RD_PLAN_HDR + 4 * b + 3];  // key column c is cache row c - kv_shift
   // query tiles of one (row, head, key range) are neighbours in dispatch order, so they run
   // together and the second read of the K/V tiles is served by the L2
   const int q_tiles = gridDim.x / a.H;
@@ -170,8 +171,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const bool wave_active = q_tile * kRowsPerWG + row_wave * 32 < rows.n;
   const bool row_valid = q_row < rows.n;
 
-  const __bf16* kbase = reinterpret_cast<const __bf16*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh;
-  const __bf16* vbase = reinterpret_cast<const __bf16*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh;
+  const __bf16* kbase = reinterpret_cast<const __bf16*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh - (int64_t)kv_shift * a.k_ss;
+  const __bf16* vbase = reinterpret_cast<const __bf16*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh - (int64_t)kv_shift * a.v_ss;
 
   // Q fragments: B operand of S^T = K Q^T; lane (r,g) holds Q[q_row][16*ks + 8*g .. +8)
   bf16x8 qf[8];
@@ -639,8 +640,9 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
   const RowSpan rows = row_span(a, b);
   if (q >= rows.n) return;
   const T* qp = reinterpret_cast<const T*>(a.q) + rows.q_off + (int64_t)h * a.q_sh + (int64_t)q * a.q_ss;
-  const T* kb = reinterpret_cast<const T*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh;
-  const T* vb = reinterpret_cast<const T*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh;
+  const int kv_shift = a.plan[RD_PLAN_HDR + 4 * b + 3];
+  const T* kb = reinterpret_cast<const T*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh - (int64_t)kv_shift * a.k_ss;
+  const T* vb = reinterpret_cast<const T*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh - (int64_t)kv_shift * a.v_ss;
   if (tid < D) s_q[tid] = ld<T>(qp + tid) * a.scale;
   __syncthreads();
   const uint64_t* brow = a.bits + ((int64_t)b * a.n_q + q) * a.words;

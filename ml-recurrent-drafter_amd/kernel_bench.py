@@ -187,6 +187,19 @@ def case_kv(rows, reps):
         moved = sum((t + 1) for t in n_tok) + sum(prev for t in n_tok if m - (t + 1) != 0)
         report(rows, f"realign + kv_compact prev {prev}, {label}", k, {"kv_compact_kernel": 2 * row * moved},
                {"kv_compact_kernel": "GB/s"})
+    # the same re-alignment with the cache rows kept in place (what the decode loop does): only the
+    # accepted rows are copied, the change of the left padding goes into the per-row shift
+    cache.rows_in_place = True
+
+    def compact_in_place():
+        cache.set_length(prev + n)
+        cache.shift.zero_()
+        acceptance.realign(ids, nt, sb, beams, cache, 0, unpacker=tree.unpacker)
+
+    k = timed(compact_in_place, reps)
+    k.pop("vectorized_elementwise_kernel", None)
+    report(rows, f"realign + kv_compact prev {prev}, 7 of 8 rows shift, cache rows kept in place", k,
+           {"kv_compact_kernel": 2 * row * sum((t + 1) for t in n_tok)}, {"kv_compact_kernel": "GB/s"})
 
 
 def case_rope(rows, reps):

@@ -35,19 +35,21 @@ _PROTOTYPES = {
     "rd_accept_greedy": (_I, [_P, _P, _L, _P, _I, _I, _I, _P, _P, _P, _P, _P]),
     "rd_count_left_paddings": (_I, [_P, _L, _L, _I, _L, _P, _P]),
     "rd_realign_plan_ints": (_Z, [_I, _I]),
-    "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P]),
+    "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P, _P]),
     "rd_kv_unpack": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _I, _I, _P]),
     "rd_kv_compact": (_I, [_P, _I, _I, _I, _L, _L, _L, _I, _P, _P]),
+    "rd_kv_materialize_plan_ints": (_Z, [_I]),
+    "rd_kv_materialize": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _P, _P]),
     "rd_add_rms_norm": (_I, [_P, _L, _P, _L, _P, _P, _L, _P, _L, _I, _L, _I, _F, _P]),
     "rd_silu_mul": (_I, [_P, _P, _L, _P, _L, _I, _L, _I, _P]),
     "rd_silu_add": (_I, [_P, _L, _P, _L, _P, _L, _P, _L, _I, _I, _L, _I, _P]),
     "rd_rope_append": (
         _I,
-        [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _L, _P, _P],
+        [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _L, _P, _P, _P],
     ),
     "rd_attn_plan_ints": (_Z, [_I, _I, _I]),
     "rd_attn_bits_words": (_Z, [_I, _I, _I]),
-    "rd_attn_prepare": (_I, [_P, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P]),
+    "rd_attn_prepare": (_I, [_P, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P]),
     "rd_attention_workspace_bytes": (_Z, [_I, _I, _I, _I, _I]),
     "rd_verify_attention": (
         _I,

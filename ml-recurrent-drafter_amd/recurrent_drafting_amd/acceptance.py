@@ -157,9 +157,12 @@ def realign_enqueue(
         lib.rd_realign_plan(
             _hip.ptr(input_ids) if prev > 0 else None, input_ids.stride(0), prev,
             _hip.ptr(n_tokens_in_seq), _hip.ptr(seq_in_beam), _hip.ptr(beams), _hip.ptr(unpacker),
-            B, W, L, pad_token_id, _hip.ptr(plan), _hip.ptr(ids_buf), _hip.stream(),
+            B, W, L, pad_token_id, _hip.ptr(plan), _hip.ptr(ids_buf),
+            _hip.ptr(cache.shift) if cache.rows_in_place else None, _hip.stream(),
         )
     )
+    if cache.rows_in_place:
+        cache._shifted = True
     _hip.check(
         lib.rd_kv_compact(
             _hip.ptr(cache._cache), *cache._geometry()[:4], cache._geometry()[4], prev, L,

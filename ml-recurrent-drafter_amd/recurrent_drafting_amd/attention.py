@@ -62,13 +62,16 @@ class PreparedMask:
     workspace: Optional[torch.Tensor] = None
 
 
-def prepare(mask: torch.Tensor, fix_empty_rows: bool = True, n_heads: int = 32) -> PreparedMask:
+def prepare(mask: torch.Tensor, fix_empty_rows: bool = True, n_heads: int = 32,
+            kv_shift: Optional[torch.Tensor] = None) -> PreparedMask:
     """mask: (B, n_q, kv_len) bool/uint8, keys contiguous.  n_heads: query heads of the attention
-    calls that will use the result (only sizes the work items)."""
+    calls that will use the result (only sizes the work items).  kv_shift: (B,) int32 or None; key
+    column c of row b is then read from row c - kv_shift[b] of k and v (kv_cache.Cache.shift)."""
     assert mask.dim() == 3 and mask.dtype in (torch.bool, torch.uint8)
     if mask.stride(2) != 1:
         mask = mask.contiguous()
     B, n_q, kv_len = mask.shape
+    assert kv_shift is None or (kv_shift.shape == (B,) and kv_shift.dtype == torch.int32 and kv_shift.is_contiguous())
     lib = _hip.lib()
     dev = mask.device
     bits = torch.empty(lib.rd_attn_bits_words(B, n_q, kv_len), dtype=torch.int64, device=dev)
@@ -77,7 +80,7 @@ def prepare(mask: torch.Tensor, fix_empty_rows: bool = True, n_heads: int = 32) 
         lib.rd_attn_prepare(
             _hip.ptr(mask), mask.stride(0), mask.stride(1), B, n_q, kv_len, int(n_heads),
             int(fix_empty_rows),
-            _hip.ptr(bits), _hip.ptr(plan), _hip.stream(),
+            _hip.ptr(bits), _hip.ptr(plan), _hip.ptr(kv_shift), _hip.stream(),
         )
     )
     return PreparedMask(bits.view(B, n_q, -1), plan, B, n_q, kv_len)

@@ -3,6 +3,13 @@
 One dense tensor (n_layers, 2, batch, n_heads, max_length, head_dim) lives in HBM for the whole
 generation; `View.cat` appends in place and hands back a strided view, `Cache.unpack` and
 `Cache.compact` move rows with the HIP kernels rd_kv_unpack / rd_kv_compact (in place, no clone).
+
+Rows in place: the reference re-right-aligns the whole live cache after every step
+(recurrent_drafting.py:200-209).  With `Cache.rows_in_place = True` (the decode loop of
+`RecurrentDrafting` sets it) the cache rows never move: a per-row `Cache.shift` says that token
+column c of row b lives in cache row c - shift[b]; the re-alignment adds the change of the left
+padding to it, and `rope_append` and the attention subtract it.  `Cache.materialize()` moves the rows
+once to the reference's layout; `View.cat`, `View.slice` and `Cache.unpack` call it first.
 """
 
 from __future__ import annotations
@@ -19,10 +26,11 @@ from .packed_rows import PackedRows
 class View:
     """Key or value rows of one layer: cache[layer, kv, :, :, 0:length, :] (kv_cache.py:10-35)."""
 
-    def __init__(self, cache: torch.Tensor, layer: int, kv: int):
+    def __init__(self, cache: torch.Tensor, layer: int, kv: int, owner: Optional["Cache"] = None):
         self._cache = cache
         self._layer = layer
         self._kv = kv  # 0 = key, 1 = value
+        self._owner = owner
         self.length = 0
 
     @property
@@ -36,6 +44,8 @@ class View:
         n_new = new_kv.shape[2]
         assert new_kv.shape == (batch_size, n_heads, n_new, head_dim)
         assert self.length + n_new <= max_length
+        if self._owner is not None:
+            self._owner.materialize()
         slab = self._cache[self._layer, self._kv]
         slab[:, :, self.length : self.length + n_new, :] = new_kv
         self.length += n_new
@@ -43,6 +53,8 @@ class View:
 
     def slice(self, prev: int) -> torch.Tensor:
         """Rows [prev, length)."""
+        if self._owner is not None:
+            self._owner.materialize()
         return self._cache[self._layer, self._kv, :, :, prev : self.length, :]
 
 
@@ -83,6 +95,8 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
     assert value_view._cache is cache and key_view._layer == value_view._layer
     k_slab = cache[key_view._layer, 0]
     v_slab = cache[key_view._layer, 1]
+    owner = key_view._owner
+    shift = owner.shift if owner is not None and owner.rows_in_place else None
     _hip.check(
         _hip.lib().rd_rope_append(
             _hip.ptr(q), strides(q), _hip.ptr(k), strides(k), _hip.ptr(v), strides(v),
@@ -90,7 +104,7 @@ def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Te
             n_kv_heads, head_dim, _hip.ptr(cos), _hip.ptr(sin), cos.shape[0], _hip.ptr(position_ids),
             position_ids.stride(0), _hip.ptr(q), strides(q), _hip.ptr(k_slab), _hip.ptr(v_slab),
             (ctypes.c_int64 * 3)(k_slab.stride(0), k_slab.stride(1), k_slab.stride(2)), key_view.length,
-            max_length, _hip.ptr(rows.row_start) if rows is not None else None, _hip.stream(),
+            max_length, _hip.ptr(rows.row_start) if rows is not None else None, _hip.ptr(shift), _hip.stream(),
         )
     )
     key_view.length += n_new
@@ -113,17 +127,43 @@ class Cache:
         dtype: torch.dtype,
         device: torch.device,
     ) -> None:
-        self._cache = torch.zeros(
-            [n_layers, 2, batch_size, n_heads, max_length, head_dim], dtype=dtype, device=device
-        )
+        # 64 rows of readable memory in front of the first slab: with rows in place the attention
+        # loads whole 64-key tiles and the first tile of a row may begin below the row's first key
+        shape = [n_layers, 2, batch_size, n_heads, max_length, head_dim]
+        numel = 1
+        for d in shape:
+            numel *= d
+        guard = 64 * head_dim
+        self._storage = torch.zeros(guard + numel, dtype=dtype, device=device)
+        self._cache = self._storage[guard:].view(shape)
         self.sliced = tuple(
-            (View(self._cache, layer, 0), View(self._cache, layer, 1)) for layer in range(n_layers)
+            (View(self._cache, layer, 0, self), View(self._cache, layer, 1, self)) for layer in range(n_layers)
         )
+        # token column c of batch row b lives in cache row c - shift[b] (all zero: the reference's layout)
+        self.shift = torch.zeros(batch_size, dtype=torch.int32, device=device)
+        self.rows_in_place = False
+        self._shifted = False  # host-side: a re-alignment may have left non-zero shifts
 
     # -- geometry handed to the C ABI ---------------------------------------------------------
     def _geometry(self):
         n_layers, _, batch, n_heads, max_len, head_dim = self._cache.shape
         return n_layers, batch, n_heads, max_len, head_dim * self._cache.element_size()
+
+    def materialize(self) -> None:
+        """Moves the rows to the layout in which column and cache row agree (no-op unless a
+        re-alignment with rows in place has happened since the last call)."""
+        if not self._shifted:
+            return
+        n_layers, batch, n_heads, max_len, row_bytes = self._geometry()
+        lib = _hip.lib()
+        plan = torch.empty(lib.rd_kv_materialize_plan_ints(batch), dtype=torch.int32, device=self._cache.device)
+        _hip.check(
+            lib.rd_kv_materialize(
+                _hip.ptr(self._cache), n_layers, batch, n_heads, max_len, row_bytes,
+                self.sliced[0][0].length, _hip.ptr(self.shift), _hip.ptr(plan), _hip.stream(),
+            )
+        )
+        self._shifted = False
 
     def set_length(self, length: int) -> None:
         for key, value in self.sliced:
@@ -136,6 +176,7 @@ class Cache:
         batch, width, length = tree_attn_index.shape
         n_layers, cb, n_heads, max_len, row_bytes = self._geometry()
         assert cb == batch
+        self.materialize()
         n_out = width * length
         n_src = self.sliced[0][0].length - prompt_length
         assert n_src > 0, "no packed rows behind the prompt"

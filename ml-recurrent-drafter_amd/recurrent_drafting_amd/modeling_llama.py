@@ -235,7 +235,8 @@ class LlamaModel(LlamaPreTrainedModel):
         (rows.rows, hidden); input_ids, attention_mask and position_ids keep their (B, q) shapes."""
         if not isinstance(attention_mask, attention.PreparedMask):
             attention_mask = attention.prepare(
-                attention_mask, fix_empty_rows=False, n_heads=self.config.num_attention_heads)
+                attention_mask, fix_empty_rows=False, n_heads=self.config.num_attention_heads,
+                kv_shift=_kv_shift(past_key_values))
         if rows is not None:
             input_ids = rows.take(input_ids)
         hidden_states, delta = self.embed_tokens(input_ids), None
@@ -243,6 +244,12 @@ class LlamaModel(LlamaPreTrainedModel):
             hidden_states, delta = layer.forward_deferred(hidden_states, delta, position_ids, key_value,
                                                           attention_mask, rows)
         return self.norm(hidden_states, delta)
+
+
+def _kv_shift(past_key_values) -> Optional[torch.Tensor]:
+    """Per-row shift of the cache these views belong to, if its rows are kept in place."""
+    owner = past_key_values[0][0]._owner if len(past_key_values) else None
+    return owner.shift if owner is not None and owner.rows_in_place else None
 
 
 class LlamaForCausalLM(LlamaPreTrainedModel):
@@ -266,7 +273,8 @@ class LlamaForCausalLM(LlamaPreTrainedModel):
         exist; rows that attend to nothing attend to everything, as the reference arranges on a
         GPU (modeling_llama.py:264-265)."""
         prepared = attention.prepare(
-            attention_mask, fix_empty_rows=True, n_heads=self.config.num_attention_heads)
+            attention_mask, fix_empty_rows=True, n_heads=self.config.num_attention_heads,
+            kv_shift=_kv_shift(past_key_values))
         return self.model(input_ids=input_ids, attention_mask=prepared, position_ids=position_ids,
                           past_key_values=past_key_values, rows=rows)
 

@@ -145,6 +145,9 @@ class RecurrentDrafting(torch.nn.Module):
         self.llm = llm
         self.drafter = drafter
         gemm_tuning.load()  # kernel selection table for the dense layers' GEMMs (no-op without one)
+        # True: the decode loop leaves the KV cache rows where they are when the ids are re-aligned
+        # (kv_cache.Cache.rows_in_place); False: it moves them every step, as the reference does.
+        self.kv_rows_in_place = True
 
     def llm_n_kv_heads(self) -> int:
         if isinstance(self.llm, modeling_llama.LlamaForCausalLM):
@@ -243,9 +246,12 @@ class RecurrentDrafting(torch.nn.Module):
         batch_size, seq_len = input_ids.shape
         init_seq_len = seq_len
         cfg = self.llm.config
+        # The cache rows stay in place when the ids are re-aligned (kv_cache.Cache.rows_in_place): a row
+        # can then end up to its initial left padding further right than the ids do.
+        initial_pads = int(acceptance._count_left_paddings(input_ids, special_tokens.pad).max()) if seq_len else 0
         cache = kv_cache.Cache(
             batch_size=batch_size,
-            max_length=max_length + beam_shape.length * beam_shape.width,
+            max_length=max_length + beam_shape.length * beam_shape.width + initial_pads,
             n_layers=cfg.num_hidden_layers,
             n_heads=self.llm_n_kv_heads(),
             head_dim=cfg.hidden_size // cfg.num_attention_heads,
@@ -255,6 +261,7 @@ class RecurrentDrafting(torch.nn.Module):
         context, init_tokens = _comprehend_prompt(
             self.llm, input_ids, cache, sampling_args, special_tokens.pad
         )
+        cache.rows_in_place = self.kv_rows_in_place
         drafted, tree = None, None  # what has been drafted for the coming step
         while seq_len < max_length:
             with text_generation.step() as step_record:
