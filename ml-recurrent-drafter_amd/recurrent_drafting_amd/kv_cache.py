@@ -141,8 +141,19 @@ class Cache:
         )
         # token column c of batch row b lives in cache row c - shift[b] (all zero: the reference's layout)
         self.shift = torch.zeros(batch_size, dtype=torch.int32, device=device)
-        self.rows_in_place = False
+        self._rows_in_place = False
         self._shifted = False  # host-side: a re-alignment may have left non-zero shifts
+
+    @property
+    def rows_in_place(self) -> bool:
+        """True: re-alignments leave the cache rows where they are and update `shift` instead."""
+        return self._rows_in_place
+
+    @rows_in_place.setter
+    def rows_in_place(self, value: bool) -> None:
+        if not value:
+            self.materialize()  # nobody would follow the shifts any more
+        self._rows_in_place = bool(value)
 
     # -- geometry handed to the C ABI ---------------------------------------------------------
     def _geometry(self):

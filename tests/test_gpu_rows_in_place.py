@@ -28,8 +28,8 @@ def _pair(B, max_len, layers=2, heads=3, D=16, dtype=torch.float32):
     return a, b
 
 
-@pytest.mark.parametrize("seed", [0, 1, 2])
-def test_successive_realignments_then_materialize_equal_the_moved_cache(seed):
+@pytest.mark.parametrize("seed,switch_off", [(0, False), (1, False), (2, True)])
+def test_successive_realignments_then_materialize_equal_the_moved_cache(seed, switch_off):
     """Three re-alignments with random accepted lengths and ragged left padding; between them the
     tree rows of the next step are written through rope_append's cache rows (here: plain copies)."""
     from recurrent_drafting_amd import acceptance
@@ -63,7 +63,10 @@ def test_successive_realignments_then_materialize_equal_the_moved_cache(seed):
         assert torch.equal(ids_a, ids_b)
     assert in_place._shifted and in_place.shift.abs().sum() > 0, "the case never shifted a row"
     length = ids_a.shape[1]
-    in_place.materialize()
+    if switch_off:
+        in_place.rows_in_place = False  # switching the mode off brings the rows home first
+    else:
+        in_place.materialize()
     assert not in_place._shifted and int(in_place.shift.abs().sum()) == 0
     new_pads = (ids_a == 0).long().cumprod(1).sum(1).cpu().tolist()
     for r in range(B):
