@@ -184,6 +184,11 @@ RD_API int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride, int
 RD_API int rd_kv_unpack(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
                         int64_t row_bytes, int64_t prev, const int64_t* index, int n_out, int n_src,
                         void* stream);
+/* rd_kv_append: rd_kv_compact for plans in which no row moves (old_pads == new_pads for every row,
+ * as rd_realign_plan writes them when it is given kv_row_shift): only the accepted rows are copied
+ * behind the live ones.  length * row_bytes <= 4096. */
+RD_API int rd_kv_append(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
+                        int64_t row_bytes, int length, const int32_t* plan, void* stream);
 /* rd_kv_materialize: undoes kv_row_shift (see rd_realign_plan): every row's cache rows move to
  * the place where column and cache row agree (columns [0, length)), and the shifts are cleared.
  * plan: rd_kv_materialize_plan_ints(batch) int32 of workspace.  No counterpart in the reference,

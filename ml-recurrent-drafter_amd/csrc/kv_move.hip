@@ -119,6 +119,44 @@ __global__ __launch_bounds__(kThreads) void kv_compact_kernel(
   for (int v = threadIdx.x; v < n_new * vpr; v += kThreads) tail[v] = s_acc[v];
 }
 
+// The re-alignment when no row moves (plans written for rows kept in place: old_pads == new_pads):
+// only the accepted rows are copied behind the live ones.  Eight slabs per workgroup, 32 threads
+// each: one slab per workgroup is 16 384 workgroups of which most threads have nothing to do.
+constexpr int kAppendSlabs = 8, kAppendPer = 8;  // slabs per workgroup, vectors per thread
+
+__global__ __launch_bounds__(kThreads) void kv_append_kernel(
+    char* __restrict__ cache, int64_t slabs, int B, int H, int64_t max_len, int64_t row_bytes,
+    const int32_t* __restrict__ plan, int L) {
+  const int sub = threadIdx.x >> 5, lane = threadIdx.x & 31;
+  const int64_t slab = (int64_t)blockIdx.x * kAppendSlabs + sub;
+  const bool valid = slab < slabs;
+  const int b = valid ? (int)((slab / H) % B) : 0;
+  const int32_t* rp = plan + 4 + (int64_t)b * (4 + L);
+  const int start = rp[1], live = rp[3];
+  int n_new = rp[2];
+  if (!valid || start < 0 || live < 0 || n_new < 0 || n_new > L || (int64_t)start + live + n_new > max_len) n_new = 0;
+  char* base = cache + (valid ? slab : 0) * max_len * row_bytes;
+  const int vpr = (int)(row_bytes >> 4);
+  const int total = n_new * vpr;
+  vec16 r[kAppendPer];
+#pragma unroll
+  for (int u = 0; u < kAppendPer; ++u) {
+    int v = lane + 32 * u;
+    v = v < total ? v : 0;  // clamped, not skipped: keeps the array in registers
+    const int j = v / vpr, c = v - j * vpr;
+    int64_t row = total > 0 ? rp[4 + j] : 0;
+    row = (row < 0 || row >= max_len) ? 0 : row;
+    r[u] = *reinterpret_cast<const vec16*>(base + row * row_bytes + (c << 4));
+  }
+  __syncthreads();  // source and destination rows of a slab overlap: every read precedes every write
+  vec16* tail = reinterpret_cast<vec16*>(base + (int64_t)(start + live) * row_bytes);
+#pragma unroll
+  for (int u = 0; u < kAppendPer; ++u) {
+    const int v = lane + 32 * u;
+    if (v < total) tail[v] = r[u];
+  }
+}
+
 // Plan that moves every row of the cache from where it physically is (token column c in cache row
 // c - shift[b]) to the layout in which column and cache row agree; the shifts are cleared.
 __global__ void materialize_plan_kernel(int32_t* __restrict__ shift, int B, int64_t length,
@@ -243,4 +281,19 @@ extern "C" int rd_kv_materialize(void* cache, int n_layers, int batch, int n_hea
   { rd::ScopedTiming rd_t("kv_compact_kernel", s); hipLaunchKernelGGL(kv_compact_kernel, dim3(slabs), dim3(kThreads), (size_t)row_bytes, s,
                      reinterpret_cast<char*>(cache), batch, n_heads, max_len, row_bytes, plan, 1); }
   return rd::check_launch("rd_kv_materialize");
+}
+
+extern "C" int rd_kv_append(void* cache, int n_layers, int batch, int n_heads, int64_t max_len,
+                            int64_t row_bytes, int length, const int32_t* plan, void* stream) {
+  if (int e = check_cache_args("rd_kv_append", cache, n_layers, batch, n_heads, max_len, row_bytes))
+    return e;
+  RD_REQUIRE(plan && length > 0, RD_EINVAL, "rd_kv_append: null plan or length %d", length);
+  RD_REQUIRE((int64_t)length * (row_bytes >> 4) <= 32 * kAppendPer, RD_ELIMIT,
+             "rd_kv_append: length %d x row_bytes %lld is more than %d bytes per slab", length,
+             (long long)row_bytes, 32 * kAppendPer * 16);
+  const int64_t slabs = (int64_t)n_layers * 2 * batch * n_heads;
+  const int64_t grid = (slabs + kAppendSlabs - 1) / kAppendSlabs;
+  { rd::ScopedTiming rd_t("kv_append_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(kv_append_kernel, dim3((unsigned)grid), dim3(kThreads), 0, rd::as_stream(stream),
+                     reinterpret_cast<char*>(cache), slabs, batch, n_heads, max_len, row_bytes, plan, length); }
+  return rd::check_launch("rd_kv_append");
 }

@@ -38,6 +38,7 @@ _PROTOTYPES = {
     "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P, _P]),
     "rd_kv_unpack": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _I, _I, _P]),
     "rd_kv_compact": (_I, [_P, _I, _I, _I, _L, _L, _L, _I, _P, _P]),
+    "rd_kv_append": (_I, [_P, _I, _I, _I, _L, _L, _I, _P, _P]),
     "rd_kv_materialize_plan_ints": (_Z, [_I]),
     "rd_kv_materialize": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _P, _P]),
     "rd_add_rms_norm": (_I, [_P, _L, _P, _L, _P, _P, _L, _P, _L, _I, _L, _I, _F, _P]),

@@ -163,12 +163,22 @@ def realign_enqueue(
     )
     if cache.rows_in_place:
         cache._shifted = True
-    _hip.check(
-        lib.rd_kv_compact(
-            _hip.ptr(cache._cache), *cache._geometry()[:4], cache._geometry()[4], prev, L,
-            _hip.ptr(plan), _hip.stream(),
+    n_layers, batch, n_heads, max_len, row_bytes = cache._geometry()
+    if cache.rows_in_place and L * (row_bytes // 16) <= 256:
+        # no row moves: the accepted rows are appended behind the live ones
+        _hip.check(
+            lib.rd_kv_append(
+                _hip.ptr(cache._cache), n_layers, batch, n_heads, max_len, row_bytes, L,
+                _hip.ptr(plan), _hip.stream(),
+            )
         )
-    )
+    else:
+        _hip.check(
+            lib.rd_kv_compact(
+                _hip.ptr(cache._cache), n_layers, batch, n_heads, max_len, row_bytes, prev, L,
+                _hip.ptr(plan), _hip.stream(),
+            )
+        )
     return PendingRealign(ids_buf, plan, cache, B)
 
 
