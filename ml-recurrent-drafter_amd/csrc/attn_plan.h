@@ -5,7 +5,7 @@
 //   per batch row b, 4 ints at RD_PLAN_HDR + 4*b:  {kv_begin, n_splits, first_item, kv_shift}
 //     (kv_shift: key column c of this row lives in cache row c - kv_shift; 0 unless the cache is
 //      kept in place when the token ids are re-aligned)
-//   items, 4 ints each at RD_PLAN_HDR + 4*batch:   {b, kv_lo, kv_hi, split}  (longest first)
+//   items, 4 ints each at RD_PLAN_HDR + 4*batch:   {b, kv_lo, kv_hi, split | kv_shift << 12}  (longest first)
 //   scratch: first attended key of every (b, q) row
 //   arrival counters, one per (b, head, query tile), zero between launches: the work items of a
 //   split row count themselves in, and the last one to arrive merges the partials of all

@@ -145,7 +145,9 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
     items[4 * rank + 0] = b;
     items[4 * rank + 1] = lo;
     items[4 * rank + 2] = hi;
-    items[4 * rank + 3] = s;
+    // split index in the low 12 bits, the row's cache shift above them: the attention kernel then
+    // has everything it needs for its first loads from this one record
+    items[4 * rank + 3] = (s & 0xfff) | (per_row[4 * b + 3] * 4096);
   }
 }
 
@@ -185,6 +187,8 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
   RD_REQUIRE(batch <= 65535 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
              "rd_attn_prepare: batch %d too large for kv_len %d", batch, kv_len);
   RD_REQUIRE(mask && bits && plan, RD_EINVAL, "rd_attn_prepare: null pointer");
+  RD_REQUIRE(rd::attn_max_splits(kv_len) <= 4095 && (!kv_row_shift || kv_len < (1 << 19)), RD_ELIMIT,
+             "rd_attn_prepare: kv_len %d is beyond what a work item record can describe", kv_len);
   RD_REQUIRE(mask_stride_q >= kv_len && mask_stride_b >= 0, RD_EINVAL,
              "rd_attn_prepare: mask_stride_q %lld < kv_len %d", (long long)mask_stride_q, kv_len);
   const int words = (kv_len + 63) / 64;

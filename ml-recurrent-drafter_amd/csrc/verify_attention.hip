@@ -146,13 +146,14 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const int item = blockIdx.y;
   const int32_t* it = a.plan + RD_PLAN_HDR + 4 * a.B + 4 * item;
   const int n_items = a.plan[0];
-  int b = it[0], lo = it[1], hi = it[2], split = it[3];
+  int b = it[0], lo = it[1], hi = it[2], split = it[3];  // (split: with the row's cache shift above bit 12)
   asm volatile("" : "+s"(b), "+s"(lo), "+s"(hi), "+s"(split));
   asm volatile("" ::"s"(a.q), "s"(a.q_sb), "s"(a.q_sh), "s"(a.q_ss), "s"(a.k), "s"(a.k_sb), "s"(a.k_sh), "s"(a.k_ss));
   asm volatile("" ::"s"(a.v), "s"(a.v_sb), "s"(a.v_sh), "s"(a.v_ss), "s"(a.bits), "s"(a.n_q), "s"(a.kv_len), "s"(a.words));
   if (item >= n_items) return;
+  const int kv_shift = split >> 12;  // key column c of this row is cache row c - kv_shift
+  split &= 0xfff;
   const int n_splits = a.plan[RD_PLAN_HDR + 4 * b + 1];
-  const int kv_shift = a.plan[RD_PLAN_HDR + 4 * b + 3];  // key column c is cache row c - kv_shift
   // query tiles of one (row, head, key range) are neighbours in dispatch order, so they run
   // together and the second read of the K/V tiles is served by the L2
   const int q_tiles = gridDim.x / a.H;

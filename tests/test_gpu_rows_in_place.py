@@ -75,14 +75,15 @@ def test_successive_realignments_then_materialize_equal_the_moved_cache(seed, sw
         assert torch.equal(got, want), f"row {r}"
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_attention_and_rope_append_follow_the_shift(dtype):
+@pytest.mark.parametrize("dtype,prev", [(torch.float32, 70), (torch.bfloat16, 70), (torch.bfloat16, 1400)])
+def test_attention_and_rope_append_follow_the_shift(dtype, prev):
     """rope_append writes and the attention reads cache row c - shift[b]: same output as the same
-    data laid out without a shift."""
+    data laid out without a shift.  (1400 cached keys: the rows are cut into several work items, so
+    the shift also travels with split rows and their merge.)"""
     from recurrent_drafting_amd import attention, kv_cache
 
     torch.manual_seed(3)
-    B, H, D, prev, n = 3, 4, 128, 70, 9
+    B, H, D, n = 3, 4, 128, 9
     max_len = prev + n + 40
     shift = torch.tensor([5, 0, -3], dtype=torch.int32, device="cuda")  # row 2 sits 3 rows further right
     plain = kv_cache.Cache(B, max_len, 1, H, D, dtype, torch.device("cuda"))
@@ -112,6 +113,8 @@ def test_attention_and_rope_append_follow_the_shift(dtype):
         qq, keys, values = kv_cache.rope_append(q.clone(), k, v, cos, sin, pos, cache.sliced[0])
         prepared = attention.prepare(mask, n_heads=H, kv_shift=cache.shift if cache.rows_in_place else None)
         outs.append(attention.masked_attention(qq, keys, values, prepared))
+        if prev > 1000:
+            assert int(prepared.plan[0]) > B, "the rows were not split"
     assert torch.equal(outs[0], outs[1])
     shifted.materialize()
     for b in range(B):
