@@ -115,7 +115,16 @@ def ptr(t: torch.Tensor | None):
     return t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def stream():
+    """Handle of torch's current stream on the current device.  Every launch asks for it, so the two
+    direct calls are used where this torch build has them (a few tenths of a microsecond against
+    about three for `torch.cuda.current_stream()`)."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
