@@ -42,6 +42,12 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
 
 def _count_left_paddings(tokens: torch.Tensor, pad_token_id: int) -> torch.Tensor:
     """Leading run of pad ids per row, int64 (B,) (recurrent_drafting.py:387-388)."""
+    return _count_left_paddings_int32(tokens, pad_token_id).to(torch.long)
+
+
+def _count_left_paddings_int32(tokens: torch.Tensor, pad_token_id: int) -> torch.Tensor:
+    """The same counts as the kernel leaves them (int32): one launch less for callers that only do
+    arithmetic with them."""
     assert tokens.dim() == 2 and tokens.dtype == torch.long
     if tokens.shape[1] > 0 and tokens.stride(1) != 1:
         tokens = tokens.contiguous()
@@ -53,7 +59,7 @@ def _count_left_paddings(tokens: torch.Tensor, pad_token_id: int) -> torch.Tenso
             _hip.ptr(pads), _hip.stream(),
         )
     )
-    return pads.to(torch.long)
+    return pads
 
 
 def greedy_accept(
