@@ -76,15 +76,17 @@ RD_API int rd_timing_collect(char* out, size_t out_bytes);
  * the slots that exist, listed row after row without the padding -- row_start[b] = number of
  * slots of the rows before b (row_start[batch] = total), row_slots[row_start[b] + t] = b*max_n + t
  * for t < counts[b]; the entries from total up to the next multiple of 32 (or the capacity) are 0,
- * so that a caller may round its row count up.  (No counterpart in the reference, which runs the
- * model on the padding too.)
+ * so that a caller may round its row count up.  row_tokens (int64, same capacity, optional): the
+ * token of each of those slots in the same order, zeros in the rounding entries.  (No counterpart
+ * in the reference, which runs the model on the padding too.)
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_tree_workspace_bytes(int batch, int width, int length);
 RD_API int rd_tree_build(const int64_t* beams, int batch, int width, int length,
                   int64_t* prefix_tree, int64_t* unpacker,
                   int64_t* packed_tokens, int64_t* packed_token_indices,
                   int64_t* position_offsets, int32_t* counts, int32_t* row_start,
-                  int64_t* row_slots, void* workspace, size_t workspace_bytes, void* stream);
+                  int64_t* row_slots, int64_t* row_tokens, void* workspace, size_t workspace_bytes,
+                  void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Tree attention mask, rows of the packed tokens only.

@@ -85,7 +85,8 @@ __global__ __launch_bounds__(kThreads) void tree_fill_kernel(
     const int64_t* __restrict__ sel_tok, const int32_t* __restrict__ sel_idx, int B, int WL, int L,
     int32_t* __restrict__ counts, int64_t* __restrict__ packed_tokens,
     int64_t* __restrict__ packed_token_indices, int64_t* __restrict__ position_offsets,
-    int32_t* __restrict__ row_start, int64_t* __restrict__ row_slots) {
+    int32_t* __restrict__ row_start, int64_t* __restrict__ row_slots,
+    int64_t* __restrict__ row_tokens) {
   __shared__ int s_red[3][kThreads / 64];
   const int b = blockIdx.x;
   int before = 0, total = 0, mx = 0;
@@ -129,6 +130,16 @@ __global__ __launch_bounds__(kThreads) void tree_fill_kernel(
       int64_t end = ((int64_t)total + kRowSlotsPad - 1) / kRowSlotsPad * kRowSlotsPad;
       end = end < cap ? end : cap;
       for (int64_t n = total + threadIdx.x; n < end; n += kThreads) row_slots[n] = 0;
+    }
+  }
+  // and their tokens in the same order (what the embedding lookup of the packed rows needs)
+  if (row_tokens != nullptr) {
+    for (int n = threadIdx.x; n < counts[b]; n += kThreads) row_tokens[before + n] = sel_tok[(int64_t)b * WL + n];
+    if (b == 0) {
+      const int64_t cap = (int64_t)B * WL;
+      int64_t end = ((int64_t)total + kRowSlotsPad - 1) / kRowSlotsPad * kRowSlotsPad;
+      end = end < cap ? end : cap;
+      for (int64_t n = total + threadIdx.x; n < end; n += kThreads) row_tokens[n] = 0;
     }
   }
   for (int n = threadIdx.x; n < mx; n += kThreads) {
@@ -245,7 +256,7 @@ extern "C" int rd_tree_build(const int64_t* beams, int batch, int width, int len
                              int64_t* prefix_tree, int64_t* unpacker, int64_t* packed_tokens,
                              int64_t* packed_token_indices, int64_t* position_offsets,
                              int32_t* counts, int32_t* row_start, int64_t* row_slots,
-                             void* workspace, size_t workspace_bytes, void* stream) {
+                             int64_t* row_tokens, void* workspace, size_t workspace_bytes, void* stream) {
   RD_REQUIRE(batch > 0 && width > 0 && length > 0, RD_EINVAL,
              "rd_tree_build: batch/width/length must be positive (%d,%d,%d)", batch, width, length);
   RD_REQUIRE(width <= kMaxWidth && length <= kMaxLength && width * length <= kMaxTokens, RD_ELIMIT,
@@ -269,7 +280,7 @@ extern "C" int rd_tree_build(const int64_t* beams, int batch, int width, int len
   if (int e = rd::check_launch("rd_tree_build(rows)")) return e;
   { rd::ScopedTiming rd_t("tree_fill_kernel", s); hipLaunchKernelGGL(tree_fill_kernel, dim3(batch), dim3(kThreads), 0, s, sel_tok, sel_idx, batch,
                      width * length, length, counts, packed_tokens, packed_token_indices,
-                     position_offsets, row_start, row_slots); }
+                     position_offsets, row_start, row_slots, row_tokens); }
   return rd::check_launch("rd_tree_build(fill)");
 }
 

@@ -238,7 +238,7 @@ class LlamaModel(LlamaPreTrainedModel):
                 attention_mask, fix_empty_rows=False, n_heads=self.config.num_attention_heads,
                 kv_shift=_kv_shift(past_key_values))
         if rows is not None:
-            input_ids = rows.take(input_ids)
+            input_ids = rows.take_tokens(input_ids)
         hidden_states, delta = self.embed_tokens(input_ids), None
         for layer, key_value in zip(self.layers, past_key_values):
             hidden_states, delta = layer.forward_deferred(hidden_states, delta, position_ids, key_value,

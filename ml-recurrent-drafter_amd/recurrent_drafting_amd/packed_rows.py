@@ -37,6 +37,9 @@ class PackedRows:
     batch: int
     n: int  # slots per batch row in the padded layout
     rows: int  # rows handed to the dense layers: total rounded up (the extra rows are copies of slot 0)
+    # (rows,) int64 or None: the token ids of the packed rows when whoever built the rows knows them
+    # (rd_tree_build does), zeros in the extra rows; `take_tokens` then needs no gather
+    tokens: Optional[torch.Tensor] = None
 
     @staticmethod
     def from_counts(counts: torch.Tensor, total: int, n: int,
@@ -59,6 +62,14 @@ class PackedRows:
         """(batch, n, ...) -> (rows, ...): the slots that exist, then the stand-in rows."""
         assert padded.shape[:2] == (self.batch, self.n)
         return padded.flatten(0, 1).index_select(0, self.index)
+
+    def take_tokens(self, padded_ids: torch.Tensor) -> torch.Tensor:
+        """`take` for the token ids of the model's input: uses the list the tree build left, if any
+        (its extra rows hold token 0 instead of a copy of slot 0; those rows are dropped anyway)."""
+        if self.tokens is not None:
+            assert padded_ids.shape == (self.batch, self.n)
+            return self.tokens
+        return self.take(padded_ids)
 
     def scatter(self, rows: torch.Tensor, fill=0) -> torch.Tensor:
         """(rows, ...) -> (batch, n, ...), `fill` in the slots that do not exist."""

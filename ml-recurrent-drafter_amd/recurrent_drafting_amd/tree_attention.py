@@ -31,11 +31,12 @@ class PackedTree:
     total: int  # sum of the rows' counts, host value
     row_start: torch.Tensor  # (B+1,) int32: slots that exist in the rows before each row
     row_slots: torch.Tensor  # (total rounded up,) int64: slot b*n+t of every slot that exists, row after row, then zeros
+    row_tokens: Optional[torch.Tensor] = None  # (total rounded up,) int64: the tokens of those slots, then zeros
 
     def rows(self) -> PackedRows:
         """The slots that exist (slot t of row b exists iff t < counts[b])."""
         return PackedRows(self.row_start, self.row_slots, self.total, self.unpacker.shape[0], self.n,
-                          self.row_slots.shape[0])
+                          self.row_slots.shape[0], self.row_tokens)
 
 
 def _check_beams(beams: torch.Tensor) -> Tuple[int, int, int]:
@@ -49,7 +50,7 @@ class PendingTree:
     """The launches of `build_tree` are queued; the packed length and the total (two int32 at
     `sizes`, on the device) still have to reach the host before the outputs can be shaped."""
 
-    slab: torch.Tensor  # (6, B*W*L) int64
+    slab: torch.Tensor  # (7, B*W*L) int64
     counts: torch.Tensor  # (2B+3,) int32: counts (B), max, total, row_start (B+1)
     shape: Tuple[int, int, int]
 
@@ -72,6 +73,7 @@ class PendingTree:
             total=total,
             row_start=counts[B + 2 :],
             row_slots=slab[5, : round_up_rows(total, B * W * L)],
+            row_tokens=slab[6, : round_up_rows(total, B * W * L)],
         )
 
 
@@ -82,7 +84,7 @@ def build_tree_enqueue(beams: torch.Tensor) -> PendingTree:
     beams = beams.contiguous()
     dev = beams.device
     n_tok = B * W * L
-    slab = torch.empty((6, n_tok), dtype=torch.long, device=dev)
+    slab = torch.empty((7, n_tok), dtype=torch.long, device=dev)
     counts = torch.empty(2 * B + 3, dtype=torch.int32, device=dev)  # counts (B+2), then row_start (B+1)
     lib = _hip.lib()
     ws_bytes = lib.rd_tree_workspace_bytes(B, W, L)
@@ -92,7 +94,7 @@ def build_tree_enqueue(beams: torch.Tensor) -> PendingTree:
             _hip.ptr(beams), B, W, L,
             _hip.ptr(slab[0]), _hip.ptr(slab[1]), _hip.ptr(slab[2]), _hip.ptr(slab[3]),
             _hip.ptr(slab[4]), _hip.ptr(counts), _hip.ptr(counts[B + 2 :]), _hip.ptr(slab[5]),
-            _hip.ptr(ws), ws_bytes, _hip.stream(),
+            _hip.ptr(slab[6]), _hip.ptr(ws), ws_bytes, _hip.stream(),
         )
     )
     return PendingTree(slab, counts, (B, W, L))

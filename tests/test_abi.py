@@ -38,9 +38,9 @@ def test_argument_errors_are_reported_without_a_gpu():
     from recurrent_drafting_amd import _hip
 
     lib = _hip.lib()
-    rc = lib.rd_tree_build(None, 0, 45, 5, None, None, None, None, None, None, None, None, None, 0, None)
+    rc = lib.rd_tree_build(None, 0, 45, 5, None, None, None, None, None, None, None, None, None, None, 0, None)
     assert rc == -1 and b"positive" in lib.rd_last_error()
-    rc = lib.rd_tree_build(None, 8, 2000, 5, None, None, None, None, None, None, None, None, None, 0, None)
+    rc = lib.rd_tree_build(None, 8, 2000, 5, None, None, None, None, None, None, None, None, None, None, 0, None)
     assert rc == -2
     assert lib.rd_tree_workspace_bytes(8, 45, 5) >= 8 * 45 * 5 * 12
 

@@ -135,3 +135,8 @@ def test_tree_build_lists_the_slots_that_exist():
         assert torch.equal(got.row_start, want.row_start) and got.row_start.dtype == torch.int32
         assert torch.equal(got.index, want.index) and got.index.dtype == torch.long
         assert (got.total, got.batch, got.n, got.rows) == (want.total, B, tree.n, want.rows)
+        # the tokens of those rows, as the embedding lookup takes them: the existing slots' tokens, then zeros
+        taken = want.take(tree.packed_beams)
+        assert got.tokens is not None and got.tokens.shape == taken.shape
+        assert torch.equal(got.tokens[: got.total], taken[: got.total]) and not got.tokens[got.total :].any()
+        assert got.take_tokens(tree.packed_beams) is got.tokens
