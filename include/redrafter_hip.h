@@ -145,6 +145,13 @@ RD_API int rd_accept_greedy(const int64_t* beams, const int64_t* llm_tokens, int
 /* Leading pad run per row.  Replaces _count_left_paddings (recurrent_drafting.py:387-388). */
 RD_API int rd_count_left_paddings(const int64_t* input_ids, int64_t ids_row_stride, int64_t prev,
                                   int batch, int64_t pad_token_id, int32_t* pads, void* stream);
+/* rd_position_ids: position_ids[b, t] = (prev - leading pads of row b) + position_offsets[b, t],
+ * contiguous (batch, n) int64: the position rule of the verification forward
+ * (recurrent_drafting.py:449-458) with the pad count folded in. */
+RD_API int rd_position_ids(const int64_t* input_ids, int64_t ids_row_stride, int64_t prev,
+                           int batch, int64_t pad_token_id, const int64_t* position_offsets,
+                           int64_t offsets_row_stride, int n, int64_t* position_ids,
+                           void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Token ids after acceptance, right-aligned and left-padded, plus the per-row plan that

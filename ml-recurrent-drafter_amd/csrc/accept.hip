@@ -148,6 +148,29 @@ __global__ __launch_bounds__(kThreads) void count_pads_kernel(const int64_t* __r
   if (threadIdx.x == 0) pads[blockIdx.x] = s_first;
 }
 
+// position_ids[b, t] = (prev - leading pads of row b) + offsets[b, t]: the pad count of
+// count_pads_kernel and the two elementwise steps that follow it upstream, in one launch.
+__global__ __launch_bounds__(kThreads) void position_ids_kernel(
+    const int64_t* __restrict__ ids, int64_t row_stride, int64_t prev, int64_t pad,
+    const int64_t* __restrict__ offsets, int64_t offsets_row_stride, int n,
+    int64_t* __restrict__ out) {
+  const int64_t* row = ids + (int64_t)blockIdx.x * row_stride;
+  __shared__ int s_first;
+  if (threadIdx.x == 0) s_first = (int)prev;
+  __syncthreads();
+  for (int64_t base = 0; base < prev; base += kThreads) {
+    const int64_t j = base + threadIdx.x;
+    if (j < prev && row[j] != pad) atomicMin(&s_first, (int)j);
+    __syncthreads();
+    const int first = s_first;
+    __syncthreads();
+    if (first < prev) break;
+  }
+  const int64_t start = prev - s_first;
+  const int64_t* off = offsets + (int64_t)blockIdx.x * offsets_row_stride;
+  for (int t = threadIdx.x; t < n; t += kThreads) out[(int64_t)blockIdx.x * n + t] = start + off[t];
+}
+
 // plan layout (int32): [0]=M, [1]=prev, [2]=L, [3]=0, then per row 4+L ints:
 //   {old_pads, new_pads, n_new, live_len, src_row[0..L)}
 __global__ __launch_bounds__(kThreads) void realign_plan_kernel(
@@ -281,6 +304,22 @@ extern "C" int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride,
                      ids_row_stride, prev, n_tokens_in_seq, seq_in_beam, beams, unpacker, batch,
                      width, length, pad_token_id, pads, plan, new_ids, kv_row_shift); }
   return rd::check_launch("rd_realign_plan");
+}
+
+extern "C" int rd_position_ids(const int64_t* input_ids, int64_t ids_row_stride, int64_t prev,
+                               int batch, int64_t pad_token_id, const int64_t* position_offsets,
+                               int64_t offsets_row_stride, int n, int64_t* position_ids,
+                               void* stream) {
+  RD_REQUIRE(batch > 0 && n > 0 && prev >= 0 && prev < 2147483647LL, RD_EINVAL,
+             "rd_position_ids: batch %d n %d prev %lld", batch, n, (long long)prev);
+  RD_REQUIRE((prev == 0 || input_ids) && position_offsets && position_ids, RD_EINVAL,
+             "rd_position_ids: null pointer");
+  RD_REQUIRE((prev == 0 || ids_row_stride >= prev) && offsets_row_stride >= n, RD_EINVAL,
+             "rd_position_ids: a row stride is shorter than its row");
+  { rd::ScopedTiming rd_t("position_ids_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(position_ids_kernel, dim3(batch), dim3(kThreads), 0, rd::as_stream(stream),
+                     input_ids, ids_row_stride, prev, pad_token_id, position_offsets,
+                     offsets_row_stride, n, position_ids); }
+  return rd::check_launch("rd_position_ids");
 }
 
 extern "C" int rd_count_left_paddings(const int64_t* input_ids, int64_t ids_row_stride,

@@ -34,6 +34,7 @@ _PROTOTYPES = {
     "rd_argmax_rows": (_I, [_P, _I, _L, _L, _L, _P, _P]),
     "rd_accept_greedy": (_I, [_P, _P, _L, _P, _I, _I, _I, _P, _P, _P, _P, _P]),
     "rd_count_left_paddings": (_I, [_P, _L, _L, _I, _L, _P, _P]),
+    "rd_position_ids": (_I, [_P, _L, _L, _I, _L, _P, _L, _I, _P, _P]),
     "rd_realign_plan_ints": (_Z, [_I, _I]),
     "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P, _P]),
     "rd_kv_unpack": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _I, _I, _P]),

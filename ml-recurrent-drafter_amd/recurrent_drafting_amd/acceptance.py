@@ -62,6 +62,26 @@ def _count_left_paddings_int32(tokens: torch.Tensor, pad_token_id: int) -> torch
     return pads
 
 
+def tree_position_ids(input_ids: torch.Tensor, pad_token_id: int, position_offsets: torch.Tensor) -> torch.Tensor:
+    """(B, n) int64 positions of the packed tree tokens: each row's token count so far (its length
+    minus its left padding) plus the token's depth in the tree (recurrent_drafting.py:449-458)."""
+    assert input_ids.dim() == 2 and input_ids.dtype == torch.long
+    assert position_offsets.dim() == 2 and position_offsets.dtype == torch.long and position_offsets.stride(1) == 1
+    if input_ids.shape[1] > 0 and input_ids.stride(1) != 1:
+        input_ids = input_ids.contiguous()
+    B, prev = input_ids.shape
+    n = position_offsets.shape[1]
+    assert position_offsets.shape[0] == B
+    out = torch.empty((B, n), dtype=torch.long, device=input_ids.device)
+    _hip.check(
+        _hip.lib().rd_position_ids(
+            _hip.ptr(input_ids) if prev > 0 else None, input_ids.stride(0), prev, B, pad_token_id,
+            _hip.ptr(position_offsets), position_offsets.stride(0), n, _hip.ptr(out), _hip.stream(),
+        )
+    )
+    return out
+
+
 def greedy_accept(
     beams_by_drafter: torch.Tensor,
     llm_tokens: torch.Tensor,

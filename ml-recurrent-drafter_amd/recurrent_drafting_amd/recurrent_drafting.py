@@ -194,8 +194,7 @@ class RecurrentDrafting(torch.nn.Module):
         with step_record.time("verify_candidates"):
             prev = input_ids.shape[1]
             mask = tree_attention.build_mask(tree, input_ids != pad)
-            pads = acceptance._count_left_paddings_int32(input_ids, pad)
-            position_ids = (prev - pads).unsqueeze(-1) + tree.position_offsets  # int32 + int64 -> int64
+            position_ids = acceptance.tree_position_ids(input_ids, pad, tree.position_offsets)
             # the slots past a row's own tree are padding (other rows' tokens, tree_attention.py:70-122)
             # that the reference computes and never reads: the model runs on the slots that exist
             rows = tree.rows()

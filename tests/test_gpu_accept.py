@@ -137,6 +137,26 @@ def test_count_left_paddings():
         assert np.array_equal(got.cpu().numpy(), T.count_left_paddings(x, 0))
 
 
+def test_tree_position_ids_equal_the_op_chain():
+    """position_ids = (prev - left pads) + position offsets (recurrent_drafting.py:449-458), with
+    all-pad rows, rows without pads, an empty prefix, a strided offsets view and a pad id that is not 0."""
+    from recurrent_drafting_amd import acceptance
+
+    rng = np.random.default_rng(5)
+    for (B, prev, n), pad in [((1, 4, 1), 0), ((3, 17, 9), 0), ((8, 2548, 181), 0), ((5, 700, 33), 7), ((2, 0, 5), 0)]:
+        x = rng.integers(0, 9, size=(B, prev))
+        for b in range(B):
+            x[b, : rng.integers(0, prev + 1)] = pad
+        if B > 2 and prev:
+            x[0, :] = pad
+            x[1, 0] = pad + 1
+        off = rng.integers(0, 5, size=(B, n + 3))
+        offsets = _dev(off)[:, :n]  # row stride n + 3
+        got = acceptance.tree_position_ids(_dev(x), pad, offsets)
+        want = (prev - T.count_left_paddings(x, pad))[:, None] + off[:, :n]
+        assert got.dtype == torch.long and np.array_equal(got.cpu().numpy(), want)
+
+
 def test_cache_object(literals):
     """The reference's test_cache, on the GPU object."""
     from recurrent_drafting_amd import kv_cache
