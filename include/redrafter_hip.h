@@ -95,13 +95,16 @@ RD_API int rd_tree_build(const int64_t* beams, int batch, int width, int length,
  * (attention.py:12-55) and the final row slice (tree_attention.py:337).
  *
  * padding_mask: (batch, prev) of pm_elem_bytes-wide integers (1, 4 or 8), row stride
- * pm_row_stride elements; non-zero = real token.  May be NULL when prev == 0.
+ * pm_row_stride elements; an element equal to pm_pad_value is padding, any other a real token
+ * (0 for a 0/1 mask; the pad token id when the token ids themselves are handed in, which saves
+ * the caller the comparison).  May be NULL when prev == 0.
  * mask: capacity batch*width*length*(prev+width*length) bytes, written as a contiguous
  * (batch, max_n, prev+max_n) array of 0/1 bytes with max_n = counts[batch].
  * ------------------------------------------------------------------------------------------ */
 RD_API int rd_tree_mask(const int64_t* unpacker, const int64_t* packed_token_indices,
                  const int32_t* counts, const void* padding_mask, int pm_elem_bytes,
-                 int64_t pm_row_stride, int64_t prev, int batch, int width, int length,
+                 int64_t pm_row_stride, int64_t pm_pad_value, int64_t prev, int batch, int width,
+                 int length,
                  uint8_t* mask, void* stream);
 
 /* ------------------------------------------------------------------------------------------

@@ -167,7 +167,8 @@ template <typename PM>
 __global__ __launch_bounds__(kThreads) void tree_mask_kernel(
     const int64_t* __restrict__ unpacker, const int64_t* __restrict__ packed_token_indices,
     const int32_t* __restrict__ counts, const PM* __restrict__ padding_mask,
-    int64_t pm_row_stride, int64_t prev, int B, int WL, int L, uint8_t* __restrict__ mask) {
+    int64_t pm_row_stride, int64_t prev, int B, int WL, int L, uint8_t* __restrict__ mask,
+    int64_t pm_pad_value) {
   const int max_n = counts[B];
   const int n = blockIdx.x;
   const int b = blockIdx.y;
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void tree_mask_kernel(
   const PM* pm = padding_mask + (int64_t)b * pm_row_stride;
 
   auto value = [&](int64_t c) -> uint8_t {
-    if (c < prev) return pm[c] != 0;
+    if (c < prev) return pm[c] != (PM)pm_pad_value;
     const int t = (int)(c - prev);
     uint8_t hit = 0;
     for (int kk = 0; kk <= k; ++kk) hit |= (s_tgt[kk] == t);
@@ -286,8 +287,8 @@ extern "C" int rd_tree_build(const int64_t* beams, int batch, int width, int len
 
 extern "C" int rd_tree_mask(const int64_t* unpacker, const int64_t* packed_token_indices,
                             const int32_t* counts, const void* padding_mask, int pm_elem_bytes,
-                            int64_t pm_row_stride, int64_t prev, int batch, int width, int length,
-                            uint8_t* mask, void* stream) {
+                            int64_t pm_row_stride, int64_t pm_pad_value, int64_t prev, int batch,
+                            int width, int length, uint8_t* mask, void* stream) {
   RD_REQUIRE(batch > 0 && width > 0 && length > 0 && prev >= 0, RD_EINVAL,
              "rd_tree_mask: bad sizes (batch %d width %d length %d prev %lld)", batch, width, length,
              (long long)prev);
@@ -308,7 +309,7 @@ extern "C" int rd_tree_mask(const int64_t* unpacker, const int64_t* packed_token
 #define RD_LAUNCH_MASK(T)                                                                       \
   do { rd::ScopedTiming rd_t("tree_mask_kernel", s); hipLaunchKernelGGL(tree_mask_kernel<T>, grid, dim3(kThreads), 0, s, unpacker,                  \
                      packed_token_indices, counts, reinterpret_cast<const T*>(padding_mask),    \
-                     pm_row_stride, prev, batch, WL, length, mask); } while (0)
+                     pm_row_stride, prev, batch, WL, length, mask, pm_pad_value); } while (0)
   if (pm_elem_bytes == 1) RD_LAUNCH_MASK(uint8_t);
   else if (pm_elem_bytes == 4) RD_LAUNCH_MASK(int32_t);
   else RD_LAUNCH_MASK(int64_t);

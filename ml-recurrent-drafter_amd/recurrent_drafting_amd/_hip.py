@@ -29,7 +29,7 @@ _PROTOTYPES = {
     "rd_timing_collect": (_I, [C.c_char_p, _Z]),
     "rd_tree_workspace_bytes": (_Z, [_I, _I, _I]),
     "rd_tree_build": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
-    "rd_tree_mask": (_I, [_P, _P, _P, _P, _I, _L, _L, _I, _I, _I, _P, _P]),
+    "rd_tree_mask": (_I, [_P, _P, _P, _P, _I, _L, _L, _L, _I, _I, _I, _P, _P]),
     "rd_unpack_rows": (_I, [_P, _L, _L, _P, _L, _I, _I, _I, _P, _L, _L, _P]),
     "rd_argmax_rows": (_I, [_P, _I, _L, _L, _L, _P, _P]),
     "rd_accept_greedy": (_I, [_P, _P, _L, _P, _I, _I, _I, _P, _P, _P, _P, _P]),

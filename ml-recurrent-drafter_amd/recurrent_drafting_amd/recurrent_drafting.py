@@ -193,7 +193,7 @@ class RecurrentDrafting(torch.nn.Module):
         greedy = sampling_args.greedy
         with step_record.time("verify_candidates"):
             prev = input_ids.shape[1]
-            mask = tree_attention.build_mask(tree, input_ids != pad)
+            mask = tree_attention.build_mask(tree, input_ids, pad_value=pad)  # (no `input_ids != pad` launch)
             position_ids = acceptance.tree_position_ids(input_ids, pad, tree.position_offsets)
             # the slots past a row's own tree are padding (other rows' tokens, tree_attention.py:70-122)
             # that the reference computes and never reads: the model runs on the slots that exist

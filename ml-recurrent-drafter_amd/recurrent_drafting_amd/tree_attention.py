@@ -107,8 +107,10 @@ def build_tree(beams: torch.Tensor) -> PackedTree:
     return pending.finish(n, total)
 
 
-def build_mask(tree: PackedTree, padding_mask: torch.Tensor) -> torch.Tensor:
-    """(B, n, prev+n) bool mask of the packed rows (tree_attention.py:336-337)."""
+def build_mask(tree: PackedTree, padding_mask: torch.Tensor, pad_value: int = 0) -> torch.Tensor:
+    """(B, n, prev+n) bool mask of the packed rows (tree_attention.py:336-337).  An element of
+    padding_mask equal to pad_value is padding: a 0/1 mask with the default, or the token ids
+    themselves with the pad token id."""
     B, W, L = tree.unpacker.shape
     assert padding_mask.dim() == 2 and padding_mask.shape[0] == B
     assert padding_mask.dtype in (torch.int32, torch.int64, torch.bool, torch.uint8)
@@ -121,7 +123,7 @@ def build_mask(tree: PackedTree, padding_mask: torch.Tensor) -> torch.Tensor:
         _hip.lib().rd_tree_mask(
             _hip.ptr(tree.unpacker), _hip.ptr(tree.packed_token_indices), _hip.ptr(tree.counts),
             _hip.ptr(padding_mask) if prev > 0 else None, padding_mask.element_size(),
-            padding_mask.stride(0) if prev > 0 else 0, prev, B, W, L, _hip.ptr(out), _hip.stream(),
+            padding_mask.stride(0) if prev > 0 else 0, int(pad_value), prev, B, W, L, _hip.ptr(out), _hip.stream(),
         )
     )
     return out

@@ -108,3 +108,20 @@ def test_limits_raise():
         tree_attention.build_tree(torch.zeros((1, 2048, 2), dtype=torch.long, device="cuda"))
     with pytest.raises(AssertionError):
         tree_attention.build_tree(torch.zeros((1, 4, 2), dtype=torch.int32, device="cuda"))
+
+
+def test_mask_from_token_ids_equals_mask_from_the_comparison():
+    """rd_tree_mask takes the token ids with the pad id in place of a 0/1 padding mask."""
+    from recurrent_drafting_amd import tree_attention
+
+    rng = np.random.default_rng(11)
+    for B, W, L, prev, pad in ((2, 3, 4, 9, 0), (8, 45, 5, 600, 0), (3, 5, 3, 40, 7)):
+        beams = torch.tensor(T.synthetic_beams(B, W, L, vocab=50, seed=prev), device="cuda")
+        ids = rng.integers(0, 12, size=(B, prev))
+        for b in range(B):
+            ids[b, : rng.integers(0, prev // 2)] = pad
+        ids = torch.tensor(ids, device="cuda")
+        tree = tree_attention.build_tree(beams)
+        want = tree_attention.build_mask(tree, ids != pad)
+        got = tree_attention.build_mask(tree, ids, pad_value=pad)
+        assert torch.equal(got, want)
