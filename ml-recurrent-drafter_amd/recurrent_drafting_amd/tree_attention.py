@@ -54,26 +54,37 @@ class PendingTree:
     counts: torch.Tensor  # (2B+3,) int32: counts (B), max, total, row_start (B+1)
     shape: Tuple[int, int, int]
 
+    def __post_init__(self):
+        # every view that does not depend on the sizes is cut now: `finish` runs between the step's
+        # one read and the first launch of the verify forward, with the GPU waiting
+        B, W, L = self.shape
+        self._rows = self.slab.unbind(0)
+        self._unpacker = self._rows[1].view(B, W, L)
+        self._prefix_tree = self._rows[0].view(B, W, L)
+        self._counts = self.counts[: B + 2]
+        self._row_start = self.counts[B + 2 :]
+        self._sizes = self.counts[B : B + 2]
+
     @property
     def sizes(self) -> torch.Tensor:
-        B = self.shape[0]
-        return self.counts[B : B + 2]
+        return self._sizes
 
     def finish(self, n: int, total: int) -> PackedTree:
         B, W, L = self.shape
-        slab, counts = self.slab, self.counts
+        rows = self._rows
+        padded = round_up_rows(total, B * W * L)
         return PackedTree(
-            packed_beams=slab[2, : B * n].view(B, n),
-            unpacker=slab[1].view(B, W, L),
-            packed_token_indices=slab[3, : B * n].view(B, n),
-            position_offsets=slab[4, : B * n].view(B, n),
-            prefix_tree=slab[0].view(B, W, L),
-            counts=counts[: B + 2],
+            packed_beams=rows[2].as_strided((B, n), (n, 1)),
+            unpacker=self._unpacker,
+            packed_token_indices=rows[3].as_strided((B, n), (n, 1)),
+            position_offsets=rows[4].as_strided((B, n), (n, 1)),
+            prefix_tree=self._prefix_tree,
+            counts=self._counts,
             n=n,
             total=total,
-            row_start=counts[B + 2 :],
-            row_slots=slab[5, : round_up_rows(total, B * W * L)],
-            row_tokens=slab[6, : round_up_rows(total, B * W * L)],
+            row_start=self._row_start,
+            row_slots=rows[5][:padded],
+            row_tokens=rows[6][:padded],
         )
 
 
