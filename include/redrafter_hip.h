@@ -345,10 +345,13 @@ RD_API int rd_causal_mask(const void* padding_mask, int pm_elem_bytes, int64_t p
  * new token under each INPUT beam (rounded through `dtype` as upstream), row stride in elements.
  * Limits: width <= 64, vocab <= 65536, top_k <= 512.  force_fallback != 0 runs the slow exact
  * path that otherwise only serves rows with very many tied logits.
+ * Row (b, w) of the logits starts at logits + b*batch_stride + w*row_stride elements; batch_stride 0
+ * stands for width*row_stride, and row_stride 0 (with a batch stride) lets every beam of a batch
+ * row read the same logits -- the first iteration, in which all beams are copies of one.
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_beam_topk_workspace_bytes(int batch, int width);
-RD_API int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, int batch, int width,
-                        int vocab, const float* log_p_beam, int top_k, float mask_value,
+RD_API int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, int64_t batch_stride,
+                        int batch, int width, int vocab, const float* log_p_beam, int top_k, float mask_value,
                         const int64_t* beams_in, int t_len, float* new_log_p_beam, int64_t* tokens,
                         int64_t* parents, int64_t* beams_out, float* logp_out,
                         int64_t logp_row_stride, void* workspace, size_t workspace_bytes,

@@ -115,15 +115,16 @@ __device__ void beam_row_fallback(const T* __restrict__ x_row, int V, float row_
 // ITEMS elements per thread, held as ITEMS/VEC vectors of VEC = 16 bytes / sizeof(T).
 template <typename T, int ITEMS, int THREADS>
 __global__ __launch_bounds__(THREADS) void beam_row_kernel(
-    const T* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ log_p_beam,
-    int W, int top_k, float mask_value, float* __restrict__ cand_score,
+    const T* __restrict__ logits, int64_t row_stride, int64_t batch_stride, int V,
+    const float* __restrict__ log_p_beam, int W, int top_k, float mask_value,
+    float* __restrict__ cand_score,
     int32_t* __restrict__ cand_tok, float* __restrict__ logp_out, int64_t logp_row_stride,
     int force_fallback) {
   constexpr int VEC = 16 / sizeof(T);
   __shared__ RowShared sh;
   const int row = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const T* x_row = logits + (int64_t)row * row_stride;
+  const T* x_row = logits + (int64_t)(row / W) * batch_stride + (int64_t)(row % W) * row_stride;
 
   // ---- load the row; maximum; pivot on the raw values -------------------------------------------
   float x[ITEMS];
@@ -303,14 +304,16 @@ __global__ __launch_bounds__(kMergeThreads) void beam_merge_kernel(
 }
 
 template <typename T>
-int launch_rows(const void* logits, int64_t row_stride, int rows, int V, const float* lpb, int W,
+int launch_rows(const void* logits, int64_t row_stride, int64_t batch_stride, int rows, int V,
+                const float* lpb, int W,
                 int top_k, float mask_value, float* cs, int32_t* ct, float* logp_out,
                 int64_t logp_row_stride, int force_fallback, hipStream_t s) {
   const T* x = reinterpret_cast<const T*>(logits);
 #define RD_ROWS(ITEMS, THREADS)                                                                     \
   do { rd::ScopedTiming rd_t("beam_row_kernel", s);                                                  \
     hipLaunchKernelGGL((beam_row_kernel<T, ITEMS, THREADS>), dim3(rows), dim3(THREADS), 0, s, x,     \
-                       row_stride, V, lpb, W, top_k, mask_value, cs, ct, logp_out, logp_row_stride,  \
+                       row_stride, batch_stride, V, lpb, W, top_k, mask_value, cs, ct, logp_out,     \
+                       logp_row_stride,                                                              \
                        force_fallback); } while (0)
   switch (row_geometry(V)) {
     case 0: RD_ROWS(32, 256); break;
@@ -331,8 +334,8 @@ extern "C" size_t rd_beam_topk_workspace_bytes(int batch, int width) {
   return rd::align_up(n * sizeof(float), 256) + rd::align_up(n * sizeof(int32_t), 256);
 }
 
-extern "C" int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, int batch, int width,
-                            int vocab, const float* log_p_beam, int top_k, float mask_value,
+extern "C" int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, int64_t batch_stride,
+                            int batch, int width, int vocab, const float* log_p_beam, int top_k, float mask_value,
                             const int64_t* beams_in, int t_len, float* new_log_p_beam,
                             int64_t* tokens, int64_t* parents, int64_t* beams_out, float* logp_out,
                             int64_t logp_row_stride, void* workspace, size_t workspace_bytes,
@@ -346,10 +349,14 @@ extern "C" int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, i
   RD_REQUIRE(logits && log_p_beam && new_log_p_beam && tokens && parents && workspace, RD_EINVAL,
              "rd_beam_topk: null pointer");
   RD_REQUIRE(!beams_out || (beams_in && t_len > 0), RD_EINVAL, "rd_beam_topk: beams_out needs beams_in and t_len > 0");
-  RD_REQUIRE(row_stride >= vocab, RD_EINVAL, "rd_beam_topk: row_stride %lld < vocab %d", (long long)row_stride, vocab);
+  if (batch_stride == 0) batch_stride = (int64_t)width * row_stride;
+  RD_REQUIRE(row_stride >= vocab || (row_stride == 0 && batch_stride >= vocab), RD_EINVAL,
+             "rd_beam_topk: row_stride %lld < vocab %d (0 is allowed with a batch stride: every beam of a row reads the same logits)",
+             (long long)row_stride, vocab);
+  RD_REQUIRE(batch_stride >= 0, RD_EINVAL, "rd_beam_topk: negative batch_stride");
   const int es = dtype == RD_F32 ? 4 : 2;
   RD_REQUIRE(dtype == RD_F32 || dtype == RD_BF16 || dtype == RD_F16, RD_EINVAL, "rd_beam_topk: unknown dtype %d", dtype);
-  RD_REQUIRE(((uintptr_t)logits % 16) == 0 && (row_stride * es) % 16 == 0, RD_EINVAL,
+  RD_REQUIRE(((uintptr_t)logits % 16) == 0 && (row_stride * es) % 16 == 0 && (batch_stride * es) % 16 == 0, RD_EINVAL,
              "rd_beam_topk: logits rows must be 16-byte aligned (row_stride %lld)", (long long)row_stride);
   RD_REQUIRE(!logp_out || logp_row_stride >= vocab, RD_EINVAL, "rd_beam_topk: logp_row_stride < vocab");
   RD_REQUIRE(workspace_bytes >= rd_beam_topk_workspace_bytes(batch, width), RD_EWORKSPACE,
@@ -363,9 +370,9 @@ extern "C" int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, i
   const int rows = batch * width;
   int e;
   switch (dtype) {
-    case RD_F32: e = launch_rows<float>(logits, row_stride, rows, vocab, log_p_beam, width, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback, s); break;
-    case RD_BF16: e = launch_rows<__hip_bfloat16>(logits, row_stride, rows, vocab, log_p_beam, width, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback, s); break;
-    default: e = launch_rows<__half>(logits, row_stride, rows, vocab, log_p_beam, width, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback, s); break;
+    case RD_F32: e = launch_rows<float>(logits, row_stride, batch_stride, rows, vocab, log_p_beam, width, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback, s); break;
+    case RD_BF16: e = launch_rows<__hip_bfloat16>(logits, row_stride, batch_stride, rows, vocab, log_p_beam, width, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback, s); break;
+    default: e = launch_rows<__half>(logits, row_stride, batch_stride, rows, vocab, log_p_beam, width, top_k, mask_value, cs, ct, logp_out, logp_row_stride, force_fallback, s); break;
   }
   if (e) return e;
   { rd::ScopedTiming rd_t("beam_merge_kernel", s); hipLaunchKernelGGL(beam_merge_kernel, dim3(batch), dim3(kMergeThreads), 0, s, cs, ct, width, vocab,

@@ -70,7 +70,7 @@ _PROTOTYPES = {
     "rd_beam_topk_workspace_bytes": (_Z, [_I, _I]),
     "rd_beam_topk": (
         _I,
-        [_P, _I, _L, _I, _I, _I, _P, _I, _F, _P, _I, _P, _P, _P, _P, _P, _L, _P, _Z, _I, _P],
+        [_P, _I, _L, _L, _I, _I, _I, _P, _I, _F, _P, _I, _P, _P, _P, _P, _P, _L, _P, _Z, _I, _P],
     ),
 }
 

@@ -101,10 +101,16 @@ def beam_topk_step(
     B, W, V = logits.shape
     assert log_p_beam.dtype == torch.float32 and log_p_beam.shape == (B, W)
     assert beams.dtype == torch.long and beams.shape[:2] == (B, W)
-    x = logits.reshape(B * W, V)
-    if x.stride(0) < V:  # rows shown several times (an expanded view): the kernel wants real rows
-        x = x.contiguous()
-    x = _hip.aligned_rows(x)
+    if logits.stride(1) == 0 and logits.stride(2) == 1 and logits.stride(0) >= V \
+            and (logits.stride(0) * logits.element_size()) % 16 == 0 and logits.data_ptr() % 16 == 0:
+        # one row per batch row shown W times (the first iteration): the kernel reads it in place
+        x, row_stride, batch_stride = logits, 0, logits.stride(0)
+    else:
+        x = logits.reshape(B * W, V)
+        if x.stride(0) < V:  # rows shown several times some other way: the kernel wants real rows
+            x = x.contiguous()
+        x = _hip.aligned_rows(x)
+        row_stride, batch_stride = x.stride(0), 0
     beams = beams.contiguous()
     log_p_beam = log_p_beam.contiguous()
     t = beams.shape[2]
@@ -118,7 +124,7 @@ def beam_topk_step(
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     _hip.check(
         lib.rd_beam_topk(
-            _hip.ptr(x), _hip.dtype_code(x.dtype), x.stride(0), B, W, V, _hip.ptr(log_p_beam),
+            _hip.ptr(x), _hip.dtype_code(x.dtype), row_stride, batch_stride, B, W, V, _hip.ptr(log_p_beam),
             TOP_K, LOG_0, _hip.ptr(beams), t, _hip.ptr(new_lpb), _hip.ptr(tok_par[0]),
             _hip.ptr(tok_par[1]), _hip.ptr(new_beams), _hip.ptr(logp), V, _hip.ptr(ws), ws.numel(),
             int(force_fallback), _hip.stream(),

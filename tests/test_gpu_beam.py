@@ -69,6 +69,24 @@ def test_step_first_iteration_only_beam_zero_alive(force_fallback):
         assert torch.allclose(new_lpb, o_lpb, atol=1e-2, rtol=0)  # sums near -50000: fp32 spacing 4e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("force_fallback", [False, True])
+def test_step_reads_one_shared_row_in_place(dtype, force_fallback):
+    """The first iteration's logits are one row per batch row shown W times (stride 0): the kernel
+    reads that row in place and must return what it returns for W real copies."""
+    from recurrent_drafting_amd import modeling_drafter as md
+
+    torch.manual_seed(4)
+    for B, W, V in ((2, 45, 32000), (3, 64, 32000), (2, 5, 1000)):
+        one = (torch.randn(B, 1, V) * 3).to(dtype).cuda()
+        lpb = torch.full((B, W), O.LOG_0); lpb[:, 0] = O.LOG_1
+        beams = torch.randint(0, V, (B, 1, 1)).repeat(1, W, 1).cuda()
+        shared = md.beam_topk_step(one.expand(B, W, V), lpb.cuda(), beams, True, force_fallback)
+        copies = md.beam_topk_step(one.repeat(1, W, 1), lpb.cuda(), beams, True, force_fallback)
+        for a, b in zip(shared, copies):
+            assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("force_fallback", [False, True])
 def test_step_bf16_rounding_points(force_fallback):
     """bf16 logits: values rounded after the max subtraction, filter value -49920, log-softmax
