@@ -37,6 +37,7 @@ DRAFTER_7B = dict(vocab_size=32000, hidden_size=4096, exit_dim=8192, num_draft_l
 BATCH, PROMPT, NEW_TOKENS, WIDTH, LENGTH, SEED = 8, 500, 2048, 45, 5, 123
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
+TIMED_EVERY = 5  # the dominant kernel's launches are event-timed one in five
 
 
 def log(*a):
@@ -100,11 +101,15 @@ def gpu_run(steps: int, warmup: int):
         done += 1
     torch.cuda.synchronize()
 
-    # HIP events around every launch of the dominant kernel, live in the timed region (the events
-    # of ALL kernels would cost a few percent of the step; those are taken on the extra steps below)
+    # HIP events around the launches of the dominant kernel, live in the timed region: every
+    # TIMED_EVERY-th launch in launch order (the two events of a launch keep the GPU idle for about
+    # 11 us; around all 32 launches of a step that is 2.4 % of the step, around every fifth 0.5 %; five
+    # is coprime to the 32 layers, so the sample walks through the layers).  The events of ALL
+    # kernels are taken on the extra steps below.
     shapes = []
     attention.shape_log = shapes
     _hip.timing_select("attn_mfma_kernel")
+    _hip.timing_sample(TIMED_EVERY)
     _hip.timing_enable(True)
     elapsed, tokens, timed = 0.0, 0, 0
     first_len = last_len = None
@@ -133,6 +138,7 @@ def gpu_run(steps: int, warmup: int):
     null_us = _hip.timing_null_kernel_us(64)
     _hip.timing_enable(False)
     _hip.timing_select(None)
+    _hip.timing_sample(1)
     attention.shape_log = None
     accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
     # the generator that is still open has not posted its record yet; close it to flush
@@ -174,11 +180,12 @@ def attention_roofline(run):
     region actually ran: algorithmic FLOPs 4 * heads * head_dim * query rows * keys, algorithmic
     bytes K and V once (2 * heads * head_dim * 2 B per key) plus Q and O once, query rows = the
     tree slots that exist (the padding slots of the (batch, n_q) layout are not run); duration = HIP events
-    around every launch in the timed region.  Arithmetic intensity below the machine balance
+    around every TIMED_EVERY-th launch of the timed region (the shapes are those of the same launches).  Arithmetic intensity below the machine balance
     (2500 TFLOP/s / 8 TB/s = 312 FLOP/B) means the HBM roof binds, above it the MFMA roof."""
     H, D = LLAMA_7B["num_attention_heads"], LLAMA_7B["hidden_size"] // LLAMA_7B["num_attention_heads"]
     count, total_ms = run["dominant"].get("attn_mfma_kernel", (0, 0.0))
-    shapes = run["shapes"][:count] if count else []
+    launched = len(run["shapes"])
+    shapes = run["shapes"][::TIMED_EVERY][:count] if count else []  # the launches that were timed
     if not count or total_ms <= 0:
         return None
     flops = sum(4.0 * H * D * rows * kv for (B, n_q, kv, rows) in shapes)
@@ -198,7 +205,8 @@ def attention_roofline(run):
         out.update(bound="mfma", achieved=round(tflops, 2), peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
                    frac=round(tflops / MFMA_BF16_PEAK_TFLOPS, 4))
     out.update(
-        traffic=traffic, launches=count, avg_us=round(total_ms * 1e3 / count, 2),
+        traffic=traffic, launches=count, launches_in_timed_region=launched, timed_every=TIMED_EVERY,
+        avg_us=round(total_ms * 1e3 / count, 2),
         algorithmic_gflop_per_launch=round(flops / count / 1e9, 3),
         algorithmic_mb_per_launch=round(k_bytes / count / 1e6, 2),
         flop_per_byte=round(flops / k_bytes, 1),

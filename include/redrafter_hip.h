@@ -51,9 +51,13 @@ RD_API const char* rd_last_error(void);
  * text line per kernel, "<kernel> <launches> <total_ms>", into a HOST buffer, then resets the
  * pool.  rd_timing_enable(0) stops recording.  rd_timing_select("kernel_name") restricts the
  * recording to one kernel (the events of every launch cost a few percent of a decode step);
- * NULL or "" selects all again. */
+ * NULL or "" selects all again.  rd_timing_sample(n) times every n-th of the launches that qualify
+ * (counted from the call and from every rd_timing_enable; n = 1 times all): the two events of a
+ * launch keep the GPU idle for about 11 us, which for a kernel launched 32 times per decode step
+ * is 2.4 % of the step. */
 RD_API int rd_timing_enable(int on);
 RD_API int rd_timing_select(const char* kernel);
+RD_API int rd_timing_sample(int every);
 /* Average event-to-event time of an EMPTY kernel timed the same way, in microseconds: the fixed
  * part (dispatch and completion signalling) that the figures of rd_timing_collect include and a
  * kernel trace does not.  Synchronises the stream. */

@@ -30,6 +30,8 @@ struct TimingState {
   bool enabled = false;
   std::string only;  // when not empty: the one kernel that is timed
   int used = 0;
+  int every = 1;  // of the launches that qualify, every n-th is timed ...
+  long seen = 0;  // ... counted from the last rd_timing_enable
   std::vector<hipEvent_t> start, stop;
   std::vector<const char*> name;
 };
@@ -44,6 +46,7 @@ ScopedTiming::ScopedTiming(const char* name, hipStream_t stream) : stream_(strea
   if (!t.enabled) return;
   std::lock_guard<std::mutex> lock(t.mu);
   if (!t.only.empty() && t.only != name) return;
+  if ((t.seen++ % t.every) != 0) return;
   if (t.used >= (int)t.start.size()) return;  // pool exhausted: later launches go untimed
   slot_ = t.used++;
   t.name[slot_] = name;
@@ -56,6 +59,7 @@ void timing_events(const char* name, hipEvent_t* start, hipEvent_t* stop) {
   if (!t.enabled) return;
   std::lock_guard<std::mutex> lock(t.mu);
   if (!t.only.empty() && t.only != name) return;
+  if ((t.seen++ % t.every) != 0) return;
   if (t.used >= (int)t.start.size()) return;
   const int slot = t.used++;
   t.name[slot] = name;
@@ -86,6 +90,16 @@ extern "C" int rd_timing_enable(int on) {
   }
   t.enabled = on != 0;
   t.used = 0;
+  t.seen = 0;
+  return RD_OK;
+}
+
+extern "C" int rd_timing_sample(int every) {
+  RD_REQUIRE(every >= 1, RD_EINVAL, "rd_timing_sample: every %d < 1", every);
+  auto& t = rd::timing();
+  std::lock_guard<std::mutex> lock(t.mu);
+  t.every = every;
+  t.seen = 0;
   return RD_OK;
 }
 

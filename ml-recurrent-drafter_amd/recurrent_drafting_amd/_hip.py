@@ -25,6 +25,7 @@ _PROTOTYPES = {
     "rd_last_error": (C.c_char_p, []),
     "rd_timing_enable": (_I, [_I]),
     "rd_timing_select": (_I, [C.c_char_p]),
+    "rd_timing_sample": (_I, [_I]),
     "rd_timing_null_kernel_us": (_I, [_I, _P, C.POINTER(C.c_float)]),
     "rd_timing_collect": (_I, [C.c_char_p, _Z]),
     "rd_tree_workspace_bytes": (_Z, [_I, _I, _I]),
@@ -134,6 +135,11 @@ def dtype_code(dt: torch.dtype) -> int:
         return _DTYPES[dt]
     except KeyError:
         raise TypeError(f"unsupported dtype {dt}; expected bfloat16, float16 or float32") from None
+
+
+def timing_sample(every: int) -> None:
+    """Time every `every`-th qualifying launch only (1: all of them)."""
+    check(lib().rd_timing_sample(int(every)))
 
 
 def timing_enable(on: bool) -> None:
