@@ -197,7 +197,6 @@ def case_kv(rows, reps):
         acceptance.realign(ids, nt, sb, beams, cache, 0, unpacker=tree.unpacker)
 
     k = timed(compact_in_place, reps)
-    k.pop("vectorized_elementwise_kernel", None)
     report(rows, f"realign + kv_compact prev {prev}, 7 of 8 rows shift, cache rows kept in place", k,
            {"kv_append_kernel": 2 * row * sum((t + 1) for t in n_tok)}, {"kv_append_kernel": "GB/s"})
 
