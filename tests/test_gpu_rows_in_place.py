@@ -156,3 +156,52 @@ def test_generate_is_the_same_with_rows_in_place_and_with_moved_rows(sampling):
     b, _ = _streams(False, **args)
     assert a == b
     assert max(acc) > 0.2, "nothing was accepted: the rows never shifted"
+
+
+def test_rope_append_drops_rows_that_a_shift_would_put_outside_the_cache():
+    """A shift that leaves the slab is never followed: q is still rotated, k and v of that row are
+    dropped, nothing outside the row's slab is written."""
+    from recurrent_drafting_amd import kv_cache
+
+    torch.manual_seed(5)
+    dtype, B, H, D, prev, n, max_len = torch.float32, 2, 2, 32, 6, 4, 12
+    cache = kv_cache.Cache(B, max_len, 1, H, D, dtype, torch.device("cuda"))
+    cache._cache.fill_(7.0)
+    cache.shift.copy_(torch.tensor([-5, 9], dtype=torch.int32))  # row 0: rows 11..14 (12+ outside); row 1: rows -3..0
+    cache.rows_in_place = True
+    cache._shifted = True
+    cache.set_length(prev)
+    q = torch.randn(B, n, H * D, device="cuda")
+    k = torch.randn(B, n, H * D, device="cuda")
+    v = torch.randn(B, n, H * D, device="cuda")
+    cos = torch.ones(prev + n, D, device="cuda")
+    sin = torch.zeros(prev + n, D, device="cuda")
+    pos = (prev + torch.arange(n, device="cuda")).repeat(B, 1)
+    qq, _, _ = kv_cache.rope_append(q.clone(), k, v, cos, sin, pos, cache.sliced[0])
+    assert torch.equal(qq.transpose(1, 2).reshape(B, n, H * D), q)  # identity rotation, every row
+    raw = cache._cache[0]  # (2, B, H, max_len, D)
+    kk = k.view(B, n, H, D).transpose(1, 2)
+    # row 0: token 0 lands in cache row 11, tokens 1..3 would be rows 12..14: dropped
+    assert torch.equal(raw[0, 0, :, 11], kk[0, :, 0]) and (raw[0, 0, :, :11] == 7).all()
+    # row 1: tokens 0..2 would be rows -3..-1: dropped; token 3 lands in row 0
+    assert torch.equal(raw[0, 1, :, 0], kk[1, :, 3]) and (raw[0, 1, :, 1:] == 7).all()
+    assert (cache._storage[: 64 * D] == 0).all()  # the slack in front of the first slab is untouched
+
+
+def test_timing_sample_times_every_nth_launch():
+    from recurrent_drafting_amd import _hip, acceptance
+
+    x = torch.randn(4, 1000, device="cuda")
+    try:
+        _hip.timing_select("argmax_rows_kernel")
+        _hip.timing_sample(3)
+        _hip.timing_enable(True)
+        for _ in range(10):
+            acceptance.argmax_rows(x)
+        torch.cuda.synchronize()
+        got = _hip.timing_collect()
+        assert got["argmax_rows_kernel"][0] == 4  # launches 0, 3, 6, 9
+    finally:
+        _hip.timing_enable(False)
+        _hip.timing_select(None)
+        _hip.timing_sample(1)
