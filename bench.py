@@ -86,6 +86,7 @@ def gpu_run(steps: int, warmup: int):
     torch.cuda.synchronize()
     log(f"[bench] models on {torch.cuda.get_device_name(0)} in {time.perf_counter() - t0:.1f}s")
     model = rd.RecurrentDrafting(llm, drafter)
+    rd.gemm_tuning.load()  # opt-in kernel selection table for the dense layers' GEMMs (look-up only)
     ids = prompts(dev)
     max_length = PROMPT + NEW_TOKENS
 
@@ -271,7 +272,7 @@ def cpu_baseline(per_seq_tokens: float):
 
 def cpu_kernel_baselines(reps: int = 3):
     """Per-kernel CPU baselines: the torch restatement of each stage on the host cores, on the shapes
-    of the kernel micro-benchmarks (ml-recurrent-drafter_amd/kernel_bench.py).  Needs no GPU.  Prints one
+    of the kernel micro-benchmarks (kernel_bench.py).  Needs no GPU.  Prints one
     line per case: best of `reps` passes after one warm-up pass."""
     import numpy as np
     from oracle import torch_path as P

@@ -1,6 +1,6 @@
 """Per-kernel micro-benchmarks of libredrafter_hip.so on one MI355X.
 
-    python ml-recurrent-drafter_amd/kernel_bench.py [--only NAME[,NAME]] [--reps N] [--json]
+    python kernel_bench.py [--only NAME[,NAME]] [--reps N] [--json]
 
 Each case runs one entry point on the benchmark shapes (batch 8, beam 45x5, vocabulary 32000,
 32 heads x 128, 32 layers; cached length U[500, 2548] for the attention), times the kernels with
@@ -20,7 +20,7 @@ import numpy as np
 import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, HERE)
+sys.path.insert(0, os.path.join(HERE, "ml-recurrent-drafter_amd"))
 
 import recurrent_drafting_amd as rd  # noqa: E402
 from recurrent_drafting_amd import _hip, acceptance, attention, kv_cache, modeling_drafter, tree_attention  # noqa: E402

@@ -8,7 +8,12 @@ winners of a search over every kernel both libraries offer (torch's TunableOp, t
 buffers so that no weight is served from a cache) for the problem sizes of the 7B-shaped model of
 the benchmark; `load()` hands it to torch.  A problem that is not in the table, or a table written
 for other library versions (torch checks the versions recorded in the file), leaves the default
-heuristic in charge.  `tune_gemms.py` at the package root writes a table for other sizes.
+heuristic in charge.
+
+Opt-in: nothing in the package calls `load()`.  It switches torch's TunableOp on for the whole
+process (look-up only), so every later GEMM of the process goes through
+the table; a caller that wants it says so (`recurrent_drafting_amd.gemm_tuning.load()`, as the
+benchmark does).
 """
 
 from __future__ import annotations
@@ -35,6 +40,8 @@ def load(path: str = TABLE) -> int:
 
     tunable.enable(True)
     tunable.tuning_enable(False)  # look up only: never search inside a decode step
+    if hasattr(tunable, "write_file_on_exit"):
+        tunable.write_file_on_exit(False)  # leave no results file in the working directory
     if tunable.read_file(path):
         _loaded = len(tunable.get_results())
     if _loaded == 0:

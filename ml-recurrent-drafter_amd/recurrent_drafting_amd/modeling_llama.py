@@ -50,6 +50,18 @@ def _fused_weight(owner: nn.Module, name: str, linears) -> torch.Tensor:
     return fused
 
 
+def unfuse_weights(model: nn.Module) -> None:
+    """Gives every projection its own weight storage again (the state before the first forward).
+    After a forward q/k/v_proj and gate/up_proj share one buffer each, which `save_pretrained` with
+    safetensors refuses as shared memory; call this before saving.  The next forward fuses again."""
+    for module in model.modules():
+        for name, group in (("_qkv", ("q_proj", "k_proj", "v_proj")), ("_gate_up", ("gate_proj", "up_proj"))):
+            if module.__dict__.pop(name, None) is not None:
+                for lin in group:
+                    w = getattr(module, lin).weight
+                    w.data = w.data.clone()
+
+
 class LlamaRMSNorm(nn.Module):
     def __init__(self, hidden_size: int, eps: float = 1e-6) -> None:
         super().__init__()

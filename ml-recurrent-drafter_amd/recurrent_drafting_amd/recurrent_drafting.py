@@ -32,7 +32,7 @@ import torch
 import torch.distributions as dist
 import transformers
 
-from . import acceptance, attention, gemm_tuning, kv_cache, modeling_drafter, modeling_llama, stats, tree_attention
+from . import acceptance, attention, kv_cache, modeling_drafter, modeling_llama, stats, tree_attention
 from .acceptance import (  # noqa: F401  (re-exported: the reference's helper names)
     _choose_from_candidates,
     _count_left_paddings,
@@ -144,7 +144,6 @@ class RecurrentDrafting(torch.nn.Module):
         super().__init__()
         self.llm = llm
         self.drafter = drafter
-        gemm_tuning.load()  # kernel selection table for the dense layers' GEMMs (no-op without one)
         # True: the decode loop leaves the KV cache rows where they are when the ids are re-aligned
         # (kv_cache.Cache.rows_in_place); False: it moves them every step, as the reference does.
         self.kv_rows_in_place = True

@@ -54,5 +54,6 @@ def test_tuned_gemm_agrees_with_the_default_choice():
     assert n == 0 or tunable.is_enabled()
     # another kernel sums in another order: bf16 rounding of the result, nothing more
     assert (got - want).abs().max() <= 2e-2 * want.abs().max()
-    if not was and n == 0:
-        tunable.enable(False)
+    # leave the process as it was found: the other tests run with torch's default choice
+    tunable.enable(was)
+    gemm_tuning._loaded = None
