@@ -8,12 +8,16 @@ Pin status
                          row 3 shows the first-maximum rule), maximality invariant
   greedy_next_input      pinned: property of recurrent_drafting_test.py:11-31
   sample_choose          pinned: brute-force leading-run count with injected uniforms, the recipe of
-                         mlx/recurrent_drafting_test.py:176-204; degenerate p>=q accepts everything
+                         mlx/recurrent_drafting_test.py:176-204; degenerate p>=q accepts everything;
+                         reference vectors of _choose_from_candidates under a recorded torch.rand
+                         (tests/golden/reference_vectors.json, "choose_from_candidates")
   residual_probs         pinned: one-hot LLM distribution makes the draw deterministic
-                         (mlx/recurrent_drafting_test.py:76-90); closed form relu(p-q)
+                         (mlx/recurrent_drafting_test.py:76-90); closed form relu(p-q); the probs the
+                         reference's _prepare_next_input hands to Categorical ("prepare_next_input")
   kv_unpack              pinned: docstring example of Cache.unpack (kv_cache_test.py:38-93)
   update_kv_and_ids      pinned: docstring worked example (recurrent_drafting.py:142-160), live-region
                          invariant, and B>1 ragged vectors in tests/golden/reference_vectors.json
+                         ("kv_update", and "accept_candidate_tokens" for the sampling caller)
 """
 
 from __future__ import annotations

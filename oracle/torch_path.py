@@ -13,6 +13,9 @@ with Hugging Face Llama / ReDrafter parameter names).
   beam_search                  recurrent_drafting/modeling_drafter.py:133-232
   greedy_choose, realign       recurrent_drafting/recurrent_drafting.py:114-232, :468-496
   generate_greedy              recurrent_drafting/recurrent_drafting.py:596-705
+  sample_choose, residual_distribution, sampling_step, generate_sampling
+                               recurrent_drafting/recurrent_drafting.py:75-111, :271-343, :423-430,
+                               :499-556 (torch.rand and Categorical.sample supplied by the caller)
 
 Pin status (tests/test_oracle_torch_path.py): pack/unpack/realign/greedy_choose are checked against
 tree_oracle / accept_oracle and directly against the reference's literals and vectors; beam_search
@@ -20,6 +23,13 @@ against fp_oracle.beam_search_chain; llama_forward, prefill and the loop as a wh
 the reference's own greedy token streams (tests/golden/reference_vectors.json, "end_to_end": five
 tiny float32 models incl. left-padded prompts and pairs whose drafts get accepted), which
 generate_greedy reproduces token for token.
+The sampling half (tests/test_oracle_sampling_vectors.py) is pinned by vectors the reference
+produced with its randomness replaced (torch.rand a recorded tensor / a fixed CPU stream,
+Categorical.sample the mode of the probs it is given): sample_choose against
+_choose_from_candidates, residual_distribution bit for bit against the probs _prepare_next_input
+hands to Categorical, both + realign against _accept_candidate_tokens (whole cache tensors), and
+generate_sampling (prefill draw, T != 1, left pads, accepted drafts) against three sampling token
+streams of the reference's own loop ("sampling_end_to_end").
 Tie rule of the beam search: `tie="stable"` (lowest flat index, the documented rule) or
 `tie="topk"` (torch.topk, whatever order it yields; used only when timing the CPU baseline).
 """

@@ -1,0 +1,111 @@
+"""Pins the speculative-sampling half of the oracle against vectors the upstream reference produced
+(tests/golden/make_reference_vectors.py): _choose_from_candidates under a recorded torch.rand,
+_prepare_next_input with the probs handed to Categorical recorded and its mode drawn,
+_accept_candidate_tokens end to end, and whole sampling token streams of the tiny float32 models."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import accept_oracle as Acc
+from oracle import torch_path as P
+
+sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
+import tiny_models as tm  # noqa: E402
+
+
+def f32(flat, *shape):
+    return torch.tensor(flat, dtype=torch.float32).reshape(*shape)
+
+
+def test_choose_from_candidates_reference_vectors(ref_vectors):
+    accepted = 0
+    for c in ref_vectors["choose_from_candidates"]:
+        B, W, L, V = c["B"], c["W"], c["L"], c["V"]
+        beams = torch.tensor(c["beams"])
+        log_p, log_q, u = f32(c["log_p"], B, W, L, V), f32(c["log_q"], B, W, L - 1, V), f32(c["uniforms"], B, W, L - 1)
+        n, s = P.sample_choose(beams, log_p, log_q, u)
+        assert n.tolist() == c["n_tokens_in_seq"] and s.tolist() == c["seq_in_beam"]
+        # the loop oracle computes the ratio in float32 as well when fed float32
+        n2, s2 = Acc.sample_choose(beams.numpy(), log_p.numpy(), log_q.numpy(), u.numpy())
+        assert n2.tolist() == c["n_tokens_in_seq"] and s2.tolist() == c["seq_in_beam"]
+        accepted += sum(c["n_tokens_in_seq"])
+    assert accepted > 10  # the vectors exercise runs of accepted tokens, not only rejections
+
+
+def test_prepare_next_input_reference_vectors(ref_vectors):
+    for c in ref_vectors["prepare_next_input"]:
+        B, W, L, V, H = c["B"], c["W"], c["L"], c["V"], c["H"]
+        log_p, log_q = f32(c["log_p"], B, W, L, V), f32(c["log_q"], B, W, L - 1, V)
+        hidden = f32(c["hidden"], B, W, L, H)
+        s, n = torch.tensor(c["seq_in_beam"]), torch.tensor(c["n_tokens_in_seq"])
+        want = f32(c["probs"], B, V)
+        got = P.residual_distribution(log_q, log_p, s, n)
+        assert torch.equal(got, want)  # the same float32 torch ops: bit-identical
+        assert got.argmax(-1).tolist() == c["next_tokens"]
+        got_np = Acc.residual_probs(log_q.numpy(), log_p.numpy(), s.numpy(), n.numpy())
+        assert np.allclose(got_np, want.numpy(), rtol=1e-6, atol=1e-9)
+        rows = torch.arange(B)
+        assert torch.equal(hidden[rows, s, n], f32(c["state"], B, H))
+        assert (L - 1) in c["n_tokens_in_seq"]  # a whole-beam row is among them
+
+
+def test_accept_candidate_tokens_reference_vectors(ref_vectors):
+    for c in ref_vectors["accept_candidate_tokens"]:
+        sh = c["shape"]
+        B, W, L, V, H = sh["B"], sh["W"], sh["L"], sh["V"], sh["H"]
+        T = c["temperature"]
+        beams = torch.tensor(c["beams"])
+        logits, log_q = f32(c["logits"], B, W, L, V), f32(c["log_q"], B, W, L - 1, V)
+        hidden, u = f32(c["hidden"], B, W, L, H), f32(c["uniforms"], B, W, L - 1)
+        log_p = (logits / T).log_softmax(dim=-1)
+        n, s = P.sample_choose(beams, log_p, log_q, u)
+        assert n.tolist() == c["n_tokens_in_seq"]
+        cache = P.Cache(B, sh["max_len"], sh["layers"], sh["heads"], sh["D"], torch.float32, "cpu")
+        cache.data.copy_(torch.tensor(c["cache_in"], dtype=torch.float32).reshape(cache.data.shape))
+        cache.set_length(sh["prev"] + W * L)
+        ids = P.realign(torch.tensor(c["input_ids"]), n, s, beams, cache, 0)
+        assert ids.tolist() == c["new_ids"] and cache.length[0][0] == c["new_length"]
+        assert cache.data.flatten().long().tolist() == c["cache_out"]
+        probs = P.residual_distribution(log_q, log_p, s, n)
+        assert torch.equal(probs, f32(c["probs"], B, V))
+        assert probs.argmax(-1).tolist() == c["next_tokens"]
+        assert torch.equal(hidden[torch.arange(B), s, n], f32(c["state"], B, H))
+        # NumPy loop oracle on the same case
+        cache_np = np.array(c["cache_in"], dtype=np.float32).reshape(tuple(cache.data.shape))
+        ids_np, M = Acc.update_kv_and_ids(np.array(c["input_ids"]), n.numpy(), s.numpy(), beams.numpy(), cache_np, 0)
+        assert ids_np.tolist() == c["new_ids"] and M == c["new_length"]
+        assert cache_np.astype(np.int64).flatten().tolist() == c["cache_out"]
+
+
+def _models(llama_sd, drafter_sd):
+    import recurrent_drafting_amd as rd
+    from transformers.models.llama.configuration_llama import LlamaConfig
+
+    llm = rd.modeling_llama.LlamaForCausalLM(LlamaConfig(**tm.LLAMA))
+    drafter = rd.modeling_drafter.Drafter(rd.configuration_drafter.DrafterConfig(**tm.DRAFTER))
+    llm.load_state_dict(llama_sd, strict=False)
+    drafter.load_state_dict(drafter_sd)
+    return llm.eval(), drafter.eval()
+
+
+@pytest.mark.parametrize("case_index", [0, 1, 2])
+def test_sampling_streams_match_the_reference(ref_vectors, case_index):
+    """The reference's own sampling decode loop (CPU, float32; torch.rand a fixed stream, the
+    categorical draw replaced by the mode) produced these token streams."""
+    case = ref_vectors["sampling_end_to_end"][case_index]
+    c = case["config"]
+    if c.get("markov"):
+        llama_sd, drafter_sd = tm.markov(c["seed"])
+    else:
+        llama_sd, drafter_sd = tm.draw(tm.llama_shapes(), c["seed"]), tm.draw(tm.drafter_shapes(), c["seed"] + 1000)
+    llm, drafter = _models(llama_sd, drafter_sd)
+    ids = tm.prompt(c["batch"], c["prompt_len"], tm.LLAMA["vocab_size"], c["seed"], c["left_pads"])
+    g = torch.Generator().manual_seed(c["rand_seed"])
+    out = list(P.generate_sampling(
+        llm, drafter, ids, c["prompt_len"] + c["new_tokens"], c["W"], c["L"], c["temperature"],
+        lambda shape: torch.rand(tuple(shape), generator=g), lambda p: p.argmax(-1), pad=0, eos=None))
+    assert [t.tolist() for t, _ in out] == case["steps"]
+    assert [float(n.float().mean()) for _, n in out] == pytest.approx(case["avg_num_accepted"])
