@@ -10,7 +10,7 @@ from __future__ import annotations
 import contextlib
 import dataclasses
 import time
-from typing import Any, Dict, Generator, List
+from typing import Any, Dict, Generator, List, Tuple
 
 import torch
 
@@ -86,21 +86,61 @@ class TableStats:
         return self.avg_token_per_step / self.avg_step_time
 
 
-def summarize(ledger: Ledger, batch_size: int, candidate_len: int) -> TableStats:
-    """Means over all recorded steps (stats.py:158-215)."""
-    n_steps, tokens = 0, 0.0
+@dataclasses.dataclass
+class PlotStats:
+    sorted_steps: List[int]
+    sorted_num_tokens_step: List[float]  # batch tokens per step index, averaged over the generations
+    sorted_input_lengths: List[int]
+    sorted_num_tokens_input_length: List[float]  # the same, grouped by the step's input length
+    acceptance_rate: float
+
+
+def summarize(ledger: Ledger, batch_size: int, candidate_len: int) -> Tuple[TableStats, PlotStats]:
+    """(TableStats, PlotStats) over every recorded step of every generation (stats.py:158-215).
+
+    A step that accepted `a` drafted tokens per sequence on average produced batch_size * (a + 1)
+    tokens; the acceptance rate is the share of the candidate_len drafted tokens that were kept."""
+    per_step: Dict[int, List[float]] = {}
+    per_length: Dict[int, List[float]] = {}
     times = {"generate_candidates": [], "verify_candidates": [], "accept_candidate_tokens": []}
     for rec in ledger.records:
-        for accepted in rec.get("avg_num_accepted", []):
-            n_steps += 1
-            tokens += batch_size * (float(accepted) + 1)
+        accepted = rec.get("avg_num_accepted", [])
+        for step, a in zip(rec.get("step", []), accepted):
+            per_step.setdefault(step, []).append(batch_size * (float(a) + 1))
+        for length, a in zip(rec.get("input_id_length", []), accepted):
+            per_length.setdefault(length, []).append(batch_size * (float(a) + 1))
         for key in times:
             times[key] += rec["wall_times"].get(key, [])
-    per_step = tokens / max(n_steps, 1)
+    steps = sorted(per_step)
+    lengths = sorted(per_length)
+    n_steps = sum(len(per_step[i]) for i in steps)
+    tokens = sum(sum(per_step[i]) for i in steps)
+    per_step_tokens = tokens / max(n_steps, 1)
+    rate = 100.0 * (per_step_tokens - batch_size) / batch_size / candidate_len
     mean = {k: (sum(v) / len(v) if v else 0.0) for k, v in times.items()}
-    return TableStats(
-        per_step / batch_size,
-        100.0 * (per_step - batch_size) / batch_size / candidate_len,
+    table = TableStats(
+        per_step_tokens / batch_size, rate,
         mean["generate_candidates"], mean["verify_candidates"], mean["accept_candidate_tokens"],
         sum(mean.values()),
     )
+    plot = PlotStats(
+        steps, [sum(per_step[i]) / len(per_step[i]) for i in steps],
+        lengths, [sum(per_length[i]) / len(per_length[i]) for i in lengths], rate,
+    )
+    return table, plot
+
+
+def draw_table(title: str, ts: TableStats) -> None:
+    """Prints the summary with the reference's row labels (stats.py:218-241)."""
+    rows = [
+        ("Average number of tokens per step:", f"{ts.avg_token_per_step:.4f}"),
+        ("Average draft head acceptance rate (%):", f"{ts.acceptance_rate:.4f}"),
+        ("generate_candidates:", f"{ts.avg_generate_candidates:.4f}"),
+        ("verify_candidates:", f"{ts.avg_verify_candidates:.4f}"),
+        ("accept_candidate_tokens:", f"{ts.avg_accept_candidate_tokens:.4f}"),
+        ("Tokens/second", f"{ts.tokens_per_second:.4f}"),
+    ]
+    width = max(len(label) for label, _ in rows)
+    print(f"Title: {title}")
+    for label, value in rows:
+        print(f"{label:<{width}}  {value:>12}")

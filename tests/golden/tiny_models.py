@@ -70,23 +70,26 @@ def prompt(batch: int, length: int, vocab: int, seed: int, left_pads=()) -> torc
     return ids
 
 
-def markov(seed: int, gain: float = 40.0):
+def markov(seed: int, gain: float = 40.0, llama_cfg=LLAMA, drafter_cfg=DRAFTER, mix: float = 0.0):
     """(llama_state, drafter_state) of a toy pair in which the drafter usually agrees with the LLM,
-    so that decoding accepts drafted tokens: attention and MLP outputs are zeroed (the residual
-    stream is the token embedding, the next token depends on the last token only), embeddings are
-    non-negative, and the drafter decodes silu(gain * embedding) with the LLM's own lm_head."""
-    llama = draw(llama_shapes(), seed)
+    so that decoding accepts drafted tokens: embeddings are non-negative, the drafter decodes
+    silu(gain * embedding) with the LLM's own lm_head, and the attention and MLP outputs of the LLM
+    are scaled by `mix`.  mix = 0 (the default): the residual stream is the token embedding, the
+    next token depends on the last token only and the drafter is nearly always right; with a small
+    mix the context moves the LLM's choice now and then, so accepted lengths become ragged and
+    the attention output matters for the tokens."""
+    llama = draw(llama_shapes(llama_cfg), seed)
     llama["model.embed_tokens.weight"] = llama["model.embed_tokens.weight"].abs()
     for name in llama:
         if name.endswith("o_proj.weight") or name.endswith("down_proj.weight"):
-            llama[name] = torch.zeros_like(llama[name])
-    drafter = draw(drafter_shapes(), seed + 1000)
-    h = DRAFTER["hidden_size"]
+            llama[name] = llama[name] * mix
+    drafter = draw(drafter_shapes(drafter_cfg), seed + 1000)
+    h = drafter_cfg["hidden_size"]
     drafter["rnn_w.weight"] = torch.eye(h) * gain
     drafter["rnn_u.weight"] = torch.zeros(h, h)
     drafter["rnn_u.bias"] = torch.zeros(h)
     drafter["lm_head.0.linear.weight"] = torch.zeros_like(drafter["lm_head.0.linear.weight"])
     drafter["lm_head.0.linear.bias"] = torch.full_like(drafter["lm_head.0.linear.bias"], -30.0)
     drafter["lm_head.1.weight"] = torch.cat(
-        [torch.zeros(DRAFTER["vocab_size"], h), llama["lm_head.weight"] * 8.0], dim=1)
+        [torch.zeros(drafter_cfg["vocab_size"], h), llama["lm_head.weight"] * 8.0], dim=1)
     return llama, drafter

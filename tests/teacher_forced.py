@@ -1,0 +1,286 @@
+"""Teacher-forced comparison of the fused HIP decode loop with the torch restatement, step by step.
+
+bf16 logits of two implementations tie within an ulp or two for a share of the positions, so two
+correct decoders drift apart after a few tokens (the reference documents this for its own two
+decoders, docs/parity_check.md:77-98).  A free-running comparison of token streams therefore says
+nothing in bf16; what can be pinned is every step given the same inputs.  `run` drives
+RecurrentDrafting.generate and, at every step, hands the state the HIP loop went into the step
+with (token ids, drafter context, first token, KV cache contents) to oracle/torch_path on the
+same GPU, then compares what came out:
+
+  beams            oracle beam search on the same context and token (same bf16 torch GEMMs)
+  tree             packed tokens, unpacker, mask, position offsets of the HIP beams: bit-exact
+  packed logits    against the float32 restatement (bf16 weights upcast), within `tol` of the
+                   logits' scale; the restatement run in bf16 with stock torch ops is measured
+                   against the same float32 figures, as the yardstick for a bf16 implementation
+  argmax           a token may differ from the float32 argmax only where the float32 margin
+                   between the two tokens is below the tolerance
+  acceptance       n_tokens_in_seq / seq_in_beam from the HIP argmax tokens: bit-exact
+  next state       new ids bit-exact; next token = the HIP argmax at the chosen slot; drafter
+                   context within tolerance; KV rows: kept rows bit-identical, accepted rows
+                   bit-identical to the rows the HIP forward wrote, which in turn agree with the
+                   restatement's K/V within tolerance
+
+The functions of the package are observed by wrapping module attributes; nothing in the package
+knows about this file.
+"""
+
+from __future__ import annotations
+
+import copy
+import dataclasses
+import unittest.mock as mock
+from typing import Callable, List, Optional
+
+import numpy as np
+import torch
+
+from oracle import accept_oracle as Acc
+from oracle import torch_path as P
+
+
+@dataclasses.dataclass
+class StepReport:
+    step: int
+    prev: int
+    n_q: int
+    rows: int
+    beams_equal: bool
+    beams_shared: float  # share of the HIP beams that are among the restatement's beams of the same row
+    logits_err: float  # max |HIP - float32 restatement| / scale
+    logits_err_bf16_torch: float  # the same for the bf16 restatement (stock torch ops)
+    flips: int  # packed positions whose argmax differs from the float32 argmax
+    worst_flip_margin: float  # largest float32 margin among them / scale
+    n_tokens: List[int]
+    shifts: List[int]  # cache row shifts going into the step
+    context_err: float
+    kv_err: float
+
+
+def _snapshot(cache, length: int):
+    """Copy of the cache in the reference's layout (column c of row b in cache row c)."""
+    from recurrent_drafting_amd import kv_cache
+
+    n_layers, _, B, H, max_len, D = cache._cache.shape
+    snap = kv_cache.Cache(B, max_len, n_layers, H, D, cache._cache.dtype, cache._cache.device)
+    snap._storage.copy_(cache._storage)
+    snap.shift.copy_(cache.shift)
+    snap._rows_in_place = True
+    snap._shifted = True
+    snap.set_length(length)
+    snap.materialize()
+    torch.cuda.synchronize()
+    return snap._cache
+
+
+def forced_acceptance(seed: int) -> Callable:
+    """Replaces the acceptance decision by random accepted lengths and beams (the token streams
+    then mean nothing, but rows shift by different amounts at every step)."""
+    gen = torch.Generator().manual_seed(seed)
+
+    def force(beams, llm_tokens, unpacker, n, s, nxt, last):
+        B, W, L = beams.shape
+        n = torch.randint(0, L, (B,), generator=gen).to(beams.device)
+        s = torch.randint(0, W, (B,), generator=gen).to(beams.device)
+        rows = torch.arange(B, device=beams.device)
+        last = unpacker[rows, s, n]
+        nxt = llm_tokens[rows, last]
+        return n, s, nxt, last
+    return force
+
+
+def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int = 0,
+        tol: float = 2e-2, force: Optional[Callable] = None, check_from: int = 0,
+        log: Optional[Callable] = None) -> List[StepReport]:
+    """Runs `steps` decode steps of the fused loop; steps >= check_from are compared with the
+    restatement.  Raises AssertionError on the first violation; returns the per-step reports."""
+    import recurrent_drafting_amd as rd
+    from recurrent_drafting_amd import acceptance, tree_attention
+
+    dev = ids.device
+    llm32 = copy.deepcopy(llm).float()  # bf16 weights upcast (the drafter is compared in its own dtype)
+    model = rd.RecurrentDrafting(llm, drafter)
+    seen = {}
+    real_mask, real_argmax = tree_attention.build_mask, acceptance.argmax_rows
+    real_accept, real_realign = acceptance.greedy_accept, acceptance.realign_enqueue
+    real_draft = drafter.beam_search_candidates
+
+    def w_mask(tree, padding_mask, pad_value=0):
+        out = real_mask(tree, padding_mask, pad_value)
+        seen.update(tree=tree, ids=padding_mask, mask=out)
+        return out
+
+    def w_argmax(logits):
+        out = real_argmax(logits)
+        if "tree" in seen:  # (the prefill calls it too, before any tree exists)
+            seen.update(logits=logits, argmax=out)
+        return out
+
+    def w_accept(beams, llm_tokens, unpacker=None):
+        n, s, nxt, last = real_accept(beams, llm_tokens, unpacker)
+        natural = (n, s)
+        if force is not None:
+            n, s, nxt, last = force(beams, llm_tokens, unpacker, n, s, nxt, last)
+        seen.update(beams=beams, llm_tokens=llm_tokens, unpacker=unpacker, n=n, s=s, natural=natural,
+                    next_tokens=nxt, last_slot=last)
+        return n, s, nxt, last
+
+    def w_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker=None):
+        seen.update(cache=cache, shift=cache.shift.clone(),
+                    snap=_snapshot(cache, cache.sliced[0][0].length))
+        return real_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker)
+
+    drafts = []  # draft k feeds step k; it is queued while step k-1 is being finished
+
+    def w_draft(context, init_token, embeddings, beam_shape, return_log_probs=True):
+        out = real_draft(context, init_token, embeddings, beam_shape, return_log_probs=return_log_probs)
+        drafts.append(dict(context=context.clone(), init=init_token.clone(), beams=out[0]))
+        return out
+
+    reports: List[StepReport] = []
+    prev_step = None  # what the previous step left for the cache comparison
+    with mock.patch.object(tree_attention, "build_mask", w_mask), \
+            mock.patch.object(acceptance, "argmax_rows", w_argmax), \
+            mock.patch.object(acceptance, "greedy_accept", w_accept), \
+            mock.patch.object(acceptance, "realign_enqueue", w_realign), \
+            mock.patch.object(drafter, "beam_search_candidates", w_draft):
+        stream = model.generate(rd.stats.Ledger(), ids, max_length, rd.BeamShape(W, L),
+                                rd.SamplingArgs(1.0, True), rd.SpecialTokens(pad, None))
+        for k in range(steps):
+            seen.pop("tree", None)
+            try:
+                out = next(stream)
+            except StopIteration:
+                break
+            assert len(drafts) == k + 2
+            st = dict(seen)
+            if k >= check_from:
+                with torch.inference_mode():
+                    reports.append(_check_step(k, st, drafts[k], drafts[k + 1], out, max_length, llm, llm32,
+                                               drafter, W, L, pad, tol, prev_step,
+                                               natural_accept=force is None))
+                if log is not None:
+                    log(reports[-1])
+            prev_step = dict(snap=st["snap"], tree=st["tree"], unpacker=st["unpacker"], n=st["n"], s=st["s"],
+                             ids=st["ids"], prev=st["ids"].shape[1])
+        stream.close()
+    return reports
+
+
+def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafter, W, L, pad, tol, prev_step,
+                natural_accept: bool) -> StepReport:
+    tree, ids, beams = st["tree"], st["ids"], st["beams"]
+    dev = ids.device
+    B, prev = ids.shape
+    n_q, total = tree.n, tree.total
+    rows = tree.rows()
+    slot_of_row = rows.index[:total]  # slot b * n_q + t of every packed row that exists
+    assert torch.equal(beams, draft_in["beams"])
+
+    # -- draft: the restatement's beam search on the same context and token -----------------------
+    with torch.inference_mode():
+        o_beams, _ = P.beam_search(drafter, llm.model.embed_tokens, draft_in["context"], draft_in["init"], W, L,
+                                   want_log_probs=False)
+    beams_equal = bool(torch.equal(o_beams, beams))
+    # bf16 beam scores tie or nearly tie in numbers (the restatement computes the first iteration for
+    # all W copies of the one live beam, the package once per row: other GEMM shapes, other rounding),
+    # so the two searches may keep different candidates at the margin; the share in common is reported
+    beams_shared = float((beams[:, :, None, :] == o_beams[:, None, :, :]).all(-1).any(-1).float().mean())
+    assert torch.equal(beams[:, :, 0], draft_in["init"][:, None].expand(B, W))
+
+    # -- tree of the HIP beams: bit-exact ----------------------------------------------------------
+    o_packed, o_unpacker, o_mask, o_off = P.pack(beams, (ids != pad).to(ids.dtype))
+    assert o_packed.shape[1] == n_q, (o_packed.shape, n_q)
+    assert torch.equal(tree.unpacker, o_unpacker) and torch.equal(tree.packed_beams, o_packed)
+    assert torch.equal(tree.position_offsets, o_off) and torch.equal(st["mask"], o_mask)
+    counts = tree.counts[:B].long()
+    assert int(counts.sum()) == total and int(counts.max()) == n_q
+    exists = (torch.arange(n_q, device=dev)[None, :] < counts[:, None]).flatten()
+    assert torch.equal(exists.nonzero().flatten(), slot_of_row)
+
+    # -- verify forward: float32 restatement (and the bf16 one as the yardstick) on the same cache ---
+    snap = st["snap"]  # (layers, 2, B, H, max_len, D), columns in place, tree rows at [prev, prev+n_q)
+    pos = (prev - P.count_left_pads(ids, pad))[:, None] + o_off
+    n_layers, _, _, Hkv, max_len, D = snap.shape
+
+    def restate(model, dtype):
+        cache = P.Cache(B, prev + n_q, n_layers, Hkv, D, dtype, dev)
+        cache.data[:, :, :, :, :prev] = snap[:, :, :, :, :prev].to(dtype)
+        cache.set_length(prev)
+        with torch.inference_mode():
+            logits, hidden = P.llama_forward(model, o_packed, o_mask, pos, cache)
+        return logits.flatten(0, 1)[slot_of_row], hidden.flatten(0, 1)[slot_of_row], cache
+
+    want, want_hidden, o_cache = restate(llm32, torch.float32)
+    torch_bf16, _, _ = restate(llm, snap.dtype)
+    got = st["logits"][:total].float()
+    scale = float(want.abs().max())
+    logits_err = float((got - want).abs().max()) / scale
+    yard = float((torch_bf16 - want).abs().max()) / scale
+    assert logits_err <= tol, f"step {k}: packed logits off by {logits_err:.3g} of their scale"
+    assert logits_err <= 3 * yard + 1e-3, \
+        f"step {k}: HIP logits {logits_err:.3g} off, stock bf16 torch only {yard:.3g}"
+
+    # -- argmax: flips only inside the tolerance band ---------------------------------------------------
+    hip_tok = st["argmax"][:total]
+    assert torch.equal(st["llm_tokens"].flatten()[slot_of_row], hip_tok)
+    o_tok = want.argmax(dim=-1)
+    flipped = (hip_tok != o_tok).nonzero().flatten()
+    margins = (want[flipped, o_tok[flipped]] - want[flipped, hip_tok[flipped]]) / scale
+    worst = float(margins.max()) if flipped.numel() else 0.0
+    assert worst <= tol, f"step {k}: argmax flip with float32 margin {worst:.3g} of the scale"
+    # and the HIP argmax is the first maximum of the HIP logits themselves
+    assert torch.equal(hip_tok, st["logits"][:total].float().argmax(dim=-1))
+
+    # -- acceptance from the HIP tokens: bit-exact -------------------------------------------------------
+    llm_bwl = st["llm_tokens"].gather(1, o_unpacker.view(B, -1)).view(B, W, L)
+    o_n, o_s = P.greedy_choose(beams, llm_bwl)
+    nat_n, nat_s = st["natural"]
+    assert torch.equal(o_n, nat_n) and torch.equal(o_s, nat_s)
+    n, s = st["n"], st["s"]
+    if natural_accept:
+        assert torch.equal(n, nat_n) and torch.equal(s, nat_s)
+    b_idx = torch.arange(B, device=dev)
+    assert torch.equal(st["next_tokens"], llm_bwl[b_idx, s, n])
+    assert torch.equal(st["last_slot"], o_unpacker[b_idx, s, n])
+
+    # -- next state --------------------------------------------------------------------------------------
+    dummy = np.zeros((1, 1, B, 1, prev + W * L, 1), dtype=np.float32)
+    o_ids, M = Acc.update_kv_and_ids(ids.cpu().numpy(), n.cpu().numpy(), s.cpu().numpy(), beams.cpu().numpy(),
+                                     dummy, pad)
+    assert out.shape[1] == min(M + 1, max_length)
+    if M + 1 <= max_length:  # (otherwise the yielded tokens are cut at max_length)
+        assert np.array_equal(out[:, :-1].cpu().numpy(), o_ids)
+        assert torch.equal(out[:, -1], st["next_tokens"])
+    assert torch.equal(draft_next["init"], st["next_tokens"])
+    ctx_want = want_hidden.new_zeros((B * n_q, want_hidden.shape[1])).index_copy_(0, slot_of_row, want_hidden)
+    ctx_want = ctx_want[b_idx * n_q + st["last_slot"]]
+    ctx_scale = float(want_hidden.abs().max())
+    context_err = float((draft_next["context"].float() - ctx_want).abs().max()) / ctx_scale
+    assert context_err <= tol, f"step {k}: drafter context off by {context_err:.3g}"
+
+    # -- KV cache: the rows the HIP forward wrote against the restatement's; the rows kept and moved ----
+    hip_new = snap[:, :, :, :, prev : prev + n_q].float()
+    o_new = o_cache.data[:, :, :, :, prev : prev + n_q]
+    live = (torch.arange(n_q, device=dev)[None, :] < counts[:, None])[None, None, :, None, :, None]
+    kv_scale = float(o_new.abs().max())
+    kv_err = float(torch.where(live, hip_new - o_new, torch.zeros_like(o_new)).abs().max()) / kv_scale
+    assert kv_err <= tol, f"step {k}: appended K/V rows off by {kv_err:.3g}"
+    if prev_step is not None:
+        # what the previous step kept: its live columns, then the accepted rows of its chosen beam,
+        # bit for bit, at the columns the re-alignment gave them
+        p = prev_step
+        old_pads = P.count_left_pads(p["ids"], pad)
+        new_pads = P.count_left_pads(ids, pad)
+        for b in range(B):
+            keep = p["prev"] - int(old_pads[b])
+            lo = int(new_pads[b])
+            assert torch.equal(snap[:, :, b, :, lo : lo + keep], p["snap"][:, :, b, :, int(old_pads[b]) : p["prev"]]), \
+                f"step {k}: kept cache rows of row {b} changed"
+            for j in range(int(p["n"][b]) + 1):
+                src = p["prev"] + int(p["unpacker"][b, int(p["s"][b]), j])
+                assert torch.equal(snap[:, :, b, :, lo + keep + j], p["snap"][:, :, b, :, src]), \
+                    f"step {k}: accepted cache row {j} of row {b}"
+            assert lo + keep + int(p["n"][b]) + 1 == prev
+    return StepReport(k, prev, n_q, total, beams_equal, beams_shared, logits_err, yard, int(flipped.numel()), worst,
+                      n.tolist(), st["shift"].tolist(), context_err, kv_err)
