@@ -86,7 +86,8 @@ def gpu_run(steps: int, warmup: int):
     torch.cuda.synchronize()
     log(f"[bench] models on {torch.cuda.get_device_name(0)} in {time.perf_counter() - t0:.1f}s")
     model = rd.RecurrentDrafting(llm, drafter)
-    rd.gemm_tuning.load()  # opt-in kernel selection table for the dense layers' GEMMs (look-up only)
+    n_tuned = rd.gemm_tuning.load()  # opt-in kernel selection table for the dense layers' GEMMs (look-up only)
+    log(f"[bench] GEMM kernel selection table: {n_tuned} entries in effect")
     ids = prompts(dev)
     max_length = PROMPT + NEW_TOKENS
 

@@ -298,16 +298,18 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
  * views View.cat returns (kv_cache.py:24-31).  bf16 with head_dim 128 runs on the MFMA kernel
  * (needs 16-byte aligned q/k/v, strides that are multiples of 8 elements, and the workspace);
  * everything else (more than 128 heads included), or force_generic != 0, runs on the generic
- * kernel (head_dim <= 256).  The plan's arrival counters (its tail) are counted up and left at
- * zero by every call; calls that share a plan must not overlap in time.
+ * kernel (head_dim <= 256).  The plan is READ AND WRITTEN: its arrival counters (its tail) are
+ * counted up and left at zero by every call, so calls that share a plan must run one after the
+ * other on one stream (the layers of a forward do); a plan per stream otherwise.
  * row_start (batch + 1 int32 on the device, or NULL): packed query rows, as in rd_rope_append:
  * query t of batch row b is row row_start[b] + t of q and of out (sequence stride; their batch
  * strides are unused), queries t >= row_start[b+1] - row_start[b] are neither read nor written.
  * The mask bits keep their (batch, n_q) rows.
  * kv_row_shift (rd_attn_prepare; batch int32 on the device, or NULL): recorded in the plan; the
  * attention then reads key column c of row b from cache row c - kv_row_shift[b] of k and v (see
- * rd_realign_plan).  Whole 64-key tiles are loaded, so up to 63 rows below a row's first key are
- * touched: the caller keeps 64 rows of readable memory in front of the first slab.
+ * rd_realign_plan).  Only cache rows of keys that some query of the row attends to are read (the
+ * first and last 64-key tile of a row re-read its first / last such key in place of the others),
+ * so nothing is asked of the memory around a row's live cache rows.
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_attn_plan_ints(int batch, int n_q, int kv_len);
 RD_API size_t rd_attn_bits_words(int batch, int n_q, int kv_len);
@@ -321,7 +323,7 @@ RD_API int rd_verify_attention(const void* q, const int64_t* q_strides, const vo
                                const int64_t* k_strides, const void* v, const int64_t* v_strides,
                                void* out, const int64_t* o_strides, int dtype, int batch,
                                int n_heads, int n_kv_heads, int n_q, int kv_len, int head_dim,
-                               float scale, const uint64_t* bits, const int32_t* plan,
+                               float scale, const uint64_t* bits, int32_t* plan,
                                void* workspace, size_t workspace_bytes, int force_generic,
                                const int32_t* row_start, void* stream);
 

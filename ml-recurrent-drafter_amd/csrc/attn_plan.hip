@@ -1,9 +1,9 @@
 // Mask compression and work planning for the verification attention (gfx950).
 //   mask_bits_kernel   bool mask (batch, n_q, kv) -> one uint64 per (row, 64 keys); a wave reads 64
 //                      mask bytes coalesced and a ballot turns them into the word
-//   attn_plan_kernel   per batch row: first key any query attends to (whole 64-key tiles of left
-//                      padding are never loaded), split of the remaining keys into near-equal
-//                      chunks, and the chunk list sorted longest-first for dispatch
+//   attn_plan_kernel   per batch row: the span of keys that any query attends to (whole 64-key tiles
+//                      of left padding or behind the row's last tree slot are never loaded), split
+//                      of that span into near-equal chunks, and the chunk list sorted longest-first
 #include "attn_plan.h"
 
 namespace {
@@ -13,27 +13,32 @@ constexpr int kWaves = kThreads / 64;
 
 __global__ __launch_bounds__(kThreads) void mask_bits_kernel(
     const uint8_t* __restrict__ mask, int64_t stride_b, int64_t stride_q, int n_q, int kv_len,
-    int words, int fix_empty_rows, uint64_t* __restrict__ bits, int32_t* __restrict__ row_first) {
+    int words, int fix_empty_rows, uint64_t* __restrict__ bits, int32_t* __restrict__ row_first,
+    int32_t* __restrict__ row_last) {
   const int q = blockIdx.x, b = blockIdx.y;
   const uint8_t* row = mask + (int64_t)b * stride_b + (int64_t)q * stride_q;
   uint64_t* out = bits + ((int64_t)b * n_q + q) * words;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int first = kv_len;
+  int first = kv_len, last = -1;
   for (int w = wave; w < words; w += kWaves) {
     const int j = w * 64 + lane;
     const bool on = j < kv_len && row[j] != 0;
     const uint64_t word = __ballot(on);
     if (lane == 0) out[w] = word;
     if (word != 0) {
-      const int f = w * 64 + __builtin_ctzll(word);
+      const int f = w * 64 + __builtin_ctzll(word), l = w * 64 + 63 - __builtin_clzll(word);
       first = f < first ? f : first;
+      last = l > last ? l : last;
     }
   }
-  __shared__ int s_first[kWaves];
-  if (lane == 0) s_first[wave] = first;
+  __shared__ int s_first[kWaves], s_last[kWaves];
+  if (lane == 0) { s_first[wave] = first; s_last[wave] = last; }
   __syncthreads();
-  first = kv_len;
-  for (int w = 0; w < kWaves; ++w) first = s_first[w] < first ? s_first[w] : first;
+  first = kv_len; last = -1;
+  for (int w = 0; w < kWaves; ++w) {
+    first = s_first[w] < first ? s_first[w] : first;
+    last = s_last[w] > last ? s_last[w] : last;
+  }
   if (first == kv_len && fix_empty_rows) {
     // a query that attends to nothing attends to everything (finite-minimum bias semantics)
     for (int w = threadIdx.x; w < words; w += kThreads) {
@@ -41,11 +46,16 @@ __global__ __launch_bounds__(kThreads) void mask_bits_kernel(
       out[w] = rem >= 64 ? ~0ull : ((1ull << rem) - 1ull);
     }
     first = 0;
+    last = kv_len - 1;
   }
-  if (threadIdx.x == 0) row_first[(int64_t)b * n_q + q] = first;
+  if (threadIdx.x == 0) {
+    row_first[(int64_t)b * n_q + q] = first;
+    row_last[(int64_t)b * n_q + q] = last;
+  }
 }
 
 __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __restrict__ row_first,
+                                                             const int32_t* __restrict__ row_last,
                                                              int B, int n_q, int kv_len, int words,
                                                              int min_chunk, int max_splits,
                                                              int n_heads, int n_cu,
@@ -55,24 +65,32 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
                                                              int n_counters) {
   __shared__ int s_n_items;
   __shared__ int s_chunk;
+  extern __shared__ int s_span[];  // [2][B]: first key any query of the row attends to, last such key + 1
+  int* s_key_min = s_span;
+  int* s_key_end = s_span + B;
   for (int i = threadIdx.x; i < n_counters; i += kThreads) counters[i] = 0;
   int32_t* per_row = plan + RD_PLAN_HDR;
   int32_t* items = plan + RD_PLAN_HDR + 4 * B;
   // pass 1: per batch row, first attended key and number of splits
   // (one wave per batch row at a time: the minimum over its query rows)
   for (int b = threadIdx.x >> 6; b < B; b += kThreads / 64) {
-    int first = kv_len;
+    int first = kv_len, last = -1;
     for (int q = threadIdx.x & 63; q < n_q; q += 64) {
-      const int f = row_first[(int64_t)b * n_q + q];
+      const int f = row_first[(int64_t)b * n_q + q], l = row_last[(int64_t)b * n_q + q];
       first = f < first ? f : first;
+      last = l > last ? l : last;
     }
     for (int off = 32; off > 0; off >>= 1) {
-      const int o = __shfl_xor(first, off);
+      const int o = __shfl_xor(first, off), p = __shfl_xor(last, off);
       first = o < first ? o : first;
+      last = p > last ? p : last;
     }
     if ((threadIdx.x & 63) == 0) {
+      if (last < first) { first = kv_len - 1; last = kv_len - 1; }  // a row in which nobody attends to anything
       per_row[4 * b + 0] = (first / 64) * 64;
       per_row[4 * b + 3] = kv_shift ? kv_shift[b] : 0;  // cache row of key c is c - shift
+      s_key_min[b] = first;
+      s_key_end[b] = last + 1;
     }
   }
   __syncthreads();
@@ -81,7 +99,7 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
     // min_chunk.  Equal rows on a machine with batch*heads == compute units are then not split at
     // all (no partials to merge); ragged rows are cut so that the longest item is about one share.
     long long total = 0;
-    for (int b = 0; b < B; ++b) total += kv_len - per_row[4 * b + 0];
+    for (int b = 0; b < B; ++b) total += s_key_end[b] - per_row[4 * b + 0];
     long long share = (total * n_heads + n_cu - 1) / n_cu;
     share = (share + 63) / 64 * 64;
     s_chunk = (int)(share > min_chunk ? share : min_chunk);
@@ -89,8 +107,11 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
   __syncthreads();
   const int chunk = s_chunk;
   for (int b = threadIdx.x; b < B; b += kThreads) {
-    const int live = kv_len - per_row[4 * b + 0];
-    int splits = (live + chunk - 1) / chunk;
+    const int live = s_key_end[b] - per_row[4 * b + 0];
+    // an item may run an eighth over the share: a row a little longer than the share stays whole
+    // (cutting off a short remainder would cost it the partials, the fences and the merge, and
+    // would send the remainders into a second round of items behind the first)
+    int splits = (live + chunk - 1 - chunk / 8) / chunk;
     per_row[4 * b + 1] = splits < 1 ? 1 : (splits > max_splits ? max_splits : splits);
   }
   __syncthreads();
@@ -111,14 +132,14 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
     b = 0;
     while (b + 1 < B && per_row[4 * (b + 1) + 2] <= it) ++b;
     s = it - per_row[4 * b + 2];
-    const int begin = per_row[4 * b + 0], splits = per_row[4 * b + 1];
-    const int live = kv_len - begin;
+    const int begin = per_row[4 * b + 0], splits = per_row[4 * b + 1], end = s_key_end[b];
+    const int live = end - begin;
     int per = (live + splits - 1) / splits;
     per = (per + 63) / 64 * 64;
     lo = begin + s * per;
     hi = lo + per;
-    lo = lo < kv_len ? lo : kv_len;
-    hi = hi < kv_len ? hi : kv_len;
+    lo = lo < end ? lo : end;
+    hi = hi < end ? hi : end;
   };
   __shared__ int s_len[rd::kAttnSortLimit];
   const bool sorted = n_items <= rd::kAttnSortLimit;
@@ -142,12 +163,12 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
         rank += (olen > len) || (olen == len && o < it);
       }
     }
-    items[4 * rank + 0] = b;
-    items[4 * rank + 1] = lo;
-    items[4 * rank + 2] = hi;
-    // split index in the low 12 bits, the row's cache shift above them: the attention kernel then
-    // has everything it needs for its first loads from this one record
-    items[4 * rank + 3] = (s & 0xfff) | (per_row[4 * b + 3] * 4096);
+    int32_t* rec = items + RD_ITEM_INTS * rank;
+    rec[0] = b; rec[1] = lo; rec[2] = hi; rec[3] = s;
+    rec[4] = per_row[4 * b + 3];
+    rec[5] = s_key_min[b];
+    rec[6] = per_row[4 * b + 1];
+    rec[7] = s_key_end[b];
   }
 }
 
@@ -187,18 +208,17 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
   RD_REQUIRE(batch <= 65535 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
              "rd_attn_prepare: batch %d too large for kv_len %d", batch, kv_len);
   RD_REQUIRE(mask && bits && plan, RD_EINVAL, "rd_attn_prepare: null pointer");
-  RD_REQUIRE(rd::attn_max_splits(kv_len) <= 4095 && (!kv_row_shift || kv_len < (1 << 19)), RD_ELIMIT,
-             "rd_attn_prepare: kv_len %d is beyond what a work item record can describe", kv_len);
   RD_REQUIRE(mask_stride_q >= kv_len && mask_stride_b >= 0, RD_EINVAL,
              "rd_attn_prepare: mask_stride_q %lld < kv_len %d", (long long)mask_stride_q, kv_len);
   const int words = (kv_len + 63) / 64;
   const int max_splits = rd::attn_max_splits(kv_len);
-  int32_t* row_first = plan + RD_PLAN_HDR + 4 * (size_t)batch + 4 * (size_t)batch * max_splits;
+  int32_t* row_first = plan + RD_PLAN_HDR + 4 * (size_t)batch + RD_ITEM_INTS * (size_t)batch * max_splits;
+  int32_t* row_last = row_first + (size_t)batch * n_q;
   hipStream_t s = rd::as_stream(stream);
   { rd::ScopedTiming rd_t("mask_bits_kernel", s); hipLaunchKernelGGL(mask_bits_kernel, dim3(n_q, batch), dim3(kThreads), 0, s, mask, mask_stride_b,
-                     mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first); }
+                     mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first, row_last); }
   if (int e = rd::check_launch("rd_attn_prepare(bits)")) return e;
-  { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 0, s, row_first, batch, n_q, kv_len,
+  { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 2 * batch * sizeof(int), s, row_first, row_last, batch, n_q, kv_len,
                      words, rd::kAttnChunk, max_splits, n_heads, compute_units(), kv_row_shift, plan,
                      plan + rd::attn_counter_offset(batch, n_q, kv_len), (int)rd::attn_counter_ints(batch, n_q)); }
   return rd::check_launch("rd_attn_prepare(plan)");

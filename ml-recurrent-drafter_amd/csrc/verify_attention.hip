@@ -144,16 +144,17 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // item array has a slot for every blockIdx.y), and every kernel argument is fetched up front:
   // fetched where first used, they cost one more wait each on the way to the first tile load.
   const int item = blockIdx.y;
-  const int32_t* it = a.plan + RD_PLAN_HDR + 4 * a.B + 4 * item;
+  const int32_t* it = a.plan + RD_PLAN_HDR + 4 * a.B + RD_ITEM_INTS * item;
   const int n_items = a.plan[0];
-  int b = it[0], lo = it[1], hi = it[2], split = it[3];  // (split: with the row's cache shift above bit 12)
-  asm volatile("" : "+s"(b), "+s"(lo), "+s"(hi), "+s"(split));
+  int b = it[0], lo = it[1], hi = it[2], split = it[3];
+  int kv_shift = it[4];   // key column c of this row is cache row c - kv_shift
+  int key_min = it[5];    // the keys some query of the row attends to lie in [key_min, key_end):
+  int n_splits = it[6];
+  int key_end = it[7];    // nothing outside that span is read
+  asm volatile("" : "+s"(b), "+s"(lo), "+s"(hi), "+s"(split), "+s"(kv_shift), "+s"(key_min), "+s"(n_splits), "+s"(key_end));
   asm volatile("" ::"s"(a.q), "s"(a.q_sb), "s"(a.q_sh), "s"(a.q_ss), "s"(a.k), "s"(a.k_sb), "s"(a.k_sh), "s"(a.k_ss));
   asm volatile("" ::"s"(a.v), "s"(a.v_sb), "s"(a.v_sh), "s"(a.v_ss), "s"(a.bits), "s"(a.n_q), "s"(a.kv_len), "s"(a.words));
   if (item >= n_items) return;
-  const int kv_shift = split >> 12;  // key column c of this row is cache row c - kv_shift
-  split &= 0xfff;
-  const int n_splits = a.plan[RD_PLAN_HDR + 4 * b + 1];
   // query tiles of one (row, head, key range) are neighbours in dispatch order, so they run
   // together and the second read of the K/V tiles is served by the L2
   const int q_tiles = gridDim.x / a.H;
@@ -231,11 +232,15 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     const char* tile = base + (int64_t)key0 * row_bytes;
     const int64_t step_bytes = key_step * row_bytes;
     int64_t o0 = lane_off, o1 = step_bytes + lane_off, o2 = 2 * step_bytes + lane_off, o3 = 3 * step_bytes + lane_off;
-    if (key0 + kTile > a.kv_len) {
-      // the last tile of a row: keys past kv_len re-read the last key
+    if (key0 + kTile > key_end || key0 < key_min) {
+      // the first and the last tile of a row: keys in front of the row's first attended key (left
+      // padding) re-read that key, keys behind its last attended key (tree slots that do not exist,
+      // the end of the cache) re-read that one.  Nothing outside the row's live cache rows is ever
+      // touched: the probabilities of those keys are zero, but zero times whatever lay there
+      // could be NaN
       auto clamped = [&](int i) __attribute__((always_inline)) {
-        const int rel = first_key + i * key_step;
-        const int use = key0 + rel < a.kv_len ? rel : a.kv_len - 1 - key0;
+        const int key = key0 + first_key + i * key_step;
+        const int use = (key < key_end ? (key > key_min ? key : key_min) : key_end - 1) - key0;
         return (int64_t)use * row_bytes + 16 * chunk;
       };
       o0 = clamped(0); o1 = clamped(1); o2 = clamped(2); o3 = clamped(3);
@@ -505,15 +510,17 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // accumulator i of block db is d = 32*db + 8*(i/4) + 4*g + i%4
   if (n_splits == 1) {
     if (!writer) return;
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const bool live = l > 0.f;
+    const float inv = live ? 1.f / l : 0.f;
     __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh +
                  (int64_t)q_row * a.o_ss + 4 * g;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
-        bf16x4 w = {static_cast<__bf16>(o[db][4 * i4 + 0] * inv), static_cast<__bf16>(o[db][4 * i4 + 1] * inv),
-                    static_cast<__bf16>(o[db][4 * i4 + 2] * inv), static_cast<__bf16>(o[db][4 * i4 + 3] * inv)};
+        // (a row without any attended key gets zeros, whatever its accumulators picked up)
+        bf16x4 w = {static_cast<__bf16>(live ? o[db][4 * i4 + 0] * inv : 0.f), static_cast<__bf16>(live ? o[db][4 * i4 + 1] * inv : 0.f),
+                    static_cast<__bf16>(live ? o[db][4 * i4 + 2] * inv : 0.f), static_cast<__bf16>(live ? o[db][4 * i4 + 3] * inv : 0.f)};
         *reinterpret_cast<bf16x4*>(op + 32 * db + 8 * i4) = w;
       }
     return;
@@ -592,10 +599,11 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     for (int j = 0; j < kPass; ++j) {
       const int q = q0 + kGroups * j;
       if (q < q_end) {
-        const float inv = ls[j] > 0.f ? 1.f / ls[j] : 0.f;
+        const bool live = ls[j] > 0.f;
+        const float inv = live ? 1.f / ls[j] : 0.f;
         __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss + dq;
-        bf16x4 w = {static_cast<__bf16>(acc[j][0] * inv), static_cast<__bf16>(acc[j][1] * inv),
-                    static_cast<__bf16>(acc[j][2] * inv), static_cast<__bf16>(acc[j][3] * inv)};
+        bf16x4 w = {static_cast<__bf16>(live ? acc[j][0] * inv : 0.f), static_cast<__bf16>(live ? acc[j][1] * inv : 0.f),
+                    static_cast<__bf16>(live ? acc[j][2] * inv : 0.f), static_cast<__bf16>(live ? acc[j][3] * inv : 0.f)};
         *reinterpret_cast<bf16x4*>(op) = w;
       }
     }
@@ -709,7 +717,7 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
                                    const int64_t* v_strides, void* out, const int64_t* o_strides,
                                    int dtype, int batch, int n_heads, int n_kv_heads, int n_q,
                                    int kv_len, int head_dim, float scale, const uint64_t* bits,
-                                   const int32_t* plan, void* workspace, size_t workspace_bytes,
+                                   int32_t* plan, void* workspace, size_t workspace_bytes,
                                    int force_generic, const int32_t* row_start, void* stream) {
   RD_REQUIRE(batch > 0 && n_heads > 0 && n_kv_heads > 0 && n_q > 0 && kv_len > 0 && head_dim > 0,
              RD_EINVAL, "rd_verify_attention: bad sizes (batch %d heads %d kv_heads %d n_q %d kv %d D %d)",
@@ -733,7 +741,7 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
   a.scale = scale;
   a.part_o = nullptr; a.part_ml = nullptr;
   a.row_start = row_start;
-  a.counters = const_cast<int32_t*>(plan) + rd::attn_counter_offset(batch, n_q, kv_len);
+  a.counters = plan + rd::attn_counter_offset(batch, n_q, kv_len);
   hipStream_t s = rd::as_stream(stream);
 
   if (!force_generic && mfma_eligible(a, dtype)) {

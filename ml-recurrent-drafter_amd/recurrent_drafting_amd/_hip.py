@@ -12,7 +12,8 @@ import os
 
 import torch
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libredrafter_hip.so")
+# RD_HIP_LIBRARY names another build of the library (an A/B of two builds on one machine)
+_LIB_PATH = os.environ.get("RD_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "libredrafter_hip.so")
 _lib = None
 
 RD_BF16, RD_F16, RD_F32 = 0, 1, 2

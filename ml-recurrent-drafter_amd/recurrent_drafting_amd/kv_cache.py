@@ -127,15 +127,10 @@ class Cache:
         dtype: torch.dtype,
         device: torch.device,
     ) -> None:
-        # 64 rows of readable memory in front of the first slab: with rows in place the attention
-        # loads whole 64-key tiles and the first tile of a row may begin below the row's first key
-        shape = [n_layers, 2, batch_size, n_heads, max_length, head_dim]
-        numel = 1
-        for d in shape:
-            numel *= d
-        guard = 64 * head_dim
-        self._storage = torch.zeros(guard + numel, dtype=dtype, device=device)
-        self._cache = self._storage[guard:].view(shape)
+        # (the attention reads only the cache rows of keys that somebody attends to, so nothing is
+        # asked of the memory around a row's live rows; zeros as upstream, kv_cache.py:49-53)
+        self._storage = torch.zeros([n_layers, 2, batch_size, n_heads, max_length, head_dim], dtype=dtype, device=device)
+        self._cache = self._storage
         self.sliced = tuple(
             (View(self._cache, layer, 0, self), View(self._cache, layer, 1, self)) for layer in range(n_layers)
         )

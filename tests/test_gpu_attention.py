@@ -63,17 +63,59 @@ def test_mask_bits_and_plan():
     n_items, max_splits = plan[0], plan[4]
     assert plan[1] == nq and plan[2] == kv and plan[3] == (kv + 63) // 64
     per_row = plan[8 : 8 + 4 * B].reshape(B, 4)
-    firsts = [int(np.argmax(fixed[b].any(axis=0))) // 64 * 64 for b in range(B)]
+    attended = [np.flatnonzero(fixed[b].any(axis=0)) for b in range(B)]
+    key_min, key_end = [int(a[0]) for a in attended], [int(a[-1]) + 1 for a in attended]
+    firsts = [m // 64 * 64 for m in key_min]
     assert per_row[:, 0].tolist() == firsts
-    items = plan[8 + 4 * B : 8 + 4 * B + 4 * n_items].reshape(n_items, 4)
+    items = plan[8 + 4 * B : 8 + 4 * B + 8 * n_items].reshape(n_items, 8)
     assert n_items == per_row[:, 1].sum() and per_row[:, 1].max() <= max_splits
     lens = items[:, 2] - items[:, 1]
     assert (np.diff(lens) <= 0).all()  # longest first
-    for b in range(B):  # the items of a row tile [begin, kv) without gaps or overlap
-        mine = sorted((lo, hi) for bb, lo, hi, s in items.tolist() if bb == b)
-        assert mine[0][0] == firsts[b] and mine[-1][1] == kv
+    for b in range(B):  # the items of a row tile [begin, last attended key] without gaps or overlap
+        mine = sorted((lo, hi, s) for bb, lo, hi, s, *_ in items.tolist() if bb == b)
+        assert mine[0][0] == firsts[b] and mine[-1][1] == key_end[b]
         assert all(a[1] == c[0] for a, c in zip(mine, mine[1:]))
-        assert all(lo % 64 == 0 for lo, _ in mine)
+        assert all(lo % 64 == 0 for lo, _, _ in mine)
+        assert [s for _, _, s in mine] == list(range(len(mine)))
+        for bb, lo, hi, s, shift, kmin, n_splits, kend in items.tolist():
+            if bb == b:
+                assert (shift, kmin, n_splits, kend) == (0, key_min[b], per_row[b, 1], key_end[b])
+
+
+def test_mfma_kernel_reads_only_the_rows_of_attended_keys():
+    """Left padding in front of a row's first key, tree slots that do not exist behind its last one
+    and the tail of the cache hold NaN here (a cache made with torch.empty may hold anything): keys
+    that nobody attends to must not reach the arithmetic, not even with a zero weight."""
+    from recurrent_drafting_amd import attention
+
+    rng = np.random.default_rng(5)
+    prev_lens = [700, 333, 1, 640]
+    mask = _tree_case(4, 8, 5, prev_lens, seed=2).copy()
+    B, nq, kv = mask.shape
+    prev = kv - nq
+    counts = [nq - 5, nq, nq - 17, nq - 1]  # tree slots that exist per row; the rest attends to nothing
+    for b, c in enumerate(counts):
+        mask[b, c:, :] = False
+        mask[b, :, prev + c:] = False
+    H, D = 3, 128
+    q = torch.tensor(rng.standard_normal((B, H, nq, D)), dtype=torch.bfloat16, device="cuda")
+    k = torch.tensor(rng.standard_normal((B, H, kv + 90, D)), dtype=torch.bfloat16, device="cuda")
+    v = torch.tensor(rng.standard_normal((B, H, kv + 90, D)), dtype=torch.bfloat16, device="cuda")
+    clean_k, clean_v = k.clone(), v.clone()
+    for b in range(B):
+        for t in (k, v):
+            t[b, :, : prev - prev_lens[b]] = float("nan")
+            t[b, :, prev + counts[b]:] = float("nan")
+    tq = q.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    for heads_for_plan in (H, 1):  # whole rows, and rows split over several work items
+        prep = attention.prepare(_dev(mask, torch.bool), fix_empty_rows=False, n_heads=heads_for_plan)
+        got = attention.masked_attention(tq, k[:, :, :kv], v[:, :, :kv], prep)
+        prep2 = attention.prepare(_dev(mask, torch.bool), fix_empty_rows=False, n_heads=heads_for_plan)
+        want = attention.masked_attention(tq, clean_k[:, :, :kv], clean_v[:, :, :kv], prep2)
+        assert torch.isfinite(got).all()
+        assert torch.equal(got, want)
+        for b, c in enumerate(counts):  # queries that attend to nothing give zeros
+            assert not got[b, c:].any()
 
 
 def _run(q, k, v, mask, dtype, force_generic, cache_like=False, n_heads_for_plan=None):

@@ -185,7 +185,6 @@ def test_rope_append_drops_rows_that_a_shift_would_put_outside_the_cache():
     assert torch.equal(raw[0, 0, :, 11], kk[0, :, 0]) and (raw[0, 0, :, :11] == 7).all()
     # row 1: tokens 0..2 would be rows -3..-1: dropped; token 3 lands in row 0
     assert torch.equal(raw[0, 1, :, 0], kk[1, :, 3]) and (raw[0, 1, :, 1:] == 7).all()
-    assert (cache._storage[: 64 * D] == 0).all()  # the slack in front of the first slab is untouched
 
 
 def test_timing_sample_times_every_nth_launch():
