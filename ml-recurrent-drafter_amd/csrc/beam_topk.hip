@@ -92,16 +92,11 @@ __device__ void beam_row_fallback(const T* __restrict__ x_row, int V, float row_
     const float lp = c < n_gt + take_eq ? Num<T>::round(key_value(e) - logsum) : masked_lp;
     sh.ckey[c] = key64(lp + lpb, (uint32_t)key_index(e));
   }
-  if (tid == 0) sh.ckey[n_list] = 0ull;
+  if (tid < kKeyPad) sh.ckey[n_list + tid] = 0ull;
   __syncthreads();
   for (int c = tid; c < n_list; c += THREADS) {
     const unsigned long long mine = sh.ckey[c];
-    const ulonglong2* k2 = reinterpret_cast<const ulonglong2*>(sh.ckey);
-    int rank = 0;
-    for (int o = 0; 2 * o < n_list; ++o) {
-      const ulonglong2 kk = k2[o];
-      rank += (kk.x > mine) + (kk.y > mine);
-    }
+    const int rank = count_greater(sh.ckey, pad_keys(n_list), mine);
     if (rank < W) { c_score[rank] = key_value(mine); c_tok[rank] = key_index(mine); }
   }
   for (int w = n_list + tid; w < W; w += THREADS) { c_score[w] = -INFINITY; c_tok[w] = -1; }  // V < W
@@ -140,7 +135,7 @@ __global__ __launch_bounds__(THREADS) void beam_row_kernel(
   int32_t* c_tok = cand_tok + (int64_t)row * W;
   // (a few more maxima than k_eff: the k-th largest key then sits well above the pivot's key, and
   // a tie between the two, which costs the slow path, takes that many equal values in a row)
-  const float pivot = row_pivot<THREADS>(tmax, k_eff + kPivotMargin < THREADS ? k_eff + kPivotMargin : THREADS, sh);
+  const float pivot = row_pivot<THREADS, 8 * (sizeof(T) < 4 ? sizeof(T) : 4)>(tmax, k_eff + kPivotMargin < THREADS ? k_eff + kPivotMargin : THREADS, sh);
 
   // ---- candidates: entries >= pivot, keyed by their value after the max subtraction ------------
   // t(x) = round_T(x - max) is monotone, so the k-th largest t comes from the list; an entry

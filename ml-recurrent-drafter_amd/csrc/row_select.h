@@ -72,11 +72,33 @@ __device__ inline float wave_sum(float v) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
-// Candidate list: WAVES segments of kCap / WAVES keys (+2 so that a segment can be padded to an
-// even count for 16-byte reads); skey receives the same keys sorted descending.
-struct RowShared {
-  unsigned long long ckey[kCap + 2 * kMaxRowWaves];
-  unsigned long long skey[kCap];
+constexpr int kKeyPad = 16;  // key lists are padded with zero keys to a multiple of this many
+
+// Number of keys in list[0 .. n_pad) that are greater than `mine`.  n_pad is a multiple of kKeyPad
+// (the list is padded with zero keys, which are below every real key).  Eight 16-byte LDS reads are
+// issued before their results are used: one read per iteration would leave the loop waiting for
+// the LDS latency every time (4 us for 256 keys; 0.5 us this way).
+__device__ inline int count_greater(const unsigned long long* list, int n_pad, unsigned long long mine) {
+  const ulonglong2* k2 = reinterpret_cast<const ulonglong2*>(list);
+  int before = 0;
+  for (int o = 0; 2 * o < n_pad; o += kKeyPad / 2) {
+    ulonglong2 kk[kKeyPad / 2];
+#pragma unroll
+    for (int u = 0; u < kKeyPad / 2; ++u) kk[u] = k2[o + u];
+#pragma unroll
+    for (int u = 0; u < kKeyPad / 2; ++u) before += (kk[u].x > mine) + (kk[u].y > mine);
+  }
+  return before;
+}
+__device__ inline int pad_keys(int n) { return (n + kKeyPad - 1) / kKeyPad * kKeyPad; }
+
+// Candidate list: WAVES segments of kCap / WAVES keys (+kKeyPad so that a segment can be padded
+// with zero keys for count_greater); skey receives the same keys sorted descending.
+template <int CAP>
+struct RowSharedT {
+  static constexpr int kCapacity = CAP;
+  unsigned long long ckey[CAP + kKeyPad * kMaxRowWaves];
+  unsigned long long skey[CAP];
   float red[kMaxRowWaves];
   unsigned long long red64[kMaxRowWaves];
   int ired[kMaxRowWaves];
@@ -84,12 +106,13 @@ struct RowShared {
   int n_surv;
   float logsum;
 };
+using RowShared = RowSharedT<kCap>;
 
 __device__ inline float key_value(unsigned long long k) { return unord((uint32_t)(k >> 32)); }
 __device__ inline int key_index(unsigned long long k) { return (int)(0xffffffffu - (uint32_t)k); }
 
-template <int THREADS>
-__device__ inline float block_max(float v, RowShared& sh) {
+template <int THREADS, typename SH>
+__device__ inline float block_max(float v, SH& sh) {
   v = wave_max(v);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = v;
@@ -98,10 +121,10 @@ __device__ inline float block_max(float v, RowShared& sh) {
   for (int w = 1; w < THREADS / 64; ++w) r = fmaxf(r, sh.red[w]);
   return r;
 }
-template <int THREADS>
-__device__ inline float block_min(float v, RowShared& sh) { return -block_max<THREADS>(-v, sh); }
-template <int THREADS>
-__device__ inline float block_sum(float v, RowShared& sh) {
+template <int THREADS, typename SH>
+__device__ inline float block_min(float v, SH& sh) { return -block_max<THREADS>(-v, sh); }
+template <int THREADS, typename SH>
+__device__ inline float block_sum(float v, SH& sh) {
   v = wave_sum(v);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) sh.red[threadIdx.x >> 6] = v;
@@ -110,8 +133,8 @@ __device__ inline float block_sum(float v, RowShared& sh) {
   for (int w = 0; w < THREADS / 64; ++w) r += sh.red[w];  // fixed order
   return r;
 }
-template <int THREADS>
-__device__ inline int block_isum(int v, RowShared& sh) {
+template <int THREADS, typename SH>
+__device__ inline int block_isum(int v, SH& sh) {
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) sh.ired[threadIdx.x >> 6] = v;
@@ -120,8 +143,8 @@ __device__ inline int block_isum(int v, RowShared& sh) {
   for (int w = 0; w < THREADS / 64; ++w) r += sh.ired[w];
   return r;
 }
-template <int THREADS>
-__device__ inline uint64_t block_max64(uint64_t v, RowShared& sh) {
+template <int THREADS, typename SH>
+__device__ inline uint64_t block_max64(uint64_t v, SH& sh) {
   for (int off = 32; off > 0; off >>= 1) {
     const uint64_t o = __shfl_xor(v, off);
     v = o > v ? o : v;
@@ -172,52 +195,56 @@ __device__ inline void load_row(const T* __restrict__ x_row, int V, float (&x)[I
 }
 
 // Pivot with at least k_eff row entries >= it, from the per-thread maxima: the minimum over waves
-// of each wave's r-th largest maximum, r = ceil(k_eff / waves).
-template <int THREADS>
-__device__ inline float row_pivot(float tmax, int k_eff, RowShared& sh) {
+// of each wave's r-th largest maximum, r = ceil(k_eff / waves) (-inf when a wave holds fewer).
+// A wave finds its r-th largest by bisection on the bits of the ordered value: per bit one
+// compare, one ballot and one scalar population count -- no LDS traffic, no cross-lane reductions
+// (taking the maxima out one by one, r rounds of wave reductions, cost 2.4 us of the 9 us a quarter
+// row took; ranking all maxima against each other through LDS was bound by the LDS bandwidth once
+// eight workgroups shared a compute unit).  VALUE_BITS: 16 for bf16/fp16 data (the low half of the
+// float is zero), 32 otherwise.
+template <int THREADS, int VALUE_BITS, typename SH>
+__device__ inline float row_pivot(float tmax, int k_eff, SH& sh) {
   constexpr int WAVES = THREADS / 64;
-  const int lane = threadIdx.x & 63;
-  const int rounds = (k_eff + WAVES - 1) / WAVES;
-  float cur = tmax, wave_pivot = -INFINITY;
-  for (int it = 0; it < rounds; ++it) {
-    const float wm = wave_max(cur);
-    wave_pivot = wm;
-    const uint64_t holders = __ballot(cur == wm);
-    if (holders != 0 && lane == __builtin_ctzll(holders)) cur = -INFINITY;
+  const int r = (k_eff + WAVES - 1) / WAVES;
+  const uint32_t key = ord(tmax);
+  uint32_t found = 0u;  // wave-uniform: the largest value v with at least r lanes >= v
+#pragma unroll
+  for (int bit = 31; bit >= 32 - VALUE_BITS; --bit) {
+    const uint32_t cand = found | (1u << bit);
+    const int n = __builtin_popcountll(__ballot(key >= cand));
+    found = n >= r ? cand : found;
   }
+  // at or below the key of -inf: fewer than r lanes hold data
+  const float wave_pivot = found <= 0x007fffffu ? -INFINITY : unord(found);
   return block_min<THREADS>(wave_pivot, sh);
 }
 
-// Lists key_of(x[j], row index) for every register entry >= pivot and sorts the list descending
-// into sh.skey.  Returns the number of keys, or -1 when a wave's segment overflowed.  Keys must be
-// distinct and nonzero (key64 of distinct indices is).  Ends with a barrier.
-template <int ITEMS, int VEC, int THREADS, typename KeyFn>
-__device__ inline int row_sorted_candidates(const float (&x)[ITEMS], float pivot, RowShared& sh,
-                                            KeyFn key_of) {
-  constexpr int WAVES = THREADS / 64, SEG = kCap / WAVES, STRIDE = SEG + 2;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  {
-    unsigned long long* seg = sh.ckey + wave * STRIDE;
-    const int base = row_base<VEC>();
-    int count = 0;  // wave-uniform
+// Lists key_of(x[j], row index) for every register entry >= pivot in per-wave segments of sh.ckey
+// (sh.seg_count holds the segment lengths; a count above the segment size means overflow).  Ends
+// with a barrier.  Returns the total, or -1 on overflow.
+template <int ITEMS, int VEC, int THREADS, typename SH, typename KeyFn>
+__device__ inline int row_list_candidates(const float (&x)[ITEMS], float pivot, SH& sh, KeyFn key_of) {
+  constexpr int WAVES = THREADS / 64, SEG = SH::kCapacity / WAVES, STRIDE = SEG + kKeyPad;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned long long* seg = sh.ckey + wave * STRIDE;
+  const int base = row_base<VEC>();
+  int count = 0;  // wave-uniform
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      const bool take = x[j] >= pivot;
-      const uint64_t votes = __ballot(take);
-      if (votes != 0) {
-        if (take) {
-          const int pos = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(votes >> 32),
-                                       __builtin_amdgcn_mbcnt_lo((uint32_t)votes, 0u));
-          if (pos < SEG) seg[pos] = key_of(x[j], row_index_at<VEC, THREADS>(base, j));
-        }
-        count += __builtin_popcountll(votes);
+  for (int j = 0; j < ITEMS; ++j) {
+    const bool take = x[j] >= pivot;
+    const uint64_t votes = __ballot(take);
+    if (votes != 0) {
+      if (take) {
+        const int pos = count + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(votes >> 32),
+                                     __builtin_amdgcn_mbcnt_lo((uint32_t)votes, 0u));
+        if (pos < SEG) seg[pos] = key_of(x[j], row_index_at<VEC, THREADS>(base, j));
       }
-    }
-    if (lane == 0) {
-      sh.seg_count[wave] = count;
-      if (count < SEG) seg[count] = 0ull;  // pad to an even count with a key below every real key
+      count += __builtin_popcountll(votes);
     }
   }
+  if (lane == 0) sh.seg_count[wave] = count;
+  // pad to a multiple of kKeyPad with keys below every real key
+  if (lane < kKeyPad && count <= SEG) seg[count + lane] = 0ull;
   __syncthreads();
   int n = 0;
   bool overflow = false;
@@ -227,20 +254,30 @@ __device__ inline int row_sorted_candidates(const float (&x)[ITEMS], float pivot
     overflow |= c > SEG;
     n += c;
   }
-  if (overflow) return -1;
-  for (int c = tid; c < n; c += THREADS) {
-    int w = 0, off = c;
-    while (off >= sh.seg_count[w]) off -= sh.seg_count[w++];
-    const unsigned long long mine = sh.ckey[w * STRIDE + off];
+  return overflow ? -1 : n;
+}
+// The c-th listed key, c < total, in segment order.
+template <int THREADS, typename SH>
+__device__ inline unsigned long long row_listed_key(int c, const SH& sh) {
+  constexpr int WAVES = THREADS / 64, SEG = SH::kCapacity / WAVES, STRIDE = SEG + kKeyPad;
+  int w = 0, off = c;
+  while (off >= sh.seg_count[w]) off -= sh.seg_count[w++];
+  return sh.ckey[w * STRIDE + off];
+}
+
+// Lists key_of(x[j], row index) for every register entry >= pivot and sorts the list descending
+// into sh.skey.  Returns the number of keys, or -1 when a wave's segment overflowed.  Keys must be
+// distinct and nonzero (key64 of distinct indices is).  Ends with a barrier.
+template <int ITEMS, int VEC, int THREADS, typename SH, typename KeyFn>
+__device__ inline int row_sorted_candidates(const float (&x)[ITEMS], float pivot, SH& sh,
+                                            KeyFn key_of) {
+  constexpr int WAVES = THREADS / 64, SEG = SH::kCapacity / WAVES, STRIDE = SEG + kKeyPad;
+  const int n = row_list_candidates<ITEMS, VEC, THREADS>(x, pivot, sh, key_of);
+  if (n < 0) return -1;
+  for (int c = threadIdx.x; c < n; c += THREADS) {
+    const unsigned long long mine = row_listed_key<THREADS>(c, sh);
     int before = 0;
-    for (int w2 = 0; w2 < WAVES; ++w2) {
-      const int n2 = sh.seg_count[w2];
-      const ulonglong2* seg2 = reinterpret_cast<const ulonglong2*>(sh.ckey + w2 * STRIDE);
-      for (int o = 0; 2 * o < n2; ++o) {
-        const ulonglong2 kk = seg2[o];
-        before += (kk.x > mine) + (kk.y > mine);
-      }
-    }
+    for (int w2 = 0; w2 < WAVES; ++w2) before += count_greater(sh.ckey + w2 * STRIDE, pad_keys(sh.seg_count[w2]), mine);
     sh.skey[before] = mine;
   }
   __syncthreads();
@@ -249,8 +286,8 @@ __device__ inline int row_sorted_candidates(const float (&x)[ITEMS], float pivot
 
 // Number of sorted keys whose value part is >= the value part of sh.skey[k - 1] (k <= n): the
 // entries that are >= the k-th largest value, ties included.  Ends with a barrier.
-template <int THREADS>
-__device__ inline int row_survivors(int n, int k, RowShared& sh) {
+template <int THREADS, typename SH>
+__device__ inline int row_survivors(int n, int k, SH& sh) {
   const uint32_t thr_hi = (uint32_t)(sh.skey[k - 1] >> 32);
   for (int r = threadIdx.x; r < n; r += THREADS) {
     const bool in = (uint32_t)(sh.skey[r] >> 32) >= thr_hi;
@@ -265,9 +302,9 @@ __device__ inline int row_survivors(int n, int k, RowShared& sh) {
 // ordered bit pattern, four passes over the row in memory (it sits in L2) with a 256-bin LDS
 // histogram each.  This is the rare path; it reads memory rather than the caller's register copy so
 // that it adds nothing to the caller's register budget.  Uses sh.ckey as the histogram.
-template <typename T, int THREADS>
+template <typename T, int THREADS, typename SH>
 __device__ inline float row_kth_radix(const T* __restrict__ x_row, int V, float shift, int k_eff,
-                                      RowShared& sh) {
+                                      SH& sh) {
   int* hist = reinterpret_cast<int*>(sh.ckey);
   const int tid = threadIdx.x, lane = tid & 63;
   uint32_t prefix = 0u, known = 0u;  // bits of the answer found so far, and their mask
