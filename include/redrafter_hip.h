@@ -363,6 +363,22 @@ RD_API int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, int64
                         int64_t logp_row_stride, void* workspace, size_t workspace_bytes,
                         int force_fallback, void* stream);
 
+/* rd_beam_topk_static: rd_beam_topk without the workspace argument, for callers that cannot
+ * allocate device memory -- code under HIP graph capture, serving loops and harnesses that forbid
+ * hipMalloc.  (No counterpart in the reference.)  The candidate lists that rd_beam_topk keeps in the
+ * caller's workspace live in a 2 MiB device array that is part of the library, one copy per GPU; the
+ * call allocates and frees nothing.  Limits: batch * width <= 4096 and width <= 64, beyond which the
+ * call fails with RD_ELIMIT and enqueues nothing.  Every call on a GPU uses that GPU's one array:
+ * calls that overlap in time on one GPU (two streams, two threads) race; calls on one stream do
+ * not.  The first call on a device looks the array's address up (hipGetSymbolAddress); make it
+ * before a graph capture begins. */
+RD_API int rd_beam_topk_static(const void* logits, int dtype, int64_t row_stride, int64_t batch_stride,
+                               int batch, int width, int vocab, const float* log_p_beam, int top_k,
+                               float mask_value, const int64_t* beams_in, int t_len,
+                               float* new_log_p_beam, int64_t* tokens, int64_t* parents,
+                               int64_t* beams_out, float* logp_out, int64_t logp_row_stride,
+                               int force_fallback, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Speculative-sampling acceptance.
  *

@@ -25,6 +25,8 @@
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 #include "row_select.h"
 
 namespace {
@@ -321,6 +323,38 @@ int launch_rows(const void* logits, int64_t row_stride, int64_t batch_stride, in
   return rd::check_launch("rd_beam_topk(rows)");
 }
 
+// Scratch of rd_beam_topk_static: the candidate lists (scores, tokens) of every beam row, in device
+// memory that belongs to the library and exists from the moment it is loaded, one copy per GPU.
+constexpr int kStaticMaxRows = 4096;  // batch * width
+constexpr size_t kStaticScratchBytes = 2 * (size_t)kStaticMaxRows * kMaxWidth * 4;  // 2 MiB
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+// The array's name is only a host-side stand-in: its address on a GPU is asked for once per device
+// (with that device current) and kept; every GPU holds its own copy at its own address.
+void* static_scratch(int* error) {
+  static std::mutex mu;
+  static void* ptr[kMaxDevices] = {nullptr};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    *error = rd::fail(RD_ELAUNCH, "rd_beam_topk_static: no current device (or an ordinal above %d)", kMaxDevices - 1);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptr[dev] == nullptr) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      *error = rd::fail(RD_ELAUNCH, "rd_beam_topk_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    ptr[dev] = p;
+  }
+  return ptr[dev];
+}
 }  // namespace
 
 extern "C" size_t rd_beam_topk_workspace_bytes(int batch, int width) {
@@ -373,4 +407,24 @@ extern "C" int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, i
   { rd::ScopedTiming rd_t("beam_merge_kernel", s); hipLaunchKernelGGL(beam_merge_kernel, dim3(batch), dim3(kMergeThreads), 0, s, cs, ct, width, vocab,
                      beams_in, t_len, new_log_p_beam, tokens, parents, beams_out); }
   return rd::check_launch("rd_beam_topk(merge)");
+}
+
+extern "C" int rd_beam_topk_static(const void* logits, int dtype, int64_t row_stride, int64_t batch_stride,
+                                   int batch, int width, int vocab, const float* log_p_beam, int top_k,
+                                   float mask_value, const int64_t* beams_in, int t_len,
+                                   float* new_log_p_beam, int64_t* tokens, int64_t* parents,
+                                   int64_t* beams_out, float* logp_out, int64_t logp_row_stride,
+                                   int force_fallback, void* stream) {
+  RD_REQUIRE(batch > 0 && width > 0, RD_EINVAL, "rd_beam_topk_static: bad sizes (batch %d width %d)", batch, width);
+  const size_t need = rd_beam_topk_workspace_bytes(batch, width);
+  RD_REQUIRE((int64_t)batch * width <= kStaticMaxRows && width <= kMaxWidth && need <= kStaticScratchBytes, RD_ELIMIT,
+             "rd_beam_topk_static: batch %d x width %d is beyond the built-in scratch (batch*width <= %d, width <= %d); "
+             "use rd_beam_topk with a workspace", batch, width, kStaticMaxRows, kMaxWidth);
+  int error = RD_OK;
+  void* ws = static_scratch(&error);
+  if (ws == nullptr) return error;
+  // every beam row writes all `width` entries of its two lists, so nothing of an earlier call is read
+  return rd_beam_topk(logits, dtype, row_stride, batch_stride, batch, width, vocab, log_p_beam, top_k, mask_value,
+                      beams_in, t_len, new_log_p_beam, tokens, parents, beams_out, logp_out, logp_row_stride, ws,
+                      kStaticScratchBytes, force_fallback, stream);
 }

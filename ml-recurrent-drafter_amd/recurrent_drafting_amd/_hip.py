@@ -74,6 +74,10 @@ _PROTOTYPES = {
         _I,
         [_P, _I, _L, _L, _I, _I, _I, _P, _I, _F, _P, _I, _P, _P, _P, _P, _P, _L, _P, _Z, _I, _P],
     ),
+    "rd_beam_topk_static": (
+        _I,
+        [_P, _I, _L, _L, _I, _I, _I, _P, _I, _F, _P, _I, _P, _P, _P, _P, _P, _L, _I, _P],
+    ),
 }
 
 
