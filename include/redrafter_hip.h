@@ -177,13 +177,16 @@ RD_API int rd_position_ids(const int64_t* input_ids, int64_t ids_row_stride, int
  * the whole live cache on every step (recurrent_drafting.py:200-209); the same array is handed to
  * rd_rope_append and rd_attn_prepare, and rd_kv_materialize moves the rows once when the
  * reference's layout is wanted.
+ * left_pads (batch int32 on the device, or NULL): the leading pad run of every row of input_ids when
+ * the caller has it already (rd_tree_attn_prepare and rd_count_left_paddings write it); saves the
+ * launch that counts them.
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_realign_plan_ints(int batch, int length);
 RD_API int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride, int64_t prev,
                            const int64_t* n_tokens_in_seq, const int64_t* seq_in_beam,
                            const int64_t* beams, const int64_t* unpacker, int batch, int width,
                            int length, int64_t pad_token_id, int32_t* plan, int64_t* new_ids,
-                           int32_t* kv_row_shift, void* stream);
+                           int32_t* kv_row_shift, const int32_t* left_pads, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * KV cache, shape (n_layers, 2, batch, n_heads, max_len, head_dim), rows of row_bytes bytes.
@@ -317,6 +320,23 @@ RD_API int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64_t m
                            int batch, int n_q, int kv_len, int n_heads, int fix_empty_rows,
                            uint64_t* bits, int32_t* plan, const int32_t* kv_row_shift,
                            void* stream);
+/* rd_tree_attn_prepare: for the packed tree of a verification step, what rd_tree_mask, rd_attn_prepare
+ * and rd_position_ids produce one after the other -- the mask as bits, the plan, the position ids --
+ * in one launch and without the (batch, n, prev + n) byte mask in between.  Replaces, for a caller
+ * that goes straight to rd_verify_attention, tree_attention._get_causal_mask (tree_attention.py:191-298),
+ * the row slice (:337), attention.bias (attention.py:75-88, called at modeling_llama.py:228) and the
+ * position rule (recurrent_drafting.py:449-458).  unpacker, packed_token_indices, counts: as written
+ * by rd_tree_build; n = counts[batch], the packed length (the caller has read it); padding_mask,
+ * pm_elem_bytes, pm_row_stride, pm_pad_value, prev: as for rd_tree_mask.  bits: rd_attn_bits_words(
+ * batch, n, prev + n) words, bit-identical to rd_attn_prepare on rd_tree_mask's output; plan:
+ * rd_attn_plan_ints(batch, n, prev + n) ints.  position_ids (batch, n) int64 and left_pads (batch
+ * int32: leading padding keys of every row; rd_realign_plan takes it) are optional.  prev <= 131072. */
+RD_API int rd_tree_attn_prepare(const int64_t* unpacker, const int64_t* packed_token_indices,
+                                const int32_t* counts, const void* padding_mask, int pm_elem_bytes,
+                                int64_t pm_row_stride, int64_t pm_pad_value, int64_t prev, int batch,
+                                int width, int length, int n, int n_heads, uint64_t* bits,
+                                int32_t* plan, int64_t* position_ids, int32_t* left_pads,
+                                const int32_t* kv_row_shift, void* stream);
 RD_API size_t rd_attention_workspace_bytes(int batch, int n_heads, int n_q, int kv_len,
                                            int head_dim);
 RD_API int rd_verify_attention(const void* q, const int64_t* q_strides, const void* k,

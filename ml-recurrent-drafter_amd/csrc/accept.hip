@@ -287,7 +287,7 @@ extern "C" int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride,
                                const int64_t* n_tokens_in_seq, const int64_t* seq_in_beam,
                                const int64_t* beams, const int64_t* unpacker, int batch, int width,
                                int length, int64_t pad_token_id, int32_t* plan, int64_t* new_ids,
-                               int32_t* kv_row_shift, void* stream) {
+                               int32_t* kv_row_shift, const int32_t* left_pads, void* stream) {
   RD_REQUIRE(batch > 0 && width > 0 && length > 0 && prev >= 0, RD_EINVAL,
              "rd_realign_plan: bad sizes (batch %d width %d length %d prev %lld)", batch, width,
              length, (long long)prev);
@@ -296,10 +296,14 @@ extern "C" int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride,
   RD_REQUIRE((prev == 0 || input_ids) && n_tokens_in_seq && seq_in_beam && beams && plan && new_ids,
              RD_EINVAL, "rd_realign_plan: null pointer");
   hipStream_t s = rd::as_stream(stream);
-  int32_t* pads = plan + 4 + (size_t)batch * (4 + length);
-  { rd::ScopedTiming rd_t("count_pads_kernel", s); hipLaunchKernelGGL(count_pads_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
-                     ids_row_stride, prev, pad_token_id, pads); }
-  if (int e = rd::check_launch("rd_realign_plan(pads)")) return e;
+  const int32_t* pads = left_pads;
+  if (pads == nullptr) {
+    int32_t* own = plan + 4 + (size_t)batch * (4 + length);
+    { rd::ScopedTiming rd_t("count_pads_kernel", s); hipLaunchKernelGGL(count_pads_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
+                       ids_row_stride, prev, pad_token_id, own); }
+    if (int e = rd::check_launch("rd_realign_plan(pads)")) return e;
+    pads = own;
+  }
   { rd::ScopedTiming rd_t("realign_plan_kernel", s); hipLaunchKernelGGL(realign_plan_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
                      ids_row_stride, prev, n_tokens_in_seq, seq_in_beam, beams, unpacker, batch,
                      width, length, pad_token_id, pads, plan, new_ids, kv_row_shift); }

@@ -54,44 +54,22 @@ __global__ __launch_bounds__(kThreads) void mask_bits_kernel(
   }
 }
 
-__global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __restrict__ row_first,
-                                                             const int32_t* __restrict__ row_last,
-                                                             int B, int n_q, int kv_len, int words,
-                                                             int min_chunk, int max_splits,
-                                                             int n_heads, int n_cu,
-                                                             const int32_t* __restrict__ kv_shift,
-                                                             int32_t* __restrict__ plan,
-                                                             int32_t* __restrict__ counters,
-                                                             int n_counters) {
+// The plan from the span of attended keys of every batch row (s_key_min[b], s_key_end[b], in LDS,
+// written before the call; the call begins with a barrier).  Whole workgroup of kThreads.
+__device__ void build_plan(const int* s_key_min, const int* s_key_end, int B, int n_q, int kv_len,
+                           int words, int min_chunk, int max_splits, int n_heads, int n_cu,
+                           const int32_t* __restrict__ kv_shift, int32_t* __restrict__ plan,
+                           int32_t* __restrict__ counters, int n_counters) {
   __shared__ int s_n_items;
   __shared__ int s_chunk;
-  extern __shared__ int s_span[];  // [2][B]: first key any query of the row attends to, last such key + 1
-  int* s_key_min = s_span;
-  int* s_key_end = s_span + B;
+  __shared__ int s_len[rd::kAttnSortLimit];
   for (int i = threadIdx.x; i < n_counters; i += kThreads) counters[i] = 0;
   int32_t* per_row = plan + RD_PLAN_HDR;
   int32_t* items = plan + RD_PLAN_HDR + 4 * B;
-  // pass 1: per batch row, first attended key and number of splits
-  // (one wave per batch row at a time: the minimum over its query rows)
-  for (int b = threadIdx.x >> 6; b < B; b += kThreads / 64) {
-    int first = kv_len, last = -1;
-    for (int q = threadIdx.x & 63; q < n_q; q += 64) {
-      const int f = row_first[(int64_t)b * n_q + q], l = row_last[(int64_t)b * n_q + q];
-      first = f < first ? f : first;
-      last = l > last ? l : last;
-    }
-    for (int off = 32; off > 0; off >>= 1) {
-      const int o = __shfl_xor(first, off), p = __shfl_xor(last, off);
-      first = o < first ? o : first;
-      last = p > last ? p : last;
-    }
-    if ((threadIdx.x & 63) == 0) {
-      if (last < first) { first = kv_len - 1; last = kv_len - 1; }  // a row in which nobody attends to anything
-      per_row[4 * b + 0] = (first / 64) * 64;
-      per_row[4 * b + 3] = kv_shift ? kv_shift[b] : 0;  // cache row of key c is c - shift
-      s_key_min[b] = first;
-      s_key_end[b] = last + 1;
-    }
+  __syncthreads();
+  for (int b = threadIdx.x; b < B; b += kThreads) {
+    per_row[4 * b + 0] = (s_key_min[b] / 64) * 64;
+    per_row[4 * b + 3] = kv_shift ? kv_shift[b] : 0;  // cache row of key c is c - shift
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -127,7 +105,7 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
   }
   __syncthreads();
   const int n_items = s_n_items;
-  // pass 2: every item computes its own extent and its rank (longest first, ties by index)
+  // every item computes its own extent and its rank (longest first, ties by index)
   auto extent = [&](int it, int& b, int& s, int& lo, int& hi) {
     b = 0;
     while (b + 1 < B && per_row[4 * (b + 1) + 2] <= it) ++b;
@@ -141,7 +119,6 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
     lo = lo < end ? lo : end;
     hi = hi < end ? hi : end;
   };
-  __shared__ int s_len[rd::kAttnSortLimit];
   const bool sorted = n_items <= rd::kAttnSortLimit;
   if (sorted) {
     for (int it = threadIdx.x; it < n_items; it += kThreads) {
@@ -169,6 +146,145 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
     rec[5] = s_key_min[b];
     rec[6] = per_row[4 * b + 1];
     rec[7] = s_key_end[b];
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __restrict__ row_first,
+                                                             const int32_t* __restrict__ row_last,
+                                                             int B, int n_q, int kv_len, int words,
+                                                             int min_chunk, int max_splits,
+                                                             int n_heads, int n_cu,
+                                                             const int32_t* __restrict__ kv_shift,
+                                                             int32_t* __restrict__ plan,
+                                                             int32_t* __restrict__ counters,
+                                                             int n_counters) {
+  extern __shared__ int s_span[];  // [2][B]: first key any query of the row attends to, last such key + 1
+  int* s_key_min = s_span;
+  int* s_key_end = s_span + B;
+  // per batch row, the span of attended keys: the minimum / maximum over its query rows
+  // (one wave per batch row at a time)
+  for (int b = threadIdx.x >> 6; b < B; b += kThreads / 64) {
+    int first = kv_len, last = -1;
+    for (int q = threadIdx.x & 63; q < n_q; q += 64) {
+      const int f = row_first[(int64_t)b * n_q + q], l = row_last[(int64_t)b * n_q + q];
+      first = f < first ? f : first;
+      last = l > last ? l : last;
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+      const int o = __shfl_xor(first, off), p = __shfl_xor(last, off);
+      first = o < first ? o : first;
+      last = p > last ? p : last;
+    }
+    if ((threadIdx.x & 63) == 0) {
+      if (last < first) { first = kv_len - 1; last = kv_len - 1; }  // a row in which nobody attends to anything
+      s_key_min[b] = first;
+      s_key_end[b] = last + 1;
+    }
+  }
+  build_plan(s_key_min, s_key_end, B, n_q, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan,
+             counters, n_counters);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The packed tree straight to mask bits, position ids and plan: what tree_mask_kernel (bytes),
+// mask_bits_kernel, position_ids_kernel and attn_plan_kernel produce one after the other, in one
+// launch and without the (batch, n, prev + n) byte mask.
+//   workgroups (x, b < B): kTreeSlots packed slots of batch row b, a wave per slot at a time: the
+//     words of the left part are the same for every slot of a row (ballots of "is not padding",
+//     computed once per workgroup into LDS); the tree part of slot q sets the bits of the packed
+//     slots of its source beam's positions 0..k.  position_ids[b, q] = prev - leading pads + k.
+//   workgroup (0, B): the plan.  The span of attended keys of a row follows from its left padding
+//     and its tree size: first attended key = first key that is not padding (prev when there is
+//     none: slot 0 attends to itself), last = its last tree slot (which attends to itself).
+// ---------------------------------------------------------------------------------------------
+constexpr int kTreeSlots = 16;
+constexpr int kMaxLeftWords = 2048;  // left part of at most 131072 keys
+
+template <typename PM>
+__device__ inline int left_words(const PM* __restrict__ pm, int64_t prev, PM pad, uint64_t* s_left, int* s_first) {
+  // words of "key j < prev is not padding" into s_left; returns nothing, *s_first = first such key (prev if none)
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = (int)((prev + 63) >> 6);
+  int first = (int)prev;
+  for (int w = wave; w < nw; w += kWaves) {
+    const int64_t j = (int64_t)w * 64 + lane;
+    const bool on = j < prev && pm[j] != pad;
+    const uint64_t word = __ballot(on);
+    if (lane == 0) s_left[w] = word;
+    if (word != 0) {
+      const int f = w * 64 + __builtin_ctzll(word);
+      first = f < first ? f : first;
+    }
+  }
+  if (lane == 0) atomicMin(s_first, first);
+  return nw;
+}
+
+template <typename PM>
+__global__ __launch_bounds__(kThreads) void tree_prepare_kernel(
+    const int64_t* __restrict__ unpacker, const int64_t* __restrict__ packed_token_indices,
+    const int32_t* __restrict__ counts, const PM* __restrict__ padding_mask, int64_t pm_row_stride,
+    int64_t pm_pad_value, int64_t prev, int B, int WL, int L, int n, int words, int n_heads, int n_cu,
+    int min_chunk, int max_splits, const int32_t* __restrict__ kv_shift, uint64_t* __restrict__ bits,
+    int32_t* __restrict__ plan, int32_t* __restrict__ counters, int n_counters,
+    int64_t* __restrict__ position_ids, int32_t* __restrict__ left_pads) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kv_len = (int)prev + n;
+  if (blockIdx.y == B) {
+    // ---- the plan ------------------------------------------------------------------------------
+    if (blockIdx.x != 0) return;
+    extern __shared__ int s_span[];  // [2][B]
+    int* s_key_min = s_span;
+    int* s_key_end = s_span + B;
+    for (int b = wave; b < B; b += kWaves) {
+      const PM* pm = padding_mask + (int64_t)b * pm_row_stride;
+      int first = (int)prev;
+      for (int64_t base = 0; base < prev && first == (int)prev; base += 64) {
+        const int64_t j = base + lane;
+        const uint64_t word = __ballot(j < prev && pm[j] != (PM)pm_pad_value);
+        if (word != 0) first = (int)base + __builtin_ctzll(word);
+      }
+      if (lane == 0) {
+        s_key_min[b] = first;  // (== prev when no key of the left part is attended: slot 0 attends to itself)
+        s_key_end[b] = (int)prev + counts[b];
+        if (left_pads) left_pads[b] = first;
+      }
+    }
+    build_plan(s_key_min, s_key_end, B, n, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan,
+               counters, n_counters);
+    return;
+  }
+  // ---- mask bits and position ids of kTreeSlots slots of one batch row -------------------------
+  __shared__ uint64_t s_left[kMaxLeftWords];
+  __shared__ int s_first;
+  const int b = blockIdx.y;
+  if (threadIdx.x == 0) s_first = (int)prev;
+  __syncthreads();
+  const int nw_left = left_words<PM>(padding_mask + (int64_t)b * pm_row_stride, prev, (PM)pm_pad_value, s_left, &s_first);
+  __syncthreads();
+  const int64_t start = prev - s_first;  // tokens of the row so far: its length minus its left padding
+  const int q_end = (blockIdx.x + 1) * kTreeSlots < n ? (blockIdx.x + 1) * kTreeSlots : n;
+  for (int q = blockIdx.x * kTreeSlots + wave; q < q_end; q += kWaves) {
+    const int f = (int)packed_token_indices[(int64_t)b * n + q];
+    const int i = f / L, k = f - i * L;
+    // lane kk <= k holds the packed slot of position kk of the source beam
+    const int tgt = lane <= k ? (int)unpacker[(int64_t)b * WL + i * L + lane] : -1;
+    uint64_t* out = bits + ((int64_t)b * n + q) * words;
+    // left part from LDS; tree part: bit prev + tgt[kk] for kk <= k (every lane looks at every
+    // target and keeps the bits that fall into its word)
+    const int w_tree = (int)(prev >> 6);  // first word that can hold a tree bit
+    for (int w0 = 0; w0 < words; w0 += 64) {
+      const int w = w0 + lane;
+      uint64_t word = w < nw_left ? s_left[w] : 0ull;
+      if (w0 + 63 >= w_tree) {
+        for (int kk = 0; kk <= k; ++kk) {
+          const int c = (int)prev + __shfl(tgt, kk);
+          if ((c >> 6) == w) word |= 1ull << (c & 63);
+        }
+      }
+      if (w < words) out[w] = word;
+    }
+    if (lane == 0 && position_ids) position_ids[(int64_t)b * n + q] = start + k;
   }
 }
 
@@ -222,4 +338,45 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
                      words, rd::kAttnChunk, max_splits, n_heads, compute_units(), kv_row_shift, plan,
                      plan + rd::attn_counter_offset(batch, n_q, kv_len), (int)rd::attn_counter_ints(batch, n_q)); }
   return rd::check_launch("rd_attn_prepare(plan)");
+}
+
+extern "C" int rd_tree_attn_prepare(const int64_t* unpacker, const int64_t* packed_token_indices,
+                                    const int32_t* counts, const void* padding_mask, int pm_elem_bytes,
+                                    int64_t pm_row_stride, int64_t pm_pad_value, int64_t prev, int batch,
+                                    int width, int length, int n, int n_heads, uint64_t* bits,
+                                    int32_t* plan, int64_t* position_ids, int32_t* left_pads,
+                                    const int32_t* kv_row_shift, void* stream) {
+  RD_REQUIRE(batch > 0 && width > 0 && length > 0 && prev >= 0 && n > 0 && n_heads > 0, RD_EINVAL,
+             "rd_tree_attn_prepare: bad sizes (batch %d width %d length %d prev %lld n %d n_heads %d)", batch,
+             width, length, (long long)prev, n, n_heads);
+  RD_REQUIRE(length <= 64 && n <= width * length, RD_ELIMIT, "rd_tree_attn_prepare: length %d (<= 64), n %d (<= width*length)",
+             length, n);
+  RD_REQUIRE(prev <= (int64_t)kMaxLeftWords * 64 && prev + n < 2147483647LL, RD_ELIMIT,
+             "rd_tree_attn_prepare: prev %lld > %d (use rd_tree_mask + rd_attn_prepare)", (long long)prev, kMaxLeftWords * 64);
+  const int kv_len = (int)prev + n;
+  RD_REQUIRE(batch < 65535 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
+             "rd_tree_attn_prepare: batch %d too large for kv_len %d", batch, kv_len);
+  RD_REQUIRE(unpacker && packed_token_indices && counts && bits && plan, RD_EINVAL, "rd_tree_attn_prepare: null pointer");
+  RD_REQUIRE(prev == 0 || (padding_mask && pm_row_stride >= prev), RD_EINVAL,
+             "rd_tree_attn_prepare: padding_mask missing or pm_row_stride %lld < prev %lld", (long long)pm_row_stride, (long long)prev);
+  RD_REQUIRE(pm_elem_bytes == 1 || pm_elem_bytes == 4 || pm_elem_bytes == 8, RD_EINVAL,
+             "rd_tree_attn_prepare: pm_elem_bytes must be 1, 4 or 8 (got %d)", pm_elem_bytes);
+  const int words = (kv_len + 63) / 64;
+  const int max_splits = rd::attn_max_splits(kv_len);
+  hipStream_t s = rd::as_stream(stream);
+  const dim3 grid((n + kTreeSlots - 1) / kTreeSlots, batch + 1);
+  int32_t* counters = plan + rd::attn_counter_offset(batch, n, kv_len);
+  const int n_counters = (int)rd::attn_counter_ints(batch, n);
+#define RD_LAUNCH_TP(T)                                                                               \
+  do { rd::ScopedTiming rd_t("tree_prepare_kernel", s);                                               \
+    hipLaunchKernelGGL(tree_prepare_kernel<T>, grid, dim3(kThreads), 2 * batch * sizeof(int), s, unpacker, \
+                       packed_token_indices, counts, reinterpret_cast<const T*>(padding_mask), pm_row_stride,  \
+                       pm_pad_value, prev, batch, width * length, length, n, words, n_heads, compute_units(),  \
+                       rd::kAttnChunk, max_splits, kv_row_shift, bits, plan, counters, n_counters, position_ids, \
+                       left_pads); } while (0)
+  if (pm_elem_bytes == 1) RD_LAUNCH_TP(uint8_t);
+  else if (pm_elem_bytes == 4) RD_LAUNCH_TP(int32_t);
+  else RD_LAUNCH_TP(int64_t);
+#undef RD_LAUNCH_TP
+  return rd::check_launch("rd_tree_attn_prepare");
 }

@@ -38,7 +38,7 @@ _PROTOTYPES = {
     "rd_count_left_paddings": (_I, [_P, _L, _L, _I, _L, _P, _P]),
     "rd_position_ids": (_I, [_P, _L, _L, _I, _L, _P, _L, _I, _P, _P]),
     "rd_realign_plan_ints": (_Z, [_I, _I]),
-    "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P, _P]),
+    "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P, _P, _P]),
     "rd_kv_unpack": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _I, _I, _P]),
     "rd_kv_compact": (_I, [_P, _I, _I, _I, _L, _L, _L, _I, _P, _P]),
     "rd_kv_append": (_I, [_P, _I, _I, _I, _L, _L, _I, _P, _P]),
@@ -54,6 +54,7 @@ _PROTOTYPES = {
     "rd_attn_plan_ints": (_Z, [_I, _I, _I]),
     "rd_attn_bits_words": (_Z, [_I, _I, _I]),
     "rd_attn_prepare": (_I, [_P, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P]),
+    "rd_tree_attn_prepare": (_I, [_P, _P, _P, _P, _I, _L, _L, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P]),
     "rd_attention_workspace_bytes": (_Z, [_I, _I, _I, _I, _I]),
     "rd_verify_attention": (
         _I,

@@ -160,14 +160,17 @@ def realign_enqueue(
     cache: kv_cache.Cache,
     pad_token_id: int,
     unpacker: Optional[torch.Tensor] = None,
+    left_pads: Optional[torch.Tensor] = None,
 ) -> PendingRealign:
     """Appends the accepted tokens to ids and cache and re-right-aligns both; nothing is read back.
 
     With unpacker=None the cache must already be unpacked (Cache.unpack); with the unpacker given
-    the accepted rows are taken straight from the packed slots and the unpack step is not needed."""
+    the accepted rows are taken straight from the packed slots and the unpack step is not needed.
+    left_pads: (B,) int32 leading pad counts of input_ids, if the caller has them already."""
     assert input_ids.dtype == torch.long, f"prev_input_ids.dtype {input_ids.dtype} is not long"
     B, W, L = beams.shape
     prev = input_ids.shape[1]
+    assert left_pads is None or (left_pads.shape == (B,) and left_pads.dtype == torch.int32 and left_pads.is_contiguous())
     if prev > 0 and input_ids.stride(1) != 1:
         input_ids = input_ids.contiguous()
     beams = beams.contiguous()
@@ -184,7 +187,7 @@ def realign_enqueue(
             _hip.ptr(input_ids) if prev > 0 else None, input_ids.stride(0), prev,
             _hip.ptr(n_tokens_in_seq), _hip.ptr(seq_in_beam), _hip.ptr(beams), _hip.ptr(unpacker),
             B, W, L, pad_token_id, _hip.ptr(plan), _hip.ptr(ids_buf),
-            _hip.ptr(cache.shift) if cache.rows_in_place else None, _hip.stream(),
+            _hip.ptr(cache.shift) if cache.rows_in_place else None, _hip.ptr(left_pads), _hip.stream(),
         )
     )
     if cache.rows_in_place:

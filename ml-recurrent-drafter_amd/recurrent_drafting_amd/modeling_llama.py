@@ -283,8 +283,9 @@ class LlamaForCausalLM(LlamaPreTrainedModel):
                       rows: Optional[PackedRows] = None) -> torch.Tensor:
         """Final-norm hidden states (B, q, hidden), or (rows.rows, hidden) of the slots that
         exist; rows that attend to nothing attend to everything, as the reference arranges on a
-        GPU (modeling_llama.py:264-265)."""
-        prepared = attention.prepare(
+        GPU (modeling_llama.py:264-265).  attention_mask: (B, q, kv) bool, or an
+        attention.PreparedMask (e.g. from tree_attention.prepare_attention)."""
+        prepared = attention_mask if isinstance(attention_mask, attention.PreparedMask) else attention.prepare(
             attention_mask, fix_empty_rows=True, n_heads=self.config.num_attention_heads,
             kv_shift=_kv_shift(past_key_values))
         return self.model(input_ids=input_ids, attention_mask=prepared, position_ids=position_ids,

@@ -4,8 +4,8 @@
 (recurrent_drafting/recurrent_drafting.py:559-705).  One step is
 
     draft   beam search on the drafter head          rd_beam_topk x (L-1)      (+ torch GEMMs)
-    verify  beams -> prefix tree, mask, LLM forward   rd_tree_build, rd_tree_mask, rd_attn_prepare,
-                                                      rd_verify_attention per layer (+ torch GEMMs)
+    verify  beams -> prefix tree, mask bits + plan +  rd_tree_build, rd_tree_attn_prepare,
+            position ids, LLM forward                 rd_verify_attention per layer (+ torch GEMMs)
     accept  greedy: argmax over the packed rows,      rd_argmax_rows, rd_accept_greedy
             longest agreeing prefix
             sampling: row statistics of the packed    rd_verify_row_stats, rd_accept_sample,
@@ -191,9 +191,11 @@ class RecurrentDrafting(torch.nn.Module):
         llm, beams = self.llm, drafted.beams
         greedy = sampling_args.greedy
         with step_record.time("verify_candidates"):
-            prev = input_ids.shape[1]
-            mask = tree_attention.build_mask(tree, input_ids, pad_value=pad)  # (no `input_ids != pad` launch)
-            position_ids = acceptance.tree_position_ids(input_ids, pad, tree.position_offsets)
+            # mask bits, work plan, position ids and left pad counts of the packed tree in one launch:
+            # no byte mask, no `input_ids != pad`
+            mask, position_ids, left_pads = tree_attention.prepare_attention(
+                tree, input_ids, pad_value=pad, n_heads=llm.config.num_attention_heads,
+                kv_shift=cache.shift if cache.rows_in_place else None)
             # the slots past a row's own tree are padding (other rows' tokens, tree_attention.py:70-122)
             # that the reference computes and never reads: the model runs on the slots that exist
             rows = tree.rows()
@@ -224,7 +226,8 @@ class RecurrentDrafting(torch.nn.Module):
                     n_tokens, seq_in_beam = acceptance.sample_accept(beams, log_p, drafted.log_q, uniforms)
             with step_record.time("update_kv_cache_and_input_ids"):
                 realignment = acceptance.realign_enqueue(
-                    input_ids, n_tokens, seq_in_beam, beams, cache, pad, unpacker=tree.unpacker
+                    input_ids, n_tokens, seq_in_beam, beams, cache, pad, unpacker=tree.unpacker,
+                    left_pads=left_pads,
                 )
             if greedy:
                 with step_record.time("greedy_prepare_next_input"):

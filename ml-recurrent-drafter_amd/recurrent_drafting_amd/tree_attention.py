@@ -140,6 +140,42 @@ def build_mask(tree: PackedTree, padding_mask: torch.Tensor, pad_value: int = 0)
     return out
 
 
+def prepare_attention(tree: PackedTree, padding_mask: torch.Tensor, pad_value: int = 0, n_heads: int = 32,
+                      kv_shift: Optional[torch.Tensor] = None):
+    """For a caller that goes straight to the HIP attention: the tree mask as bits plus the work
+    plan (an `attention.PreparedMask`, what `attention.prepare(build_mask(...))` gives, bit for
+    bit), the position ids (B, n) of the packed tokens (recurrent_drafting.py:449-458) and the
+    leading pad count of every row (B,) int32 -- one launch, no (B, n, prev+n) byte mask.
+    padding_mask / pad_value as for `build_mask`; n_heads sizes the work items; kv_shift as for
+    `attention.prepare`."""
+    from . import attention
+
+    B, W, L = tree.unpacker.shape
+    assert padding_mask.dim() == 2 and padding_mask.shape[0] == B
+    assert padding_mask.dtype in (torch.int32, torch.int64, torch.bool, torch.uint8)
+    prev = padding_mask.shape[1]
+    if prev > 0 and padding_mask.stride(1) != 1:
+        padding_mask = padding_mask.contiguous()
+    assert kv_shift is None or (kv_shift.shape == (B,) and kv_shift.dtype == torch.int32 and kv_shift.is_contiguous())
+    n, kv_len = tree.n, prev + tree.n
+    lib = _hip.lib()
+    dev = tree.unpacker.device
+    bits = torch.empty(lib.rd_attn_bits_words(B, n, kv_len), dtype=torch.int64, device=dev)
+    plan = torch.empty(lib.rd_attn_plan_ints(B, n, kv_len), dtype=torch.int32, device=dev)
+    position_ids = torch.empty((B, n), dtype=torch.long, device=dev)
+    left_pads = torch.empty(B, dtype=torch.int32, device=dev)
+    _hip.check(
+        lib.rd_tree_attn_prepare(
+            _hip.ptr(tree.unpacker), _hip.ptr(tree.packed_token_indices), _hip.ptr(tree.counts),
+            _hip.ptr(padding_mask) if prev > 0 else None, padding_mask.element_size(),
+            padding_mask.stride(0) if prev > 0 else 0, int(pad_value), prev, B, W, L, n, int(n_heads),
+            _hip.ptr(bits), _hip.ptr(plan), _hip.ptr(position_ids), _hip.ptr(left_pads), _hip.ptr(kv_shift),
+            _hip.stream(),
+        )
+    )
+    return attention.PreparedMask(bits.view(B, n, -1), plan, B, n, kv_len), position_ids, left_pads
+
+
 def pack(
     beams: torch.Tensor, padding_mask: torch.Tensor
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:

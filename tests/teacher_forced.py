@@ -9,7 +9,8 @@ with (token ids, drafter context, first token, KV cache contents) to oracle/torc
 same GPU, then compares what came out:
 
   beams            oracle beam search on the same context and token (same bf16 torch GEMMs)
-  tree             packed tokens, unpacker, mask, position offsets of the HIP beams: bit-exact
+  tree             packed tokens, unpacker, position offsets and ids, left pad counts, and the mask
+                   (unpacked from the bits the attention consumes) of the HIP beams: bit-exact
   packed logits    against the float32 restatement (bf16 weights upcast), within `tol` of the
                    logits' scale; the restatement run in bf16 with stock torch ops is measured
                    against the same float32 figures, as the yardstick for a bf16 implementation
@@ -57,6 +58,14 @@ class StepReport:
     kv_err: float
 
 
+def _bits_to_mask(bits: torch.Tensor, kv_len: int) -> torch.Tensor:
+    """(B, n, words) int64 words -> (B, n, kv_len) bool."""
+    shifts = torch.arange(64, device=bits.device, dtype=torch.int64)
+    flat = ((bits.unsqueeze(-1) >> shifts) & 1).flatten(2)
+    assert not bool(flat[:, :, kv_len:].any())
+    return flat[:, :, :kv_len].bool()
+
+
 def _snapshot(cache, length: int):
     """Copy of the cache in the reference's layout (column c of row b in cache row c)."""
     from recurrent_drafting_amd import kv_cache
@@ -101,13 +110,14 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
     llm32 = copy.deepcopy(llm).float()  # bf16 weights upcast (the drafter is compared in its own dtype)
     model = rd.RecurrentDrafting(llm, drafter)
     seen = {}
-    real_mask, real_argmax = tree_attention.build_mask, acceptance.argmax_rows
+    real_prepare, real_argmax = tree_attention.prepare_attention, acceptance.argmax_rows
     real_accept, real_realign = acceptance.greedy_accept, acceptance.realign_enqueue
     real_draft = drafter.beam_search_candidates
 
-    def w_mask(tree, padding_mask, pad_value=0):
-        out = real_mask(tree, padding_mask, pad_value)
-        seen.update(tree=tree, ids=padding_mask, mask=out)
+    def w_prepare(tree, padding_mask, pad_value=0, n_heads=32, kv_shift=None):
+        out = real_prepare(tree, padding_mask, pad_value, n_heads, kv_shift)
+        prepared, position_ids, left_pads = out
+        seen.update(tree=tree, ids=padding_mask, bits=prepared.bits, position_ids=position_ids, left_pads=left_pads)
         return out
 
     def w_argmax(logits):
@@ -125,10 +135,10 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
                     next_tokens=nxt, last_slot=last)
         return n, s, nxt, last
 
-    def w_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker=None):
+    def w_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker=None, left_pads=None):
         seen.update(cache=cache, shift=cache.shift.clone(),
                     snap=_snapshot(cache, cache.sliced[0][0].length))
-        return real_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker)
+        return real_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker, left_pads)
 
     drafts = []  # draft k feeds step k; it is queued while step k-1 is being finished
 
@@ -139,7 +149,7 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
 
     reports: List[StepReport] = []
     prev_step = None  # what the previous step left for the cache comparison
-    with mock.patch.object(tree_attention, "build_mask", w_mask), \
+    with mock.patch.object(tree_attention, "prepare_attention", w_prepare), \
             mock.patch.object(acceptance, "argmax_rows", w_argmax), \
             mock.patch.object(acceptance, "greedy_accept", w_accept), \
             mock.patch.object(acceptance, "realign_enqueue", w_realign), \
@@ -192,7 +202,7 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
     o_packed, o_unpacker, o_mask, o_off = P.pack(beams, (ids != pad).to(ids.dtype))
     assert o_packed.shape[1] == n_q, (o_packed.shape, n_q)
     assert torch.equal(tree.unpacker, o_unpacker) and torch.equal(tree.packed_beams, o_packed)
-    assert torch.equal(tree.position_offsets, o_off) and torch.equal(st["mask"], o_mask)
+    assert torch.equal(tree.position_offsets, o_off) and torch.equal(_bits_to_mask(st["bits"], prev + n_q), o_mask)
     counts = tree.counts[:B].long()
     assert int(counts.sum()) == total and int(counts.max()) == n_q
     exists = (torch.arange(n_q, device=dev)[None, :] < counts[:, None]).flatten()
@@ -201,6 +211,7 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
     # -- verify forward: float32 restatement (and the bf16 one as the yardstick) on the same cache ---
     snap = st["snap"]  # (layers, 2, B, H, max_len, D), columns in place, tree rows at [prev, prev+n_q)
     pos = (prev - P.count_left_pads(ids, pad))[:, None] + o_off
+    assert torch.equal(st["position_ids"], pos) and torch.equal(st["left_pads"].long(), P.count_left_pads(ids, pad))
     n_layers, _, _, Hkv, max_len, D = snap.shape
 
     def restate(model, dtype):

@@ -1,4 +1,5 @@
-"""GPU parity: rd_tree_build / rd_tree_mask through the C ABI vs the CPU oracle (bit-exact)."""
+"""GPU parity: rd_tree_build / rd_tree_mask / rd_tree_attn_prepare through the C ABI vs the CPU
+oracle (bit-exact)."""
 import numpy as np
 import pytest
 import torch
@@ -30,6 +31,40 @@ def _check_against_oracle(beams, padding_mask):
         assert g_mask.dtype == torch.bool and g_mask.shape == mask.shape
         assert np.array_equal(g_mask.cpu().numpy(), mask)
         assert np.array_equal(g_tok.cpu().numpy(), tok) and np.array_equal(g_off.cpu().numpy(), off)
+        _check_prepare_attention(tree, _dev(padding_mask, dt), mask, off)
+
+
+def bits_to_mask(bits, kv_len):
+    """(B, n, words) int64 holding uint64 words -> (B, n, kv_len) bool; bits past kv_len must be zero."""
+    words = bits.cpu().numpy().view(np.uint64)
+    B, n, nw = words.shape
+    flat = np.unpackbits(words.reshape(B, n, nw, 1).view(np.uint8), axis=-1, bitorder="little").reshape(B, n, nw * 64)
+    assert not flat[:, :, kv_len:].any()
+    return flat[:, :, :kv_len].astype(bool)
+
+
+def _check_prepare_attention(tree, padding_mask, want_mask, want_offsets, pad_value=0, n_heads=3, shift=None):
+    """rd_tree_attn_prepare against the oracle's mask and against the two-step path
+    (rd_tree_mask -> rd_attn_prepare), bit for bit: mask bits, plan records, position ids, pad counts."""
+    from recurrent_drafting_amd import acceptance, attention, tree_attention
+
+    B, n, kv_len = want_mask.shape
+    prev = kv_len - n
+    prepared, pos, pads = tree_attention.prepare_attention(tree, padding_mask, pad_value, n_heads, shift)
+    assert np.array_equal(bits_to_mask(prepared.bits, kv_len), want_mask)
+    pm = padding_mask.cpu().numpy()
+    want_pads = np.array([next((j for j in range(prev) if pm[b, j] != pad_value), prev) for b in range(B)])
+    assert np.array_equal(pads.cpu().numpy(), want_pads)
+    assert np.array_equal(pos.cpu().numpy(), (prev - want_pads)[:, None] + want_offsets)
+    two_step = attention.prepare(tree_attention.build_mask(tree, padding_mask, pad_value), fix_empty_rows=True,
+                                 n_heads=n_heads, kv_shift=shift)
+    assert torch.equal(prepared.bits, two_step.bits)
+    a, b = prepared.plan.cpu().numpy(), two_step.plan.cpu().numpy()
+    n_items = int(b[0])
+    used = 8 + 4 * B + 8 * n_items  # header, per-row records, work items (what the attention reads)
+    assert np.array_equal(a[:used], b[:used])
+    counters = int(B * 128 * ((n + 255) // 256))
+    assert not a[-counters:].any()
 
 
 def test_reference_literals(literals):
@@ -125,3 +160,27 @@ def test_mask_from_token_ids_equals_mask_from_the_comparison():
         want = tree_attention.build_mask(tree, ids != pad)
         got = tree_attention.build_mask(tree, ids, pad_value=pad)
         assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_prepare_attention_from_token_ids_with_pads_by_value_and_row_shifts(seed):
+    """The fused loop's call: the token ids stand in for the padding mask (pad id by value, also in
+    the middle of a row), rows with nothing but padding, and a per-row cache shift in the plan."""
+    from recurrent_drafting_amd import tree_attention
+
+    rng = np.random.default_rng(seed)
+    B, W, L = [(3, 5, 4), (8, 45, 5), (2, 64, 5), (5, 7, 6)][seed]
+    prev = [9, 700, 64, 130][seed]
+    beams = T.synthetic_beams(B, W, L, vocab=40, seed=seed) + 1
+    ids = rng.integers(1, 50, size=(B, prev))
+    pad = 7
+    ids[ids == pad] = 8
+    for b in range(B):
+        ids[b, : rng.integers(0, prev // 2)] = pad
+    ids[0, prev // 2 + 1] = pad  # a generated token that equals the pad id is masked as a key
+    ids[B - 1, :] = pad          # nothing but padding: the tree rows still attend to themselves
+    tok, unp, mask, off, idx = T.pack(beams, (ids != pad).astype(np.int64))
+    tree = tree_attention.build_tree(_dev(beams))
+    shift = torch.tensor(rng.integers(-3, 4, size=B), dtype=torch.int32, device="cuda")
+    _check_prepare_attention(tree, _dev(ids), mask, off, pad_value=pad, n_heads=32, shift=shift)
+    _check_prepare_attention(tree, _dev(ids), mask, off, pad_value=pad, n_heads=1)
