@@ -4,7 +4,7 @@
 // nothing is reshaped into a matrix product.  Three kernels:
 //   tree_rows_kernel   per row: owner of every prefix, unpacker, the row's own packed list
 //   tree_fill_kernel   per row: batch-wide offsets, max over rows, spill-over fill of the padding
-//   tree_mask_kernel   per packed row: one row of the (batch, max_n, prev+max_n) byte mask
+//   tree_mask_kernel   per chunk of whole output lines: bytes of the (batch, max_n, prev+max_n) mask
 #include "rd_common.h"
 
 namespace {
@@ -160,53 +160,147 @@ __global__ __launch_bounds__(kThreads) void tree_fill_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// One workgroup per (batch row, packed slot).  Left part: the key's padding flag; tree part:
-// True at the packed slots of the source beam's positions 0..k.
+// The byte mask (batch, max_n, prev + max_n).  Left part of a row: the key's padding flag; tree
+// part: True at the packed slots of the source beam's positions 0..k.
+// A workgroup writes one CHUNK of a batch row's mask bytes: a range of whole 128-byte lines of the
+// output, about kMaskRows mask rows long (16 KiB at most), whatever the row length -- so every line
+// is written once, in full, by one workgroup (a workgroup per mask row wrote 2.7 kB rows that
+// start and end in the middle of lines: 2.3x the traffic on short rows, 90 000 workgroups on a
+// batch of 512).  Per chunk the row's padding flags are turned into bit words once (LDS), and the
+// (k, target slots) of the chunk's rows are staged in LDS.
 // ---------------------------------------------------------------------------------------------
+constexpr int kMaskRows = 30;        // mask rows per chunk, about
+constexpr int kMaskRowsLds = 34;     // rows a chunk can touch: kMaskRows + both partial ends + slack
+constexpr int kMaskMaxChunk = 16384;
+constexpr int kMaskLeftWords = 2048; // padding flags of at most 131072 keys
+
+__host__ __device__ inline int64_t mask_chunk_bytes(int64_t row_len) {
+  int64_t c = kMaskRows * row_len / 128 * 128;
+  if (c < 128) c = kMaskRows * row_len;  // rows of a few bytes: whole lines are not worth keeping to
+  return c > kMaskMaxChunk ? kMaskMaxChunk : c;
+}
+
+// eight bits -> eight bytes of 0 / 1, bit 0 in the lowest byte
+__device__ inline uint64_t bits_to_bytes(uint32_t b) {
+  const uint64_t spread = ((uint64_t)b * 0x0101010101010101ull) & 0x8040201008040201ull;
+  return ((spread + 0x7f7f7f7f7f7f7f7full) >> 7) & 0x0101010101010101ull;
+}
+
 template <typename PM>
 __global__ __launch_bounds__(kThreads) void tree_mask_kernel(
     const int64_t* __restrict__ unpacker, const int64_t* __restrict__ packed_token_indices,
     const int32_t* __restrict__ counts, const PM* __restrict__ padding_mask,
     int64_t pm_row_stride, int64_t prev, int B, int WL, int L, uint8_t* __restrict__ mask,
     int64_t pm_pad_value) {
+  __shared__ uint64_t s_left[kMaskLeftWords];
+  __shared__ int16_t s_tgt[kMaskRowsLds * kMaxLength];
+  __shared__ int s_k[kMaskRowsLds];
   const int max_n = counts[B];
-  const int n = blockIdx.x;
   const int b = blockIdx.y;
-  if (n >= max_n) return;
-  __shared__ int s_tgt[kMaxLength];
-  const int f = (int)packed_token_indices[(int64_t)b * max_n + n];
-  const int i = f / L, k = f - i * L;
-  if (threadIdx.x <= k) s_tgt[threadIdx.x] = (int)unpacker[(int64_t)b * WL + i * L + threadIdx.x];
-  __syncthreads();
-
   const int64_t row_len = prev + max_n;
-  const int64_t row_off = ((int64_t)b * max_n + n) * row_len;
-  uint8_t* out = mask + row_off;
-  const PM* pm = padding_mask + (int64_t)b * pm_row_stride;
-
-  auto value = [&](int64_t c) -> uint8_t {
-    if (c < prev) return pm[c] != (PM)pm_pad_value;
-    const int t = (int)(c - prev);
-    uint8_t hit = 0;
-    for (int kk = 0; kk <= k; ++kk) hit |= (s_tgt[kk] == t);
-    return hit;
+  const int64_t total = (int64_t)max_n * row_len;  // mask bytes of one batch row
+  const int64_t chunk = mask_chunk_bytes(row_len);
+  // chunks are cut at absolute 128-byte lines of the output
+  const uintptr_t base_addr = reinterpret_cast<uintptr_t>(mask) + (uintptr_t)((int64_t)b * total);
+  const int64_t lead = (int64_t)(base_addr & 127);  // bytes of this batch row's first line that belong to the row before
+  int64_t lo = (int64_t)blockIdx.x * chunk - lead, hi = lo + chunk;  // relative to the batch row's first byte
+  lo = lo < 0 ? 0 : lo;
+  hi = hi > total ? total : hi;
+  if (lo >= hi) return;
+  const int q0 = (int)(lo / row_len), q1 = (int)((hi - 1) / row_len);  // first and last mask row touched
+  // stage: k and the target slots of every row touched; the padding flags of the left part as bits
+  for (int t = threadIdx.x; t < (q1 - q0 + 1) * L; t += kThreads) {
+    const int r = t / L, kk = t - r * L;
+    const int f = (int)packed_token_indices[(int64_t)b * max_n + q0 + r];
+    const int i = f / L, k = f - i * L;
+    if (kk == 0) s_k[r] = k;
+    s_tgt[r * kMaxLength + kk] = kk <= k ? (int16_t)unpacker[(int64_t)b * WL + i * L + kk] : (int16_t)-1;
+  }
+  {
+    const PM* pm = padding_mask + (int64_t)b * pm_row_stride;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nw = (int)((prev + 63) >> 6);
+    // four words per wave and round: the loads of a round are in flight together
+    constexpr int kWavesHere = kThreads / 64;
+    for (int w0 = wave; w0 < nw; w0 += 4 * kWavesHere) {
+      bool on[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t j = (int64_t)(w0 + u * kWavesHere) * 64 + lane;
+        on[u] = j < prev && pm[j] != (PM)pm_pad_value;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint64_t word = __ballot(on[u]);
+        if (lane == 0 && w0 + u * kWavesHere < nw) s_left[w0 + u * kWavesHere] = word;
+      }
+    }
+  }
+  __syncthreads();
+  uint8_t* out = mask + (int64_t)b * total;
+  const int nw_left = (int)((prev + 63) >> 6);
+  // flags of columns c .. c+15 of staged row r as sixteen bits (columns past the row's end: junk)
+  auto row_flags = [&](int r, int64_t c) -> uint32_t {
+    uint32_t f = 0;
+    if (c < prev) {
+      const int w = (int)(c >> 6), sh = (int)(c & 63);
+      uint64_t x = s_left[w] >> sh;
+      if (sh > 48 && w + 1 < nw_left) x |= s_left[w + 1] << (64 - sh);
+      f = (uint32_t)x & 0xffffu;  // (bits of columns >= prev are zero in the words)
+    }
+    if (c + 16 > prev) {
+      const int16_t* tg = s_tgt + r * kMaxLength;
+      const int k = s_k[r];
+      for (int kk = 0; kk <= k; ++kk) {
+        const int64_t d = prev + tg[kk] - c;
+        if ((uint64_t)d < 16) f |= 1u << d;
+      }
+    }
+    return f;
   };
-
-  int64_t head = (16 - (row_off & 15)) & 15;
-  head = head < row_len ? head : row_len;
-  for (int64_t c = threadIdx.x; c < head; c += kThreads) out[c] = value(c);
-  const int64_t nvec = (row_len - head) >> 4;
+  // sixteen consecutive mask bytes that begin at column c of staged row r, as bits; they may run on
+  // into the following rows
+  auto flags16 = [&](int r, int64_t c) -> uint32_t {
+    uint32_t f = row_flags(r, c);
+    int64_t have = row_len - c;  // bytes of f that belong to row r
+    while (have < 16) {
+      ++r;
+      f = (f & ((1u << have) - 1u)) | (row_flags(r, 0) << have);
+      have += row_len;
+    }
+    return f & 0xffffu;
+  };
+  // bytes in front of the first 16-byte boundary, whole 16-byte vectors, bytes behind the last one
+  int64_t head = (16 - (int64_t)((base_addr + (uintptr_t)lo) & 15)) & 15;
+  head = head < hi - lo ? head : hi - lo;
+  const int64_t nvec = (hi - lo - head) >> 4;
+  for (int64_t o = lo + threadIdx.x; o < lo + head; o += kThreads)
+    out[o] = (uint8_t)(row_flags((int)(o / row_len) - q0, o % row_len) & 1u);
+  // a thread's vectors are kThreads * 16 bytes apart: (row, column) of the first one by division,
+  // of the others by stepping
+  int r_next = 0;
+  int64_t c_next = 0;
+  if (threadIdx.x < nvec) {
+    const int64_t o = lo + head + ((int64_t)threadIdx.x << 4);
+    r_next = (int)(o / row_len);
+    c_next = o - (int64_t)r_next * row_len;
+    r_next -= q0;
+  }
   for (int64_t v = threadIdx.x; v < nvec; v += kThreads) {
-    const int64_t c0 = head + (v << 4);
+    const int64_t o = lo + head + (v << 4);
+    const uint32_t f = flags16(r_next, c_next);
+    c_next += kThreads * 16;
+    while (c_next >= row_len) { c_next -= row_len; ++r_next; }
     union {
-      uint8_t b8[16];
+      uint64_t b64[2];
       uint4 v4;
     } u;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) u.b8[e] = value(c0 + e);
-    *reinterpret_cast<uint4*>(out + c0) = u.v4;
+    u.b64[0] = bits_to_bytes(f & 0xffu);
+    u.b64[1] = bits_to_bytes(f >> 8);
+    *reinterpret_cast<uint4*>(out + o) = u.v4;
   }
-  for (int64_t c = head + (nvec << 4) + threadIdx.x; c < row_len; c += kThreads) out[c] = value(c);
+  for (int64_t o = lo + head + (nvec << 4) + threadIdx.x; o < hi; o += kThreads)
+    out[o] = (uint8_t)(row_flags((int)(o / row_len) - q0, o % row_len) & 1u);
 }
 
 template <typename PM>
@@ -303,9 +397,16 @@ extern "C" int rd_tree_mask(const int64_t* unpacker, const int64_t* packed_token
              (long long)prev);
   RD_REQUIRE(pm_elem_bytes == 1 || pm_elem_bytes == 4 || pm_elem_bytes == 8, RD_EINVAL,
              "rd_tree_mask: pm_elem_bytes must be 1, 4 or 8 (got %d)", pm_elem_bytes);
+  RD_REQUIRE(prev <= (int64_t)kMaskLeftWords * 64, RD_ELIMIT, "rd_tree_mask: prev %lld > %d", (long long)prev,
+             kMaskLeftWords * 64);
   hipStream_t s = rd::as_stream(stream);
-  const dim3 grid(width * length, batch);
   const int WL = width * length;
+  // chunks per batch row for the largest tree the buffers allow (the real size is on the device):
+  // 64 KiB chunks of long rows, or about kMaskRows rows of short ones
+  const int64_t cap_bytes = (int64_t)WL * (prev + WL);
+  const int64_t chunks = cap_bytes / kMaskMaxChunk + WL / (kMaskRows - 2) + 4;  // (an upper bound for any tree size)
+  RD_REQUIRE(chunks <= 2147483647LL, RD_ELIMIT, "rd_tree_mask: mask too large");
+  const dim3 grid((unsigned)chunks, batch);
 #define RD_LAUNCH_MASK(T)                                                                       \
   do { rd::ScopedTiming rd_t("tree_mask_kernel", s); hipLaunchKernelGGL(tree_mask_kernel<T>, grid, dim3(kThreads), 0, s, unpacker,                  \
                      packed_token_indices, counts, reinterpret_cast<const T*>(padding_mask),    \
