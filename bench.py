@@ -1,6 +1,6 @@
 """Benchmark of the ReDrafter decode step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--extra-steps E] [--no-cpu-baseline]
     python bench.py --cpu-kernels      (per-kernel CPU baselines only; no GPU needed)
 
 Workload (the configuration the headline metric is quoted on): random-init Vicuna-7B-shaped Llama
@@ -12,7 +12,11 @@ greedy, generation capped at 500 + 2048 tokens.  A step is one draft -> verify -
 One JSON line on stdout: tokens/sec over the K timed steps (all eight sequences together), the
 roofline entry of the dominant hand-written kernel (attn_mfma_kernel, timed with HIP events inside
 the library while the timed region runs), and a CPU baseline: the torch restatement of the same
-step (oracle/torch_path.py) timed on this machine's host cores on a bounded sample.
+step (oracle/torch_path.py) timed on this machine's host cores on a bounded sample.  Beside the
+headline, the same step at other points of its operating range, E timed steps each (`long_context`:
+prompts of 1500 and 2500 tokens; `ragged_acceptance`: prompts of 1200 tokens with the acceptance
+decision replaced by random accepted lengths, so that rows shift, accepted rows are appended and
+the trees grow -- random-init models accept nothing by themselves).
 """
 
 from __future__ import annotations
@@ -38,6 +42,7 @@ BATCH, PROMPT, NEW_TOKENS, WIDTH, LENGTH, SEED = 8, 500, 2048, 45, 5, 123
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 TIMED_EVERY = 5  # the dominant kernel's launches are event-timed one in five
+CPU_STEPS = 3  # timed steps per layer count of the CPU baseline
 
 
 def log(*a):
@@ -68,17 +73,107 @@ def build_models(device: str, dtype: torch.dtype, n_layers: int, seed: int):
     return llm.eval(), drafter.eval()
 
 
-def prompts(device: str) -> torch.Tensor:
+def prompts(device: str, length: int = PROMPT) -> torch.Tensor:
     gen = torch.Generator(device="cpu").manual_seed(SEED)
-    return torch.randint(1, LLAMA_7B["vocab_size"], (BATCH, PROMPT), generator=gen).to(device)
+    return torch.randint(1, LLAMA_7B["vocab_size"], (BATCH, length), generator=gen).to(device)
 
 
 # -------------------------------------------------------------------------------------------------
 # GPU run
 # -------------------------------------------------------------------------------------------------
-def gpu_run(steps: int, warmup: int):
+def forced_acceptance(seed: int):
+    """Stand-in for the acceptance decision: random accepted lengths (0 .. length-1) and beams per
+    row and step.  Random-init models never accept a drafted token, so with the real decision the
+    rows never shift, nothing is appended behind a prompt of ragged length and the trees stay at
+    their smallest; this puts those paths into the timed region.  The tokens then mean nothing."""
+    gen = torch.Generator().manual_seed(seed)
+
+    def force(real):
+        def accept(beams, llm_tokens, unpacker=None):
+            n, s, nxt, last = real(beams, llm_tokens, unpacker)
+            B, W, L = beams.shape
+            n = torch.randint(0, L, (B,), generator=gen).to(beams.device)
+            s = torch.randint(0, W, (B,), generator=gen).to(beams.device)
+            rows = torch.arange(B, device=beams.device)
+            last = unpacker[rows, s, n] if unpacker is not None else s * L + n
+            nxt = llm_tokens[rows, last] if unpacker is not None else llm_tokens.reshape(B, -1)[rows, last]
+            return n, s, nxt, last
+        return accept
+    return force
+
+
+def timed_decode(model, ids, steps: int, warmup: int, max_new: int, force=None):
+    """Runs warmup + steps decode steps of one generation (a new one is started, prefill untimed,
+    whenever the cap is reached) and returns the timing of the `steps` steps, the shapes of the
+    attention launches in them and the HIP-event time of every TIMED_EVERY-th of those launches."""
     import recurrent_drafting_amd as rd
-    from recurrent_drafting_amd import _hip, attention
+    from recurrent_drafting_amd import _hip, acceptance, attention
+
+    max_length = ids.shape[1] + max_new
+    real_accept = acceptance.greedy_accept
+    if force is not None:
+        acceptance.greedy_accept = force(real_accept)
+    try:
+        ledger = rd.stats.Ledger(sync=False)
+
+        def new_stream():
+            return model.generate(ledger, ids, max_length, rd.BeamShape(WIDTH, LENGTH),
+                                  rd.SamplingArgs(1.0, True), rd.SpecialTokens(0, None))
+
+        stream = new_stream()
+        for _ in range(warmup):
+            next(stream)
+        torch.cuda.synchronize()
+        # HIP events around the launches of the dominant kernel, live in the timed region: every
+        # TIMED_EVERY-th launch in launch order (the two events of a launch keep the GPU idle for about
+        # 11 us; around all 32 launches of a step that is 2.4 % of the step, around every fifth 0.5 %;
+        # five is coprime to the 32 layers, so the sample walks through the layers).
+        shapes = []
+        attention.shape_log = shapes
+        _hip.timing_select("attn_mfma_kernel")
+        _hip.timing_sample(TIMED_EVERY)
+        _hip.timing_enable(True)
+        elapsed, timed = 0.0, 0
+        first_len = last_len = None
+        out = None
+        while timed < steps:
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            seg, exhausted = 0, False
+            while timed + seg < steps:
+                try:
+                    out = next(stream)
+                except StopIteration:
+                    exhausted = True
+                    break
+                seg += 1
+                first_len = out.shape[1] if first_len is None else first_len
+                last_len = out.shape[1]
+            torch.cuda.synchronize()
+            elapsed += time.perf_counter() - start
+            timed += seg
+            if exhausted:  # generation reached its cap: start another one (prefill is not timed)
+                stream = new_stream()
+                for _ in range(warmup):
+                    next(stream)
+        dominant = _hip.timing_collect()
+        _hip.timing_enable(False)
+        _hip.timing_select(None)
+        _hip.timing_sample(1)
+        attention.shape_log = None
+        final_pads = int((out == 0).long().cumprod(dim=-1).sum()) if out is not None else 0
+        stream.close()  # posts the open generation's record
+    finally:
+        acceptance.greedy_accept = real_accept
+    accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
+    per_seq_tokens = sum(a + 1 for a in accepted) / max(len(accepted), 1)
+    return dict(elapsed=elapsed, steps=timed, per_seq_tokens=per_seq_tokens, tokens=per_seq_tokens * BATCH * timed,
+                dominant=dominant, shapes=shapes, context=(first_len, last_len), final_left_pads=final_pads)
+
+
+def gpu_run(steps: int, warmup: int, extra_steps: int):
+    import recurrent_drafting_amd as rd
+    from recurrent_drafting_amd import _hip
 
     dev = "cuda:0"
     t0 = time.perf_counter()
@@ -88,71 +183,27 @@ def gpu_run(steps: int, warmup: int):
     model = rd.RecurrentDrafting(llm, drafter)
     n_tuned = rd.gemm_tuning.load()  # opt-in kernel selection table for the dense layers' GEMMs (look-up only)
     log(f"[bench] GEMM kernel selection table: {n_tuned} entries in effect")
-    ids = prompts(dev)
-    max_length = PROMPT + NEW_TOKENS
 
-    def new_stream(ledger):
-        return model.generate(ledger, ids, max_length, rd.BeamShape(WIDTH, LENGTH),
-                              rd.SamplingArgs(1.0, True), rd.SpecialTokens(0, None))
+    # ---- the headline: prompt 500, generation capped at 2048 new tokens ------------------------------
+    run = timed_decode(model, prompts(dev, PROMPT), steps, warmup, NEW_TOKENS)
+    run["null_us"] = _hip.timing_null_kernel_us(64)
 
-    ledger = rd.stats.Ledger(sync=False)
-    stream = new_stream(ledger)
-    done = 0
-    for _ in range(warmup):
-        next(stream)
-        done += 1
-    torch.cuda.synchronize()
+    # ---- the same step further along the trajectory, and with rows that accept drafted tokens -------
+    others = {}
+    if extra_steps > 0:
+        for name, prompt_len, force in (("context_1500", 1500, None), ("context_2500", 2500, None),
+                                        ("ragged_acceptance_context_1200", 1200, forced_acceptance(SEED))):
+            r = timed_decode(model, prompts(dev, prompt_len), extra_steps, warmup, 64 + 5 * (extra_steps + warmup), force)
+            r["null_us"] = run["null_us"]
+            others[name] = r
+            log(f"[bench] {name}: {r['elapsed'] / r['steps'] * 1e3:.2f} ms/step over {r['steps']} steps, "
+                f"context {r['context']}, {r['per_seq_tokens']:.2f} tokens per sequence and step")
 
-    # HIP events around the launches of the dominant kernel, live in the timed region: every
-    # TIMED_EVERY-th launch in launch order (the two events of a launch keep the GPU idle for about
-    # 11 us; around all 32 launches of a step that is 2.4 % of the step, around every fifth 0.5 %; five
-    # is coprime to the 32 layers, so the sample walks through the layers).  The events of ALL
-    # kernels are taken on the extra steps below.
-    shapes = []
-    attention.shape_log = shapes
-    _hip.timing_select("attn_mfma_kernel")
-    _hip.timing_sample(TIMED_EVERY)
-    _hip.timing_enable(True)
-    elapsed, tokens, timed = 0.0, 0, 0
-    first_len = last_len = None
-    while timed < steps:
-        torch.cuda.synchronize()
-        start = time.perf_counter()
-        seg = 0
-        exhausted = False
-        while timed + seg < steps:
-            try:
-                out = next(stream)
-            except StopIteration:
-                exhausted = True
-                break
-            seg += 1
-            first_len = out.shape[1] if first_len is None else first_len
-            last_len = out.shape[1]
-        torch.cuda.synchronize()
-        elapsed += time.perf_counter() - start
-        timed += seg
-        if exhausted:  # generation reached its cap: start another one (prefill is not timed)
-            stream = new_stream(ledger)
-            for _ in range(warmup):
-                next(stream)
-    dominant = _hip.timing_collect()
-    null_us = _hip.timing_null_kernel_us(64)
-    _hip.timing_enable(False)
-    _hip.timing_select(None)
-    _hip.timing_sample(1)
-    attention.shape_log = None
-    accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
-    # the generator that is still open has not posted its record yet; close it to flush
-    stream.close()
-    accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
-    per_seq_tokens = sum(a + 1 for a in accepted) / max(len(accepted), 1)
-    tokens = per_seq_tokens * BATCH * timed
-    no_pads = bool((out[:, 0] != 0).all())
-
-    # stage breakdown with the reference's synchronised timers, on a few extra steps
+    # ---- stage breakdown with the reference's synchronised timers, on a few extra steps ---------------
     ledger2 = rd.stats.Ledger(sync=True)
-    s2 = new_stream(ledger2)
+    ids = prompts(dev, PROMPT)
+    s2 = model.generate(ledger2, ids, PROMPT + NEW_TOKENS, rd.BeamShape(WIDTH, LENGTH),
+                        rd.SamplingArgs(1.0, True), rd.SpecialTokens(0, None))
     next(s2)
     next(s2)
     _hip.timing_enable(True)  # every kernel of the library, on four steps
@@ -162,52 +213,60 @@ def gpu_run(steps: int, warmup: int):
     kernels = _hip.timing_collect()
     _hip.timing_enable(False)
     s2.close()
-    wt = ledger2.records[0]["wall_times"]
-    stage = {k: sum(v[2:]) / len(v[2:]) for k, v in wt.items()}
-    ref_style = (per_seq_tokens) / (stage["generate_candidates"] + stage["verify_candidates"] + stage["accept_candidate_tokens"])
-
-    result = dict(
-        elapsed=elapsed, steps=timed, tokens=tokens, per_seq_tokens=per_seq_tokens, kernels=kernels,
-        dominant=dominant, null_us=null_us,
-        shapes=shapes, stage=stage, ref_style_tokens_per_second=ref_style,
-        context=(first_len, last_len), no_pads=no_pads,
-    )
+    rec = ledger2.records[0]
+    for key in ("step", "input_id_length", "avg_num_accepted"):  # drop the two warm-up steps
+        rec[key] = rec[key][2:]
+    rec["wall_times"] = {k: v[2:] for k, v in rec["wall_times"].items()}
+    stage = {k: sum(v) / len(v) for k, v in rec["wall_times"].items()}
+    table, _ = rd.stats.summarize(ledger2, BATCH, LENGTH - 1)  # the reference's own summary (stats.py:158-215)
+    run.update(kernels=kernels, stage=stage, ref_style_tokens_per_second=table.tokens_per_second, others=others)
     del model, llm, drafter
     torch.cuda.empty_cache()
-    return result
+    return run
 
 
 def attention_roofline(run):
     """The dominant kernel against the roof that binds it.  Per launch, from the shapes the timed
     region actually ran: algorithmic FLOPs 4 * heads * head_dim * query rows * keys, algorithmic
     bytes K and V once (2 * heads * head_dim * 2 B per key) plus Q and O once, query rows = the
-    tree slots that exist (the padding slots of the (batch, n_q) layout are not run); duration = HIP events
-    around every TIMED_EVERY-th launch of the timed region (the shapes are those of the same launches).  Arithmetic intensity below the machine balance
-    (2500 TFLOP/s / 8 TB/s = 312 FLOP/B) means the HBM roof binds, above it the MFMA roof."""
+    tree slots that exist (the padding slots of the (batch, n_q) layout are not run), keys = the
+    keys between a row's left padding and its last tree slot; duration = HIP events around every
+    TIMED_EVERY-th launch of the timed region (the shapes are those of the same launches).
+    Arithmetic intensity below the machine balance (2500 TFLOP/s / 8 TB/s = 312 FLOP/B) means the
+    HBM roof binds, above it the MFMA roof."""
     H, D = LLAMA_7B["num_attention_heads"], LLAMA_7B["hidden_size"] // LLAMA_7B["num_attention_heads"]
     count, total_ms = run["dominant"].get("attn_mfma_kernel", (0, 0.0))
     launched = len(run["shapes"])
     shapes = run["shapes"][::TIMED_EVERY][:count] if count else []  # the launches that were timed
     if not count or total_ms <= 0:
         return None
-    flops = sum(4.0 * H * D * rows * kv for (B, n_q, kv, rows) in shapes)
-    k_bytes = sum(2.0 * H * D * 2 * B * kv + 2.0 * rows * H * D * 2 for (B, n_q, kv, rows) in shapes)
+    # keys: every row from its first real token to its last tree slot.  Left padding only appears
+    # with forced acceptance (rows grow at different rates); its average over the run is taken as
+    # half of what the last step shows, and the tree slots a row does not have are left out.
+    pads = run.get("final_left_pads", 0) / 2.0
+    keys = [B * (kv - n_q) - pads + rows for (B, n_q, kv, rows) in shapes]
+    flops = sum(4.0 * H * D * (rows / B) * k for (B, n_q, kv, rows), k in zip(shapes, keys))
+    k_bytes = sum(2.0 * H * D * 2 * k + 2.0 * rows * H * D * 2 for (B, n_q, kv, rows), k in zip(shapes, keys))
     seconds = total_ms * 1e-3
     tflops, gbs = flops / seconds / 1e12, k_bytes / seconds / 1e9
     hbm_bound = flops / k_bytes < MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
-    traffic = None
-    path = os.path.join(ROOT, "profiles", "attn_mfma_kernel_traffic.json")
-    if os.path.exists(path):
-        with open(path) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
     out = dict(kernel="attn_mfma_kernel")
     if hbm_bound:
         out.update(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(gbs / HBM_PEAK_GBS, 4))
     else:
         out.update(bound="mfma", achieved=round(tflops, 2), peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
                    frac=round(tflops / MFMA_BF16_PEAK_TFLOPS, 4))
+    # HBM bytes by counters belong to the run they were counted on, not to this one: the figure of
+    # this run is null, and the ratio (counted / algorithmic bytes) of the profiled run is named
+    profiled = None
+    path = os.path.join(ROOT, "profiles", "attn_mfma_kernel_traffic.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            j = json.load(f)
+        profiled = dict(ratio=j.get("ratio"), workload=j.get("workload"))
     out.update(
-        traffic=traffic, launches=count, launches_in_timed_region=launched, timed_every=TIMED_EVERY,
+        traffic=None, traffic_ratio_profiled=profiled,
+        launches=count, launches_in_timed_region=launched, timed_every=TIMED_EVERY,
         avg_us=round(total_ms * 1e3 / count, 2),
         algorithmic_gflop_per_launch=round(flops / count / 1e9, 3),
         algorithmic_mb_per_launch=round(k_bytes / count / 1e6, 2),
@@ -222,6 +281,20 @@ def attention_roofline(run):
         mean_kv_len=round(sum(kv for (_, _, kv, _) in shapes) / len(shapes), 1),
     )
     return out
+
+
+def summary_of(run):
+    """One of the additional operating points: step time, throughput, the attention kernel."""
+    r = attention_roofline(run)
+    return dict(
+        ms_per_step=round(run["elapsed"] / run["steps"] * 1e3, 3), steps=run["steps"],
+        tokens_per_second=round(run["tokens"] / run["elapsed"], 2),
+        tokens_per_step_per_sequence=round(run["per_seq_tokens"], 3),
+        context_tokens=list(run["context"]),
+        attention=None if r is None else {k: r[k] for k in (
+            "avg_us", "bound", "achieved", "unit", "frac", "mfma_frac_of_peak", "algorithmic_mb_per_launch",
+            "mean_n_q", "mean_query_rows", "mean_kv_len", "launches")},
+    )
 
 
 # -------------------------------------------------------------------------------------------------
@@ -240,7 +313,7 @@ def cpu_baseline(per_seq_tokens: float):
     layers = (4, 12) if gflops > 300 else (1, 2)
     log(f"[bench] cpu baseline: {threads} threads, bf16 GEMM {gflops:.0f} GFLOP/s, sample layers {layers}")
     gen = torch.Generator().manual_seed(SEED)
-    times = []
+    medians, samples = [], {}
     for n_layers in layers:
         llm, drafter = build_models("cpu", torch.bfloat16, n_layers, SEED)
         cache = P.Cache(BATCH, PROMPT + NEW_TOKENS + WIDTH * LENGTH, n_layers, 32, 128, torch.bfloat16, "cpu")
@@ -251,23 +324,27 @@ def cpu_baseline(per_seq_tokens: float):
         tok = torch.randint(1, 32000, (BATCH,), generator=gen)
         with torch.inference_mode():
             step_times = []
-            for _ in range(2):  # the first pass pays one-time costs (allocator, kernel selection)
+            for i in range(1 + CPU_STEPS):  # the first pass pays one-time costs (allocator, kernel selection)
                 cache.set_length(PROMPT)
                 t = time.perf_counter()
                 P.greedy_step(llm, drafter, ids, ctx, tok, cache, WIDTH, LENGTH, 0, tie="topk")
-                step_times.append(time.perf_counter() - t)
-            times.append(min(step_times))
-        log(f"[bench] cpu step with {n_layers} layers: {times[-1]:.2f}s")
+                if i > 0:
+                    step_times.append(time.perf_counter() - t)
+        samples[n_layers] = [round(x, 3) for x in step_times]
+        medians.append(sorted(step_times)[len(step_times) // 2])
+        log(f"[bench] cpu steps with {n_layers} layers: {samples[n_layers]} s")
         del llm, drafter, cache
-    per_layer = (times[1] - times[0]) / (layers[1] - layers[0])
-    full = times[0] + (LLAMA_7B["num_hidden_layers"] - layers[0]) * per_layer
+    per_layer = (medians[1] - medians[0]) / (layers[1] - layers[0])
+    full = medians[0] + (LLAMA_7B["num_hidden_layers"] - layers[0]) * per_layer
     return dict(
         value=round(per_seq_tokens * BATCH / full, 3), unit="tokens/s", cores=threads, kind="port",
-        sample=(f"one decode step of the same workload (batch {BATCH}, context {PROMPT}, beam {WIDTH}x{LENGTH}, bf16) "
-                f"through the torch restatement with {layers[0]} and {layers[1]} of 32 layers "
-                f"({times[0]:.2f}s, {times[1]:.2f}s; faster of two passes each), extrapolated linearly to 32 layers = {full:.2f}s/step; "
-                f"tokens per step taken from the GPU run"),
+        sample=(f"decode steps of the same workload (batch {BATCH}, context {PROMPT}, beam {WIDTH}x{LENGTH}, bf16; the "
+                f"cache pre-filled, the prefill not timed) through the torch restatement with {layers[0]} and "
+                f"{layers[1]} of 32 layers: median of {CPU_STEPS} steps each after one warm-up step "
+                f"({medians[0]:.2f}s, {medians[1]:.2f}s), extrapolated linearly in the layer count to 32 layers = "
+                f"{full:.2f}s/step; tokens per step taken from the GPU run"),
         seconds_per_step=round(full, 3),
+        raw_step_seconds={str(k): v for k, v in samples.items()},
     )
 
 
@@ -379,6 +456,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--extra-steps", type=int, default=32,
+                    help="timed steps of each additional operating point (long context, ragged acceptance); 0 skips them")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-kernels", action="store_true",
                     help="only time the CPU restatement of each stage on the micro-benchmark shapes (no GPU needed)")
@@ -396,7 +475,7 @@ def main():
 
     import recurrent_drafting_amd  # noqa: F401  (fails loudly if the HIP library is missing)
 
-    run = gpu_run(args.steps, args.warmup)
+    run = gpu_run(args.steps, args.warmup, args.extra_steps)
     value = run["tokens"] / run["elapsed"]
     line = {
         "metric": "tokens/sec on 1 MI355X, Vicuna-7B-shape bs8 bw45 bl5 bf16; verify-step us",
@@ -421,6 +500,10 @@ def main():
         "stage_seconds_synchronised": {k: round(v, 6) for k, v in run["stage"].items()},
         "reference_style_tokens_per_second_per_sequence": round(run["ref_style_tokens_per_second"], 2),
         "roofline": attention_roofline(run),
+        # the same decode step at other points of its operating range (the headline sits at the start
+        # of the 500 -> 2548 trajectory, and random-init models accept no drafted token)
+        "long_context": {k: summary_of(r) for k, r in run["others"].items() if k.startswith("context_")},
+        "ragged_acceptance": {k: summary_of(r) for k, r in run["others"].items() if k.startswith("ragged_")},
         "kernel_avg_us": {k: round(ms * 1e3 / n, 2) for k, (n, ms) in sorted(run["kernels"].items())},
     }
     line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(run["per_seq_tokens"])
