@@ -346,6 +346,33 @@ RD_API int rd_verify_attention(const void* q, const int64_t* q_strides, const vo
                                float scale, const uint64_t* bits, int32_t* plan,
                                void* workspace, size_t workspace_bytes, int force_generic,
                                const int32_t* row_start, void* stream);
+/* rd_rope_verify_attention: rd_rope_append followed by rd_verify_attention for the new tokens of one
+ * layer, as ONE launch: modeling_llama.py:148-159 (rotation, kv_cache.py:24-32 append) and :161-169
+ * (attention).  The attention kernel rotates its query rows in registers (q itself is left as it
+ * was) and writes the rotated new keys and the new values to their cache rows before it reads them,
+ * so the separate rotation kernel and its pass over q, k and v go away.  Output and cache hold the
+ * same bits as after the two calls.
+ * q (batch, n_heads, n_q, head_dim) through q_strides {batch, head, token}; k_new, v_new
+ * (batch, n_q, n_kv_heads, head_dim) with heads head_dim apart, *_new_strides = {batch, token};
+ * cos, sin, table_rows, position_ids, pos_batch_stride as for rd_rope_append; k_cache / v_cache
+ * with cache_strides {batch, head, row} and max_len rows per slab; kv_len counts the cache rows
+ * AFTER the append (new token t is key column kv_len - n_q + t); bits, plan (built for kv_len, with
+ * the row shifts of the cache if it has any), workspace, row_start as for rd_verify_attention
+ * (with row_start, k_new and v_new are packed like q and a row's missing tokens are not written).
+ * Only bf16, head_dim 128, n_q <= 256, 16-byte aligned operands: rd_rope_verify_attention_eligible
+ * says whether a shape qualifies, and a call that does not fails with RD_ELIMIT and enqueues
+ * nothing (use the two calls then). */
+RD_API int rd_rope_verify_attention_eligible(int dtype, int n_heads, int head_dim, int n_q);
+RD_API int rd_rope_verify_attention(const void* q, const int64_t* q_strides, const void* k_new,
+                                    const int64_t* k_new_strides, const void* v_new,
+                                    const int64_t* v_new_strides, const void* cos, const void* sin,
+                                    int64_t table_rows, const int64_t* position_ids,
+                                    int64_t pos_batch_stride, void* k_cache, void* v_cache,
+                                    const int64_t* cache_strides, int64_t max_len, void* out,
+                                    const int64_t* o_strides, int dtype, int batch, int n_heads,
+                                    int n_kv_heads, int n_q, int kv_len, int head_dim, float scale,
+                                    const uint64_t* bits, int32_t* plan, void* workspace,
+                                    size_t workspace_bytes, const int32_t* row_start, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Causal mask from a padding mask: mask[b,i,j] = (j <= kv_len - query_len + i) && padding[b,j].

@@ -54,17 +54,41 @@ struct AttnArgs {
   int32_t* counters;  // arrival counters of the plan: [batch][kAttnMaxHeads][query tiles], zero between launches
   int B, H, Hkv, n_q, kv_len, words, max_splits, D;
   float scale;  // softmax scale; the MFMA kernel works in log2 units (scale * log2 e)
+  // Rotary embedding and cache append fused in (the ROPE instantiation of the MFMA kernel): q arrives
+  // unrotated; k_new / v_new (token rows like q's, heads D apart, strides {batch, token}) are the new
+  // keys and values, whose rotated / copied rows belong at key columns [new_col0, new_col0 + n_q) of
+  // k and v; cos / sin (table_rows, D) and position_ids (batch, n_q) as for rd_rope_append.
+  const void* k_new; int64_t kn_sb, kn_st;
+  const void* v_new; int64_t vn_sb, vn_st;
+  const void* cos; const void* sin; int64_t table_rows;
+  const int64_t* position_ids; int64_t pos_sb;
+  int new_col0;       // kv_len - n_q
+  int64_t max_len;    // cache rows of a slab: a new row that a shift would put outside is dropped
 };
 
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Query rows of batch row b: their count and the element offsets of row 0 in q and out.
-struct RowSpan { int n; int64_t q_off, o_off; };
+struct RowSpan { int n; int64_t q_off, o_off; int r0; };  // r0: first packed row, or -1 (padded layout)
 __device__ inline RowSpan row_span(const AttnArgs& a, int b) {
-  if (a.row_start == nullptr) return {a.n_q, (int64_t)b * a.q_sb, (int64_t)b * a.o_sb};
+  if (a.row_start == nullptr) return {a.n_q, (int64_t)b * a.q_sb, (int64_t)b * a.o_sb, -1};
   const int r0 = a.row_start[b], r1 = a.row_start[b + 1];
   const int n = r1 - r0;
-  return {n < a.n_q ? n : a.n_q, (int64_t)r0 * a.q_ss, (int64_t)r0 * a.o_ss};
+  return {n < a.n_q ? n : a.n_q, (int64_t)r0 * a.q_ss, (int64_t)r0 * a.o_ss, r0};
+}
+
+// round to bf16 and back; products and sums of the rotation are rounded one by one, as the separate
+// elementwise kernels of the reference's op chain round them (no fused multiply-add)
+__device__ inline float bf16_round(float v) { return static_cast<float>(static_cast<__bf16>(v)); }
+__device__ inline float rope_lo(float x1, float x2, float c, float s) {
+#pragma clang fp contract(off)
+  const float p = bf16_round(x1 * c), q = bf16_round(x2 * s);
+  return p - q;
+}
+__device__ inline float rope_hi(float x1, float x2, float c, float s) {
+#pragma clang fp contract(off)
+  const float p = bf16_round(x2 * c), q = bf16_round(x1 * s);
+  return p + q;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -131,7 +155,7 @@ __device__ inline float pair_sum(float v) {
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
-template <int LAYOUT>
+template <int LAYOUT, bool ROPE>
 __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   constexpr int kRowsPerWG = rows_per_wg(LAYOUT);
   constexpr bool kHasFull = LAYOUT != kSplit, kHasHalf = LAYOUT != kFull;
@@ -176,17 +200,155 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const __bf16* kbase = reinterpret_cast<const __bf16*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh - (int64_t)kv_shift * a.k_ss;
   const __bf16* vbase = reinterpret_cast<const __bf16*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh - (int64_t)kv_shift * a.v_ss;
 
+  // ---- new cache rows and rotated queries (ROPE) ---------------------------------------------------
+  // The new keys and values of this (batch row, kv head) go to their cache rows before anybody's
+  // tile loads ask for them: the keys rotated by their positions, the values as they are -- what a
+  // separate kernel did between the projection and this one (a launch, and a pass over q, k and v).
+  // A workgroup writes the rows that its own tile loop may read (its item's share of the key
+  // columns [new_col0, new_col0 + rows.n)); workgroups that share them (grouped heads) write the
+  // same bytes.  Nobody else reads them in this launch.  The item that ends the row's key span
+  // also writes what lies behind the span, so that rows nobody attends to reach the cache too.
+  // A round covers 128 tokens: 1024 rotation tasks (a 16-byte chunk of the first half of a key and
+  // its partner in the second half), two per thread, and 2048 copy tasks, four per thread.
+  //
+  // Order.  Loads return in the order of their issue, and the tile loads of the prologue keep the
+  // memory system busy for microseconds: whatever this code reads is therefore requested BEFORE
+  // the first tile (`issue`: positions, then the table rows and the new keys and values), and used
+  // (`finish`) after the last tile load of the prologue has been issued.  The stores are not waited
+  // for there either: the first tile that holds new rows is requested many steps into the loop,
+  // and the step before that request waits for them (t_sync), ahead of its barrier.
+  const bool writes = ROPE && (hi > a.new_col0 || hi >= key_end);  // (uniform over the workgroup)
+  const int t_lo = lo > a.new_col0 ? lo - a.new_col0 : 0;
+  const int t_hi = !writes ? 0 : (hi >= key_end || hi - a.new_col0 > rows.n ? rows.n : hi - a.new_col0);
+  const bool has_new = t_lo < t_hi;
+  // K tile j is requested in step j - 2 - kRing (the prologue for j < 2 + kRing), V tiles later
+  const int first_new_tile = a.new_col0 > lo ? (a.new_col0 - lo) / kTile : 0;
+  const int t_sync = has_new ? first_new_tile - 3 - kRing : -1;  // the step whose barrier the rows need
+  const bool early = has_new && t_sync < 0;  // the prologue's own tiles hold new rows: write first
+  struct NewRows {
+    int64_t pos[2]; bf16x8 x1[2], x2[2], vv[4], c1[2], c2[2], s1[2], s2[2];
+    int kt[2], kc[2], vt[4], vc[4];  // token and chunk of every task; token -1: no task
+  } nr;
+  const __bf16* kn = nullptr; const __bf16* vn = nullptr;
+  if constexpr (ROPE) {
+    const int64_t new_off = rows.r0 >= 0 ? (int64_t)rows.r0 * a.kn_st : (int64_t)b * a.kn_sb;
+    const int64_t newv_off = rows.r0 >= 0 ? (int64_t)rows.r0 * a.vn_st : (int64_t)b * a.vn_sb;
+    kn = reinterpret_cast<const __bf16*>(a.k_new) + new_off + (int64_t)hk * kD;
+    vn = reinterpret_cast<const __bf16*>(a.v_new) + newv_off + (int64_t)hk * kD;
+  }
+  auto table_row = [&](const void* table, int64_t pos) __attribute__((always_inline)) {
+    pos = pos < 0 ? 0 : (pos >= a.table_rows ? a.table_rows - 1 : pos);  // never read outside the table
+    return reinterpret_cast<const __bf16*>(table) + pos * kD;
+  };
+  auto new_rows_issue = [&](int round) __attribute__((always_inline)) {
+    // every load reads a token that exists (the round's first one stands in where a thread has no
+    // task): the loads are then unconditional and the compiler keeps them together
+    const int t0 = t_lo + 128 * round;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int task = tid + kMfmaThreads * i, t = t0 + (task >> 3);
+      const int64_t cache_row = (int64_t)a.new_col0 + t - kv_shift;
+      // (a shift that leaves the slab is not followed: the row is dropped)
+      const bool on = t < t_hi && cache_row >= 0 && cache_row < a.max_len;
+      nr.kt[i] = on ? t : -1;
+      nr.kc[i] = task & 7;
+      const int tl = on ? t : t0;
+      nr.pos[i] = a.position_ids[(int64_t)b * a.pos_sb + tl];
+      nr.x1[i] = *reinterpret_cast<const bf16x8*>(kn + (int64_t)tl * a.kn_st + 8 * nr.kc[i]);
+      nr.x2[i] = *reinterpret_cast<const bf16x8*>(kn + (int64_t)tl * a.kn_st + kD / 2 + 8 * nr.kc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int task = tid + kMfmaThreads * i, t = t0 + (task >> 4);
+      const int64_t cache_row = (int64_t)a.new_col0 + t - kv_shift;
+      const bool on = t < t_hi && cache_row >= 0 && cache_row < a.max_len;
+      nr.vt[i] = on ? t : -1;
+      nr.vc[i] = task & 15;
+      nr.vv[i] = *reinterpret_cast<const bf16x8*>(vn + (int64_t)(on ? t : t0) * a.vn_st + 8 * nr.vc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const __bf16* cos_row = table_row(a.cos, nr.pos[i]) + 8 * nr.kc[i];
+      const __bf16* sin_row = table_row(a.sin, nr.pos[i]) + 8 * nr.kc[i];
+      nr.c1[i] = *reinterpret_cast<const bf16x8*>(cos_row); nr.c2[i] = *reinterpret_cast<const bf16x8*>(cos_row + kD / 2);
+      nr.s1[i] = *reinterpret_cast<const bf16x8*>(sin_row); nr.s2[i] = *reinterpret_cast<const bf16x8*>(sin_row + kD / 2);
+    }
+  };
+  auto new_rows_finish = [&]() __attribute__((always_inline)) {
+    __bf16* kw = const_cast<__bf16*>(kbase);
+    __bf16* vw = const_cast<__bf16*>(vbase);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (nr.vt[i] >= 0)
+        *reinterpret_cast<bf16x8*>(vw + ((int64_t)a.new_col0 + nr.vt[i]) * a.v_ss + 8 * nr.vc[i]) = nr.vv[i];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      bf16x8 o1, o2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        o1[e] = static_cast<__bf16>(rope_lo((float)nr.x1[i][e], (float)nr.x2[i][e], (float)nr.c1[i][e], (float)nr.s1[i][e]));
+        o2[e] = static_cast<__bf16>(rope_hi((float)nr.x1[i][e], (float)nr.x2[i][e], (float)nr.c2[i][e], (float)nr.s2[i][e]));
+      }
+      if (nr.kt[i] >= 0) {
+        __bf16* dst = kw + ((int64_t)a.new_col0 + nr.kt[i]) * a.k_ss + 8 * nr.kc[i];
+        *reinterpret_cast<bf16x8*>(dst) = o1;
+        *reinterpret_cast<bf16x8*>(dst + kD / 2) = o2;
+      }
+    }
+  };
+  // the rest of the work after the first round's loads: its second half and further rounds (more
+  // than 128 tokens, rare); the rows are in memory after new_rows_wait
+  auto new_rows_complete = [&]() __attribute__((always_inline)) {
+    new_rows_finish();
+    for (int round = 1; t_lo + 128 * round < t_hi; ++round) {
+      new_rows_issue(round);
+      new_rows_finish();
+    }
+  };
+  auto new_rows_wait = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+
   // Q fragments: B operand of S^T = K Q^T; lane (r,g) holds Q[q_row][16*ks + 8*g .. +8)
   bf16x8 qf[8];
+  // (ROPE) the table rows of the query's position: the lane holds dims 16*ks + 8*g + e, so the
+  // partner of a first-half dim (ks < 4) sits in fragment ks + 4 of the same lane
+  bf16x8 qc[8], qs[8];
   {
     const __bf16* qp = reinterpret_cast<const __bf16*>(a.q) + rows.q_off + (int64_t)h * a.q_sh +
                        (int64_t)(row_valid ? q_row : 0) * a.q_ss + 8 * g;
+    int64_t q_pos = 0;
+    if constexpr (ROPE) q_pos = a.position_ids[(int64_t)b * a.pos_sb + (row_valid ? q_row : 0)];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
       qf[ks] = row_valid ? *reinterpret_cast<const bf16x8*>(qp + 16 * ks) : z;
     }
+    if constexpr (ROPE) {
+      if (has_new) new_rows_issue(0);
+      const __bf16* cos_row = table_row(a.cos, q_pos) + 8 * g;
+      const __bf16* sin_row = table_row(a.sin, q_pos) + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        qc[ks] = *reinterpret_cast<const bf16x8*>(cos_row + 16 * ks);
+        qs[ks] = *reinterpret_cast<const bf16x8*>(sin_row + 16 * ks);
+      }
+      if (early) {
+        new_rows_complete();
+        new_rows_wait();
+        __syncthreads();
+      }
+    }
   }
+  auto rotate_q = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const bf16x8 x1 = qf[ks], x2 = qf[ks + 4];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        qf[ks][e] = static_cast<__bf16>(rope_lo((float)x1[e], (float)x2[e], (float)qc[ks][e], (float)qs[ks][e]));
+        qf[ks + 4][e] = static_cast<__bf16>(rope_hi((float)x1[e], (float)x2[e], (float)qc[ks + 4][e], (float)qs[ks + 4][e]));
+      }
+    }
+  };
   const uint64_t* brow = a.bits + ((int64_t)b * a.n_q + (row_valid ? q_row : 0)) * a.words;
 
   f32x16 o[4];
@@ -296,14 +458,29 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // the tile that step t stages in ring slot (t + 1) % kRing, so that one piece of code, with
   // the same registers, serves both.
   const int ahead = k_loader ? 2 : 1;
-  if (k_loader) {
-    fetch_tile(S0{}, 0);
-    fetch_tile(S1{}, 1);
-    stage_k(S0{}, 0);
-    stage_k(S1{}, 1);
+  if constexpr (!ROPE) {
+    if (k_loader) {
+      fetch_tile(S0{}, 0);
+      fetch_tile(S1{}, 1);
+      stage_k(S0{}, 0);
+      stage_k(S1{}, 1);
+    } else {
+      fetch_tile(S0{}, 0);
+      stage_v(S0{}, 0);
+    }
   } else {
+    // the first tiles are requested, and while they are on their way the vector ALU rotates the
+    // queries and the new keys (whose operands were requested before the tiles and arrive first)
     fetch_tile(S0{}, 0);
-    stage_v(S0{}, 0);
+    if (k_loader) fetch_tile(S1{}, 1);
+    if (has_new && !early) new_rows_complete();
+    rotate_q();
+    if (k_loader) {
+      stage_k(S0{}, 0);
+      stage_k(S1{}, 1);
+    } else {
+      stage_v(S0{}, 0);
+    }
   }
   // The ring is filled in the order in which the steps refill it (tile, then mask word, slot by
   // slot): the loads in flight at the top of the first step are then the same as at the top of
@@ -436,6 +613,9 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     if (kLast) {
       // this tile's mask word is done with: the word of tile t+kRing takes its slot
       fetch_word(std::integral_constant<int, J>{}, t + kRing);
+      if constexpr (ROPE) {
+        if (t == t_sync) new_rows_wait();  // (uniform) the next step may request a tile with new rows
+      }
       __syncthreads();
     }
   };
@@ -712,24 +892,33 @@ extern "C" size_t rd_attention_workspace_bytes(int batch, int n_heads, int n_q, 
          rd::align_up(slots * n_q * 2 * sizeof(float), 256);
 }
 
-extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, const void* k,
-                                   const int64_t* k_strides, const void* v,
-                                   const int64_t* v_strides, void* out, const int64_t* o_strides,
-                                   int dtype, int batch, int n_heads, int n_kv_heads, int n_q,
-                                   int kv_len, int head_dim, float scale, const uint64_t* bits,
-                                   int32_t* plan, void* workspace, size_t workspace_bytes,
-                                   int force_generic, const int32_t* row_start, void* stream) {
+namespace {
+
+// The new keys and values of a fused call (null: the cache already holds them).
+struct RopeInputs {
+  const void* k_new; const int64_t* k_new_strides;
+  const void* v_new; const int64_t* v_new_strides;
+  const void* cos; const void* sin; int64_t table_rows;
+  const int64_t* position_ids; int64_t pos_batch_stride;
+  int64_t max_len;
+};
+
+int verify_attention(const char* who, const void* q, const int64_t* q_strides, const void* k,
+                     const int64_t* k_strides, const void* v, const int64_t* v_strides, void* out,
+                     const int64_t* o_strides, int dtype, int batch, int n_heads, int n_kv_heads, int n_q,
+                     int kv_len, int head_dim, float scale, const uint64_t* bits, int32_t* plan,
+                     void* workspace, size_t workspace_bytes, int force_generic, const int32_t* row_start,
+                     const RopeInputs* rope, void* stream) {
   RD_REQUIRE(batch > 0 && n_heads > 0 && n_kv_heads > 0 && n_q > 0 && kv_len > 0 && head_dim > 0,
-             RD_EINVAL, "rd_verify_attention: bad sizes (batch %d heads %d kv_heads %d n_q %d kv %d D %d)",
+             RD_EINVAL, "%s: bad sizes (batch %d heads %d kv_heads %d n_q %d kv %d D %d)", who,
              batch, n_heads, n_kv_heads, n_q, kv_len, head_dim);
-  RD_REQUIRE(n_heads % n_kv_heads == 0, RD_EINVAL, "rd_verify_attention: heads %d not a multiple of kv heads %d",
+  RD_REQUIRE(n_heads % n_kv_heads == 0, RD_EINVAL, "%s: heads %d not a multiple of kv heads %d", who,
              n_heads, n_kv_heads);
-  RD_REQUIRE(head_dim <= 256, RD_ELIMIT, "rd_verify_attention: head_dim %d > 256", head_dim);
-  RD_REQUIRE(batch <= 65535 && n_heads <= 65535, RD_ELIMIT, "rd_verify_attention: batch/heads > 65535");
+  RD_REQUIRE(head_dim <= 256, RD_ELIMIT, "%s: head_dim %d > 256", who, head_dim);
+  RD_REQUIRE(batch <= 65535 && n_heads <= 65535, RD_ELIMIT, "%s: batch/heads > 65535", who);
   RD_REQUIRE(q && k && v && out && bits && plan && q_strides && k_strides && v_strides && o_strides,
-             RD_EINVAL, "rd_verify_attention: null pointer");
-  RD_REQUIRE(dtype == RD_BF16 || dtype == RD_F16 || dtype == RD_F32, RD_EINVAL,
-             "rd_verify_attention: unknown dtype %d", dtype);
+             RD_EINVAL, "%s: null pointer", who);
+  RD_REQUIRE(dtype == RD_BF16 || dtype == RD_F16 || dtype == RD_F32, RD_EINVAL, "%s: unknown dtype %d", who, dtype);
   AttnArgs a;
   a.q = q; a.q_sb = q_strides[0]; a.q_sh = q_strides[1]; a.q_ss = q_strides[2];
   a.k = k; a.k_sb = k_strides[0]; a.k_sh = k_strides[1]; a.k_ss = k_strides[2];
@@ -742,13 +931,40 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
   a.part_o = nullptr; a.part_ml = nullptr;
   a.row_start = row_start;
   a.counters = plan + rd::attn_counter_offset(batch, n_q, kv_len);
+  a.k_new = a.v_new = a.cos = a.sin = nullptr;
+  a.kn_sb = a.kn_st = a.vn_sb = a.vn_st = a.table_rows = a.pos_sb = a.max_len = 0;
+  a.position_ids = nullptr; a.new_col0 = kv_len;
   hipStream_t s = rd::as_stream(stream);
 
-  if (!force_generic && mfma_eligible(a, dtype)) {
+  const bool mfma = !force_generic && mfma_eligible(a, dtype);
+  if (rope != nullptr) {
+    auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    RD_REQUIRE(mfma && n_q <= rows_per_wg(kFull), RD_ELIMIT, "%s: only bf16, head_dim %d, n_q <= %d, 16-byte aligned "
+               "operands (use rd_rope_append and rd_verify_attention)", who, kD, rows_per_wg(kFull));
+    RD_REQUIRE(rope->k_new && rope->v_new && rope->cos && rope->sin && rope->position_ids && rope->k_new_strides &&
+                   rope->v_new_strides, RD_EINVAL, "%s: null pointer", who);
+    RD_REQUIRE(al(rope->k_new) && al(rope->v_new) && al(rope->cos) && al(rope->sin), RD_EINVAL,
+               "%s: pointers must be 16-byte aligned", who);
+    RD_REQUIRE(rope->table_rows > 0, RD_EINVAL, "%s: empty cos/sin table", who);
+    RD_REQUIRE(kv_len >= n_q && kv_len <= rope->max_len, RD_EINVAL, "%s: kv_len %d must lie in [n_q %d, max_len %lld]",
+               who, kv_len, n_q, (long long)rope->max_len);
+    for (const int64_t* st : {rope->k_new_strides, rope->v_new_strides})
+      RD_REQUIRE(st[0] % 8 == 0 && st[1] % 8 == 0 && st[0] >= 0 && st[1] >= (int64_t)n_kv_heads * kD, RD_EINVAL,
+                 "%s: token and batch strides of the new keys and values must be multiples of 8 elements, "
+                 "tokens at least kv_heads * head_dim apart", who);
+    a.k_new = rope->k_new; a.kn_sb = rope->k_new_strides[0]; a.kn_st = rope->k_new_strides[1];
+    a.v_new = rope->v_new; a.vn_sb = rope->v_new_strides[0]; a.vn_st = rope->v_new_strides[1];
+    a.cos = rope->cos; a.sin = rope->sin; a.table_rows = rope->table_rows;
+    a.position_ids = rope->position_ids; a.pos_sb = rope->pos_batch_stride;
+    a.new_col0 = kv_len - n_q;
+    a.max_len = rope->max_len;
+  }
+
+  if (mfma) {
     const size_t need = rd_attention_workspace_bytes(batch, n_heads, n_q, kv_len, head_dim);
-    RD_REQUIRE(workspace && workspace_bytes >= need, RD_EWORKSPACE,
-               "rd_verify_attention: workspace %zu < %zu bytes", workspace_bytes, need);
-    RD_REQUIRE(((uintptr_t)workspace & 255) == 0, RD_EINVAL, "rd_verify_attention: workspace not 256B aligned");
+    RD_REQUIRE(workspace && workspace_bytes >= need, RD_EWORKSPACE, "%s: workspace %zu < %zu bytes", who,
+               workspace_bytes, need);
+    RD_REQUIRE(((uintptr_t)workspace & 255) == 0, RD_EINVAL, "%s: workspace not 256B aligned", who);
     const size_t slots = (size_t)batch * n_heads * a.max_splits;
     a.part_o = reinterpret_cast<float*>(workspace);
     a.part_ml = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
@@ -756,21 +972,25 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
     const int max_items = batch * a.max_splits;
     const int layout = layout_for(n_q);
     const int q_tiles = (n_q + rows_per_wg(layout) - 1) / rows_per_wg(layout);
-    RD_REQUIRE(max_items <= 65535 && (int64_t)q_tiles * n_heads <= 2147483647LL, RD_ELIMIT,
-               "rd_verify_attention: grid too large");
+    RD_REQUIRE(max_items <= 65535 && (int64_t)q_tiles * n_heads <= 2147483647LL, RD_ELIMIT, "%s: grid too large", who);
     {
       // when timed, the events carry the kernel's own begin and end (what a kernel trace reports)
       hipEvent_t t0, t1;
       rd::timing_events("attn_mfma_kernel", &t0, &t1);
       const dim3 grid(n_heads * q_tiles, max_items), block(kMfmaThreads);
+      auto launch = [&](auto layout_c) {
+        constexpr int L = decltype(layout_c)::value;
+        if (rope) hipExtLaunchKernelGGL((attn_mfma_kernel<L, true>), grid, block, 0, s, t0, t1, 0, a);
+        else hipExtLaunchKernelGGL((attn_mfma_kernel<L, false>), grid, block, 0, s, t0, t1, 0, a);
+      };
       switch (layout) {
-        case kSplit: hipExtLaunchKernelGGL(attn_mfma_kernel<kSplit>, grid, block, 0, s, t0, t1, 0, a); break;
-        case kMix5: hipExtLaunchKernelGGL(attn_mfma_kernel<kMix5>, grid, block, 0, s, t0, t1, 0, a); break;
-        case kMix6: hipExtLaunchKernelGGL(attn_mfma_kernel<kMix6>, grid, block, 0, s, t0, t1, 0, a); break;
-        default: hipExtLaunchKernelGGL(attn_mfma_kernel<kFull>, grid, block, 0, s, t0, t1, 0, a); break;
+        case kSplit: launch(std::integral_constant<int, kSplit>{}); break;
+        case kMix5: launch(std::integral_constant<int, kMix5>{}); break;
+        case kMix6: launch(std::integral_constant<int, kMix6>{}); break;
+        default: launch(std::integral_constant<int, kFull>{}); break;
       }
     }
-    return rd::check_launch("rd_verify_attention(mfma)");
+    return rd::check_launch(who);
   }
   const dim3 grid(n_q, n_heads, batch);
   switch (dtype) {
@@ -778,5 +998,40 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
     case RD_F16: { rd::ScopedTiming rd_t("attn_generic_kernel", s); hipLaunchKernelGGL(attn_generic_kernel<__half>, grid, dim3(kGenThreads), 0, s, a); } break;
     default: { rd::ScopedTiming rd_t("attn_generic_kernel", s); hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(kGenThreads), 0, s, a); } break;
   }
-  return rd::check_launch("rd_verify_attention(generic)");
+  return rd::check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, const void* k,
+                                   const int64_t* k_strides, const void* v,
+                                   const int64_t* v_strides, void* out, const int64_t* o_strides,
+                                   int dtype, int batch, int n_heads, int n_kv_heads, int n_q,
+                                   int kv_len, int head_dim, float scale, const uint64_t* bits,
+                                   int32_t* plan, void* workspace, size_t workspace_bytes,
+                                   int force_generic, const int32_t* row_start, void* stream) {
+  return verify_attention("rd_verify_attention", q, q_strides, k, k_strides, v, v_strides, out, o_strides, dtype,
+                          batch, n_heads, n_kv_heads, n_q, kv_len, head_dim, scale, bits, plan, workspace,
+                          workspace_bytes, force_generic, row_start, nullptr, stream);
+}
+
+extern "C" int rd_rope_verify_attention_eligible(int dtype, int n_heads, int head_dim, int n_q) {
+  return dtype == RD_BF16 && head_dim == kD && n_heads <= rd::kAttnMaxHeads && n_q > 0 && n_q <= rows_per_wg(kFull);
+}
+
+extern "C" int rd_rope_verify_attention(const void* q, const int64_t* q_strides, const void* k_new,
+                                        const int64_t* k_new_strides, const void* v_new,
+                                        const int64_t* v_new_strides, const void* cos, const void* sin,
+                                        int64_t table_rows, const int64_t* position_ids,
+                                        int64_t pos_batch_stride, void* k_cache, void* v_cache,
+                                        const int64_t* cache_strides, int64_t max_len, void* out,
+                                        const int64_t* o_strides, int dtype, int batch, int n_heads,
+                                        int n_kv_heads, int n_q, int kv_len, int head_dim, float scale,
+                                        const uint64_t* bits, int32_t* plan, void* workspace,
+                                        size_t workspace_bytes, const int32_t* row_start, void* stream) {
+  const RopeInputs rope{k_new, k_new_strides, v_new, v_new_strides, cos, sin, table_rows, position_ids,
+                        pos_batch_stride, max_len};
+  return verify_attention("rd_rope_verify_attention", q, q_strides, k_cache, cache_strides, v_cache, cache_strides,
+                          out, o_strides, dtype, batch, n_heads, n_kv_heads, n_q, kv_len, head_dim, scale, bits,
+                          plan, workspace, workspace_bytes, 0, row_start, &rope, stream);
 }

@@ -60,6 +60,12 @@ _PROTOTYPES = {
         _I,
         [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P, _Z, _I, _P, _P],
     ),
+    "rd_rope_verify_attention_eligible": (_I, [_I, _I, _I, _I]),
+    "rd_rope_verify_attention": (
+        _I,
+        [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F,
+         _P, _P, _P, _Z, _P, _P],
+    ),
     "rd_causal_mask": (_I, [_P, _I, _L, _I, _L, _L, _P, _P]),
     "rd_verify_row_stats": (_I, [_P, _I, _L, _L, _I, _I, _F, _F, _P, _I, _P]),
     "rd_accept_sample": (

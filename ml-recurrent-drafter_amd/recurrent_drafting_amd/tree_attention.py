@@ -173,7 +173,7 @@ def prepare_attention(tree: PackedTree, padding_mask: torch.Tensor, pad_value: i
             _hip.stream(),
         )
     )
-    return attention.PreparedMask(bits.view(B, n, -1), plan, B, n, kv_len), position_ids, left_pads
+    return attention.PreparedMask(bits.view(B, n, -1), plan, B, n, kv_len, shifted=kv_shift is not None), position_ids, left_pads
 
 
 def pack(

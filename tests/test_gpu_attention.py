@@ -322,3 +322,104 @@ def test_argument_errors():
     k = torch.zeros(1, 3, 5, 16, device="cuda")
     with pytest.raises(RuntimeError, match="multiple"):
         attention.masked_attention(q, k, k, prep)
+
+
+def _fused_case(B, H, Hkv, n_new, prev_lens, seed, shifted, packed, max_len=None):
+    """One layer's new tokens through kv_cache.rope_append + attention.masked_attention and through
+    attention.rope_attention(fused=True), on two caches with the same contents."""
+    import recurrent_drafting_amd as rd
+    from recurrent_drafting_amd import attention, kv_cache
+    from recurrent_drafting_amd.packed_rows import PackedRows
+
+    D = 128
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(seed)
+    prev = max(prev_lens)
+    max_len = max_len or prev + n_new + 7
+    kv_len = prev + n_new
+    caches = []
+    filler = torch.randn((1, 2, B, Hkv, max_len, D), generator=g).to(torch.bfloat16)
+    shift = torch.tensor([prev - p if shifted else 0 for p in prev_lens], dtype=torch.int32)
+    for _ in range(2):
+        c = kv_cache.Cache(B, max_len, 1, Hkv, D, torch.bfloat16, dev)
+        c._cache.copy_(filler.to(dev))
+        c.rows_in_place = shifted
+        c.shift.copy_(shift.to(dev))
+        for view in c.sliced[0]:
+            view.length = prev
+        caches.append(c)
+    # columns [prev - len_b, prev) hold row b's context (left-padded); with shifts they live at the
+    # front of the slab.  The new tokens see their context and a random lower-triangular tree.
+    mask = torch.zeros((B, n_new, kv_len), dtype=torch.bool)
+    tree = torch.rand((B, n_new, n_new), generator=g) < 0.4
+    tree = torch.tril(tree) | torch.eye(n_new, dtype=torch.bool)
+    counts = torch.randint(max(1, n_new // 2), n_new + 1, (B,), generator=g) if packed else torch.full((B,), n_new)
+    counts[0] = n_new
+    for b in range(B):
+        mask[b, :, prev - prev_lens[b]:prev] = True
+        mask[b, :, prev:] = tree[b]
+        mask[b, :, prev + int(counts[b]):] = False
+    mask = mask.to(dev)
+    nq, nk = H * D, Hkv * D
+    rows = None
+    if packed:
+        total = int(counts.sum())
+        rows = PackedRows.from_counts(counts.to(dev), total, n_new)
+        qkv = torch.randn((rows.rows, nq + 2 * nk), generator=g).to(torch.bfloat16).to(dev)
+    else:
+        qkv = torch.randn((B, n_new, nq + 2 * nk), generator=g).to(torch.bfloat16).to(dev)
+    position_ids = (torch.tensor(prev_lens).view(B, 1) + torch.randint(0, 5, (B, n_new), generator=g)).to(dev)
+    table = torch.randn((max(prev_lens) + 8, 2, D), generator=g).to(torch.bfloat16).to(dev)
+    cos, sin = table[:, 0].contiguous(), table[:, 1].contiguous()
+    outs = []
+    for c, fused in zip(caches, (False, True)):
+        x = qkv.clone()
+        q, k, v = x[..., :nq], x[..., nq:nq + nk], x[..., nq + nk:]
+        prepared = attention.prepare(mask, n_heads=H, kv_shift=c.shift if shifted else None)
+        outs.append(attention.rope_attention(q, k, v, cos, sin, position_ids, c.sliced[0], prepared,
+                                             rows=rows, fused=fused))
+        assert c.sliced[0][0].length == kv_len and c.sliced[0][1].length == kv_len
+    torch.cuda.synchronize()
+    live = outs[0].shape[0] if rows is None else rows.total
+    return outs[0][:live], outs[1][:live], caches[0]._cache, caches[1]._cache
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,H,Hkv,n_new,prev_lens,shifted,packed", [
+    (2, 4, 4, 23, [200, 131], False, False),
+    (3, 4, 2, 37, [300, 17, 150], True, False),
+    (3, 8, 2, 40, [1, 64, 129], True, True),
+    (2, 4, 4, 130, [500, 420], True, True),       # five row blocks
+    (2, 2, 2, 256, [90, 64], False, False),       # the largest fused query count
+    (4, 32, 32, 26, [2500, 300, 1800, 64], True, True),  # rows cut into several items
+])
+def test_rope_attention_one_kernel_equals_two(B, H, Hkv, n_new, prev_lens, shifted, packed):
+    two, one, cache_two, cache_one = _fused_case(B, H, Hkv, n_new, prev_lens, 11, shifted, packed)
+    assert torch.equal(one.view(torch.int16), two.view(torch.int16))
+    assert torch.equal(cache_one.view(torch.int16), cache_two.view(torch.int16))
+
+
+@pytest.mark.gpu
+def test_rope_attention_on_a_slab_that_ends_behind_the_new_tokens():
+    two, one, cache_two, cache_one = _fused_case(2, 4, 4, 20, [100, 40], 5, True, False, max_len=120)
+    assert torch.equal(one.view(torch.int16), two.view(torch.int16))
+    assert torch.equal(cache_one.view(torch.int16), cache_two.view(torch.int16))
+
+
+@pytest.mark.gpu
+def test_rope_attention_refuses_what_the_fused_kernel_does_not_cover():
+    import ctypes as C
+    from recurrent_drafting_amd import _hip
+    lib = _hip.lib()
+    assert lib.rd_rope_verify_attention_eligible(_hip.dtype_code(torch.bfloat16), 32, 128, 26) == 1
+    assert lib.rd_rope_verify_attention_eligible(_hip.dtype_code(torch.bfloat16), 32, 128, 257) == 0
+    assert lib.rd_rope_verify_attention_eligible(_hip.dtype_code(torch.bfloat16), 32, 64, 26) == 0
+    assert lib.rd_rope_verify_attention_eligible(_hip.dtype_code(torch.float16), 32, 128, 26) == 0
+    t = torch.zeros(4096, dtype=torch.bfloat16, device="cuda")
+    s3, s2 = (C.c_int64 * 3)(0, 64, 64), (C.c_int64 * 2)(0, 64)
+    rc = lib.rd_rope_verify_attention(
+        _hip.ptr(t), s3, _hip.ptr(t), s2, _hip.ptr(t), s2, _hip.ptr(t), _hip.ptr(t), 4,
+        _hip.ptr(torch.zeros(4, dtype=torch.long, device="cuda")), 1, _hip.ptr(t), _hip.ptr(t), s3, 8,
+        _hip.ptr(t), s3, _hip.dtype_code(torch.bfloat16), 1, 1, 1, 1, 8, 64, 1.0,
+        _hip.ptr(t), _hip.ptr(t.view(torch.int32)), None, 0, None, None)
+    assert rc == -2 and b"rd_rope_verify_attention" in lib.rd_last_error()

@@ -80,7 +80,11 @@ def test_bf16_mfma_decode_loop_teacher_forced_with_accepted_drafts():
     assert sum(r.beams_equal for r in reports) >= len(reports) - 1
 
 
-def test_bf16_mfma_decode_loop_teacher_forced_random_weights_forced_acceptance():
+@pytest.mark.parametrize("one_kernel", [False, True])
+def test_bf16_mfma_decode_loop_teacher_forced_random_weights_forced_acceptance(one_kernel, monkeypatch):
+    # one_kernel: rotation, cache append and attention of a layer as one launch (rd_rope_verify_attention)
+    from recurrent_drafting_amd import modeling_llama
+    monkeypatch.setattr(modeling_llama.LlamaAttention, "fused_rope_attention", None if one_kernel else False)
     llama_sd = tm.draw(tm.llama_shapes(CFG), 51)
     drafter_sd = tm.draw(tm.drafter_shapes(DCFG), 52)
     llm, drafter = _models(llama_sd, drafter_sd, CFG, DCFG)
@@ -90,6 +94,7 @@ def test_bf16_mfma_decode_loop_teacher_forced_random_weights_forced_acceptance()
                                    force=teacher_forced.forced_acceptance(9)))
     print(_summary(reports))
     assert "attn_mfma_kernel" in kernels and "attn_generic_kernel" not in kernels
+    assert ("rope_append_kernel" in kernels) == (not one_kernel), sorted(kernels)
     assert len(reports) == 10
     assert any(any(x != 0 for x in r.shifts) for r in reports)
     assert any(any(x < 0 for x in r.shifts) for r in reports) or any(any(x > 0 for x in r.shifts) for r in reports)
