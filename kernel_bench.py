@@ -201,6 +201,68 @@ def case_kv(rows, reps):
            {"kv_append_kernel": 2 * row * sum((t + 1) for t in n_tok)}, {"kv_append_kernel": "GB/s"})
 
 
+def case_slope(rows, reps):
+    """The small bandwidth-bound kernels at 1x, 2x and 4x the work of a decode step: the time of a
+    launch is a fixed part (launch, the kernel's chain of dependent loads; an empty kernel between
+    the same two events takes about 4 us) plus bytes over a marginal rate, and at the decode step's
+    size the fixed part dominates.  `marginal` is (bytes(4x) - bytes(1x)) / (time(4x) - time(1x))."""
+    torch.manual_seed(1)
+    n = 181
+
+    def series(label, kernel, make):
+        pts = []
+        for mult in (1, 2, 4):
+            fn, nbytes = make(mult)
+            k = timed(fn, reps)
+            pts.append((nbytes, k[kernel][1]))
+            report(rows, f"{label} x{mult}", {kernel: k[kernel]}, {kernel: nbytes}, {kernel: "GB/s"})
+            del fn
+            torch.cuda.empty_cache()
+        (b1, t1), _, (b4, t4) = pts
+        marginal = (b4 - b1) / ((t4 - t1) * 1e-6) / 1e9
+        fixed = t1 - b1 / (marginal * 1e9) * 1e6
+        rows.append(dict(case=f"{label}: marginal rate {marginal:.0f} GB/s ({marginal / HBM * 100:.0f}% of peak), "
+                              f"fixed part {fixed:.1f} us of {t1:.1f} us at x1", kernel=kernel, launches_per_call=0, avg_us=0.0,
+                         algorithmic_work=None, achieved=None, unit="", frac_of_peak=None, note=""))
+
+    def logits_case(op):
+        def make(mult):
+            logits = torch.randn(B * mult, n, V, device="cuda").to(torch.bfloat16)
+            return (lambda: op(logits)), B * mult * n * V * 2
+        return make
+
+    series("argmax packed bf16 logits", "argmax_rows_kernel", logits_case(acceptance.argmax_rows))
+    series("verify_row_stats packed bf16 logits", "row_stats_kernel", logits_case(lambda x: acceptance.verify_row_stats(x, 1.0)))
+
+    def gather(mult):
+        hidden = torch.randn(B * mult, n, 4096, device="cuda").to(torch.bfloat16)
+        unp = torch.randint(0, n, (B * mult, W, L), device="cuda")
+        return (lambda: tree_attention.unpack(hidden, unp)), 2 * B * mult * W * L * 4096 * 2
+
+    series("unpack hidden (B,n,4096) bf16", "gather_rows_kernel", gather)
+
+    def append(mult):
+        prev = 1500
+        layers = 8 * mult  # (a quarter of the model's layers at x1: the series stays inside 32 layers' memory)
+        cache = kv_cache.Cache(B, prev + W * L + 64, layers, H, D, torch.bfloat16, torch.device("cuda"))
+        beams = torch.tensor(synthetic_beams(B, W, L), device="cuda")
+        tree = tree_attention.build_tree(beams)
+        ids = torch.randint(1, V, (B, prev), device="cuda")
+        n_tok = [4, 0, 1, 2, 3, 0, 1, 2]
+        nt = torch.tensor(n_tok, device="cuda")
+        sb = torch.zeros(B, dtype=torch.long, device="cuda")
+        cache.rows_in_place = True
+
+        def run():
+            cache.set_length(prev + tree.n)
+            cache.shift.zero_()
+            acceptance.realign(ids, nt, sb, beams, cache, 0, unpacker=tree.unpacker)
+
+        return run, 2 * layers * 2 * H * D * 2 * sum(t + 1 for t in n_tok)
+
+    series("kv_append, 8 layers x", "kv_append_kernel", append)
+
+
 def case_rope(rows, reps):
     prev, n = 1500, 181
     cache = kv_cache.Cache(B, prev + n + 8, 1, H, D, torch.bfloat16, torch.device("cuda"))
@@ -242,7 +304,7 @@ def case_traffic(rows, reps):
 
 
 CASES = dict(rope=case_rope, traffic=case_traffic, tree=case_tree, tree_x64=lambda r, n: case_tree(r, n, 64), attention=case_attention, beam=case_beam,
-             logits=case_logits, kv=case_kv)
+             logits=case_logits, kv=case_kv, slope=case_slope)
 
 
 def main():
@@ -251,7 +313,7 @@ def main():
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
-    names = [n for n in args.only.split(",") if n] or [n for n in CASES if n != "traffic"]
+    names = [n for n in args.only.split(",") if n] or [n for n in CASES if n not in ("traffic", "slope")]
     rows = []
     for name in names:
         CASES[name](rows, args.reps)
@@ -259,6 +321,9 @@ def main():
         print(json.dumps(rows))
         return
     for r in rows:
+        if r["unit"] == "":
+            print(r["case"])
+            continue
         if r["unit"] is None and r["algorithmic_work"] is not None:
             print(f"{r['case']:<72} {r['kernel']:<22} algorithmic bytes per launch {r['algorithmic_work']:.0f}")
             continue

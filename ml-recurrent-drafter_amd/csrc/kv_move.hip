@@ -141,10 +141,19 @@ __global__ __launch_bounds__(kThreads) void kv_append_kernel(
   vec16 r[kAppendPer];
 #pragma unroll
   for (int u = 0; u < kAppendPer; ++u) {
-    int v = lane + 32 * u;
-    v = v < total ? v : 0;  // clamped, not skipped: keeps the array in registers
-    const int j = v / vpr, c = v - j * vpr;
-    int64_t row = total > 0 ? rp[4 + j] : 0;
+    // Every thread reads something, whether its vector is wanted or not (a read that is skipped on
+    // some path would send the array through scratch memory); an unwanted one re-reads the first
+    // vector of the first row.  The plan's row entry is picked without looking at n_new, so that
+    // it is requested together with the plan's counts instead of after them (entries past n_new
+    // may hold anything: they are read, never used).
+    const int v = lane + 32 * u;
+    int j = v / vpr;
+    int c = v - j * vpr;
+    j = j < L ? j : L - 1;
+    const int32_t listed = rp[4 + j], first = rp[4];
+    const bool want = v < total;
+    int64_t row = want ? listed : first;
+    c = want ? c : 0;
     row = (row < 0 || row >= max_len) ? 0 : row;
     r[u] = *reinterpret_cast<const vec16*>(base + row * row_bytes + (c << 4));
   }
