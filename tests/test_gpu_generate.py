@@ -1,8 +1,9 @@
 """GPU end-to-end: RecurrentDrafting.generate on the HIP path.
 
 float32 tiny models: token-identical to the reference's own greedy streams (fixtures) and to the
-torch restatement run on the same GPU.  bf16: teacher-forced agreement is reported by bench.py;
-here a short bf16 run is checked for self-consistency against the restatement step by step."""
+torch restatement run on the same GPU.  bf16: a short run of the tiny model is checked against the
+restatement step by step here; the bf16 / head_dim 128 path of the large configuration (MFMA
+attention, packed rows, cache rows in place) is compared teacher-forced in test_gpu_decode_bf16.py."""
 import os
 import sys
 
