@@ -16,7 +16,8 @@ step (oracle/torch_path.py) timed on this machine's host cores on a bounded samp
 headline, the same step at other points of its operating range, E timed steps each (`long_context`:
 prompts of 1500 and 2500 tokens; `ragged_acceptance`: prompts of 1200 tokens with the acceptance
 decision replaced by random accepted lengths, so that rows shift, accepted rows are appended and
-the trees grow -- random-init models accept nothing by themselves).
+the trees grow -- random-init models accept nothing by themselves; `rope_attention_launches`: the
+headline's step with the opt-in fused rotation + append + attention kernel against the default two).
 """
 
 from __future__ import annotations
@@ -198,6 +199,20 @@ def gpu_run(steps: int, warmup: int, extra_steps: int):
             others[name] = r
             log(f"[bench] {name}: {r['elapsed'] / r['steps'] * 1e3:.2f} ms/step over {r['steps']} steps, "
                 f"context {r['context']}, {r['per_seq_tokens']:.2f} tokens per sequence and step")
+        # rotation + cache append + attention of a layer as two launches (the default, and what every
+        # other figure of this line is measured on) against one (rd_rope_verify_attention), back to
+        # back on the headline's prompts
+        from recurrent_drafting_amd import modeling_llama
+        default = modeling_llama.LlamaAttention.fused_rope_attention
+        try:
+            for name, fused in (("two_kernels", False), ("one_kernel", None)):
+                modeling_llama.LlamaAttention.fused_rope_attention = fused
+                r = timed_decode(model, prompts(dev, PROMPT), extra_steps, warmup, 64 + 5 * (extra_steps + warmup))
+                r["null_us"] = run["null_us"]
+                others["rope_attention_" + name] = r
+                log(f"[bench] rope + append + attention as {name}: {r['elapsed'] / r['steps'] * 1e3:.2f} ms/step")
+        finally:
+            modeling_llama.LlamaAttention.fused_rope_attention = default
 
     # ---- stage breakdown with the reference's synchronised timers, on a few extra steps ---------------
     ledger2 = rd.stats.Ledger(sync=True)
@@ -504,6 +519,14 @@ def main():
         # of the 500 -> 2548 trajectory, and random-init models accept no drafted token)
         "long_context": {k: summary_of(r) for k, r in run["others"].items() if k.startswith("context_")},
         "ragged_acceptance": {k: summary_of(r) for k, r in run["others"].items() if k.startswith("ragged_")},
+        # opt-in fused kernel against the default pair of kernels, same prompts, back to back (the
+        # fused launch also rotates q and k and appends k and v: its time is not the attention's alone)
+        "rope_attention_launches": {
+            k[len("rope_attention_"):]: {"ms_per_step": round(r["elapsed"] / r["steps"] * 1e3, 3),
+                                         "tokens_per_second": round(r["tokens"] / r["elapsed"], 2),
+                                         "attn_mfma_kernel_avg_us": (lambda d: round(d[1] * 1e3 / d[0], 2) if d[0] else None)(
+                                             r["dominant"].get("attn_mfma_kernel", (0, 0.0)))}
+            for k, r in run["others"].items() if k.startswith("rope_attention_")},
         "kernel_avg_us": {k: round(ms * 1e3 / n, 2) for k, (n, ms) in sorted(run["kernels"].items())},
     }
     line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(run["per_seq_tokens"])

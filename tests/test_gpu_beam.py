@@ -55,7 +55,7 @@ def test_step_fp32_tie_free(B, W, V, t, force_fallback):
 
 
 @pytest.mark.parametrize("force_fallback", [False, True])
-def test_step_first_iteration_only_beam_zero_alive(force_fallback):
+def test_step_first_iteration_only_beam_zero_alive_ties_by_lowest_index_rule(force_fallback):
     """Scores [0, -50000, ...]: every winner descends from beam 0; W=64 > 50 needs filtered tokens,
     which tie exactly and are taken in increasing token id."""
     torch.manual_seed(1)
@@ -88,7 +88,7 @@ def test_step_reads_one_shared_row_in_place(dtype, force_fallback):
 
 
 @pytest.mark.parametrize("force_fallback", [False, True])
-def test_step_bf16_rounding_points(force_fallback):
+def test_step_bf16_rounding_points_ties_by_lowest_index_rule(force_fallback):
     """bf16 logits: values rounded after the max subtraction, filter value -49920, log-softmax
     rounded to bf16, score float32.  Heavy ties among rounded scores -> lowest flat index wins."""
     torch.manual_seed(2)
@@ -108,7 +108,7 @@ def test_step_bf16_rounding_points(force_fallback):
     assert logp[0, 0].min().item() < -49000  # the filter value survives as a finite constant
 
 
-def test_step_many_ties_overflow_to_exact_path():
+def test_step_many_ties_by_lowest_index_rule_overflow_to_exact_path():
     """All-equal and two-valued rows: every entry ties, the candidate list overflows, and the
     lowest indices must win."""
     V, W = 32000, 5
