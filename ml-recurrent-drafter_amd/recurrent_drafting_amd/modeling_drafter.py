@@ -150,6 +150,13 @@ class Drafter(transformers.PreTrainedModel):
         if cfg.rnn:
             self.rnn_u = torch.nn.Linear(cfg.hidden_size, cfg.hidden_size, bias=True)
             self.rnn_w = torch.nn.Linear(cfg.hidden_size, cfg.hidden_size, bias=False)
+        # transformers' bookkeeping for save_pretrained / from_pretrained (newer releases refuse to
+        # load a model whose constructor skipped it); the layers keep torch's own initialisation,
+        # as upstream's do (modeling_drafter.py:104-125 never runs transformers' initialiser)
+        self.post_init()
+
+    def _init_weights(self, module: torch.nn.Module) -> None:
+        return
 
     def raw_logits(self, x: torch.Tensor) -> torch.Tensor:
         """Vocabulary logits of [context, state] before any normalisation: `self.lm_head`, with

@@ -13,6 +13,7 @@ from __future__ import annotations
 from typing import Optional, Tuple
 
 import torch
+import transformers
 from torch import nn
 from transformers.activations import ACT2FN
 from transformers.modeling_outputs import CausalLMOutput
@@ -97,8 +98,7 @@ class LlamaRotaryEmbedding(nn.Module):
                  device: Optional[torch.device] = None):
         super().__init__()
         self.dim, self.base = dim, base
-        inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2).float().to(device) / dim))
-        self.register_buffer("inv_freq", inv_freq)
+        self.register_buffer("inv_freq", self.fresh_inv_freq(device))
         self._build(max_position_embeddings, self.inv_freq.device, torch.get_default_dtype())
 
     def _build(self, seq_len: int, device, dtype) -> None:
@@ -110,7 +110,14 @@ class LlamaRotaryEmbedding(nn.Module):
         self.sin_cached = table.sin().to(dtype)
         self._cast = {}
 
+    def fresh_inv_freq(self, device=None) -> torch.Tensor:
+        return 1.0 / (self.base ** (torch.arange(0, self.dim, 2).float().to(device) / self.dim))
+
     def forward(self, device: torch.device, dtype: torch.dtype, seq_len: int = 0):
+        if self.cos_cached.is_meta:
+            # built while transformers constructed the model without memory (from_pretrained of
+            # newer releases): the tables of the constructor, now that inv_freq holds numbers
+            self._build(max(seq_len, self.max_seq_len_cached), self.inv_freq.device, torch.get_default_dtype())
         if seq_len > self.max_seq_len_cached:
             self._build(seq_len, device, dtype)
         key = (device, dtype)
@@ -235,6 +242,14 @@ class LlamaPreTrainedModel(PreTrainedModel):
     config_class = LlamaConfig
     base_model_prefix = "model"
 
+    def _init_weights(self, module: nn.Module) -> None:
+        super()._init_weights(module)
+        # a checkpoint written by transformers' own Llama has no rotary_emb.inv_freq: what
+        # from_pretrained finds missing is what the constructor computes
+        if isinstance(module, LlamaRotaryEmbedding) and not module.inv_freq.is_meta:
+            with torch.no_grad():
+                module.inv_freq.copy_(module.fresh_inv_freq(module.inv_freq.device))
+
 
 class LlamaModel(LlamaPreTrainedModel):
     def __init__(self, config: LlamaConfig):
@@ -273,7 +288,11 @@ def _kv_shift(past_key_values) -> Optional[torch.Tensor]:
 
 
 class LlamaForCausalLM(LlamaPreTrainedModel):
-    _tied_weights_keys = ["lm_head.weight"]
+    # upstream: ["lm_head.weight"] (modeling_llama.py:241); transformers 5 wants the target too
+    _tied_weights_keys = (
+        {"lm_head.weight": "model.embed_tokens.weight"}
+        if int(transformers.__version__.split(".")[0]) >= 5 else ["lm_head.weight"]
+    )
 
     def __init__(self, config):
         super().__init__(config)
