@@ -101,10 +101,11 @@ class LlamaRotaryEmbedding(nn.Module):
         self.register_buffer("inv_freq", self.fresh_inv_freq(device))
         self._build(max_position_embeddings, self.inv_freq.device, torch.get_default_dtype())
 
-    def _build(self, seq_len: int, device, dtype) -> None:
+    def _build(self, seq_len: int, device, dtype, inv_freq: Optional[torch.Tensor] = None) -> None:
         self.max_seq_len_cached = seq_len
-        t = torch.arange(seq_len, device=device, dtype=self.inv_freq.dtype)
-        angles = torch.outer(t, self.inv_freq.to(device))
+        inv_freq = self.inv_freq if inv_freq is None else inv_freq
+        t = torch.arange(seq_len, device=device, dtype=inv_freq.dtype)
+        angles = torch.outer(t, inv_freq.to(device))
         table = torch.cat((angles, angles), dim=-1)
         self.cos_cached = table.cos().to(dtype)
         self.sin_cached = table.sin().to(dtype)
@@ -116,8 +117,9 @@ class LlamaRotaryEmbedding(nn.Module):
     def forward(self, device: torch.device, dtype: torch.dtype, seq_len: int = 0):
         if self.cos_cached.is_meta:
             # built while transformers constructed the model without memory (from_pretrained of
-            # newer releases): the tables of the constructor, now that inv_freq holds numbers
-            self._build(max(seq_len, self.max_seq_len_cached), self.inv_freq.device, torch.get_default_dtype())
+            # newer releases): the constructor's tables again, from the constructor's float32
+            # frequencies (the buffer may have been cast to the checkpoint's dtype since)
+            self._build(self.max_seq_len_cached, device, torch.float32, self.fresh_inv_freq(device))
         if seq_len > self.max_seq_len_cached:
             self._build(seq_len, device, dtype)
         key = (device, dtype)
