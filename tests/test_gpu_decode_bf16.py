@@ -11,7 +11,9 @@ which bar).
    acceptance decision replaced by random accepted lengths;
 3. one layer of the 7B shape (hidden 4096, 32 heads x 128, FFN 11008, vocabulary 32000; drafter
    4096/8192 with two blocks), batch 8, about 1500 tokens of context with ragged left padding,
-   beam 45 x 5: forced ragged acceptance for a few steps, then teacher-forced steps.
+   beam 45 x 5: forced ragged acceptance for a few steps, then teacher-forced steps;
+4. speculative sampling at temperature 1 on the pair of 1: every step's acceptance and residual
+   distribution against the oracle on the step's own logits, drafter log-probabilities and uniforms.
 """
 import os
 import sys
@@ -121,3 +123,83 @@ def test_bf16_7b_shape_one_layer_teacher_forced_steps_at_long_context():
     assert all(r.prev >= 1500 and r.n_q >= 100 for r in reports)
     assert all(r.beams_shared >= 0.5 for r in reports)
     assert any(any(x != 0 for x in r.shifts) for r in reports)
+
+
+def test_bf16_mfma_sampling_loop_accepts_as_the_oracle_does_on_the_same_logits():
+    """Speculative sampling at temperature 1 through the same bf16 / 128-wide-head path (MFMA
+    attention, packed rows spread back to their slots for the head, cache rows in place).  Every
+    step's acceptance runs on packed bf16 logits and four floats per row; the oracle gets the
+    same logits unpacked and log-softmaxed as the reference materialises them, the same drafter
+    log-probabilities and the same uniforms, and must accept the same tokens from the same beams
+    and hand the same residual distribution to the draw (the draw itself is replaced by the mode)."""
+    import unittest.mock
+
+    import numpy as np
+
+    import recurrent_drafting_amd as rd
+    from oracle import fp_oracle as O
+    from oracle import torch_path as P
+    from oracle import tree_oracle as T
+    from recurrent_drafting_amd import acceptance
+
+    llama_sd, drafter_sd = tm.markov(43, llama_cfg=CFG, drafter_cfg=DCFG, mix=0.05)
+    llm, drafter = _models(llama_sd, drafter_sd, CFG, DCFG)
+    ids = tm.prompt(4, 260, 4000, 7, left_pads=[0, 100, 5, 200]).cuda()
+    W, L, temperature, steps = 12, 5, 1.0, 10
+    seen = []
+    real_accept, real_residual = acceptance.sample_accept, acceptance.residual_probs
+
+    def oracle_log_p(packed):
+        unpacked = T.unpack_rows(packed.logits.float().cpu().numpy(), packed.unpacker.cpu().numpy())  # (B,W,L,V)
+        return (O.warp_logits(torch.tensor(unpacked)) / packed.temperature).log_softmax(dim=-1)
+
+    def w_accept(beams, log_p, log_q, uniforms):
+        n, s = real_accept(beams, log_p, log_q, uniforms)
+        ref = oracle_log_p(log_p)
+        on, os_ = P.sample_choose(beams.cpu(), ref, log_q.cpu(), uniforms.cpu())
+        tok = beams.cpu()[..., 1:, None]
+        ratio = torch.exp(ref[:, :, :-1].gather(-1, tok).squeeze(-1) - log_q.cpu().gather(-1, tok).squeeze(-1))
+        fragile = bool(((uniforms.cpu() - ratio).abs() < 1e-4 * ratio.clamp(min=1)).any())
+        seen.append(dict(n=n.cpu(), s=s.cpu(), on=on, os=os_, fragile=fragile, ref=ref))
+        return n, s
+
+    def w_residual(log_q, log_p, seq_in_beam, n_tokens):
+        got = real_residual(log_q, log_p, seq_in_beam, n_tokens)
+        want = P.residual_distribution(log_q.cpu(), seen[-1]["ref"], seq_in_beam.cpu(), n_tokens.cpu())
+        seen[-1]["residual_err"] = float((got.cpu() - want).abs().max())
+        seen[-1]["residual_negative"] = bool((got < 0).any())
+        return got
+
+    class Mode:
+        def __init__(self, probs=None, **kw):
+            self.p = probs
+
+        def sample(self):
+            return self.p.argmax(dim=-1)
+
+    def loop():
+        model = rd.RecurrentDrafting(llm, drafter)
+        out = []
+        with unittest.mock.patch.object(acceptance, "sample_accept", w_accept), \
+                unittest.mock.patch.object(acceptance, "residual_probs", w_residual), \
+                unittest.mock.patch("torch.distributions.Categorical", Mode):
+            torch.manual_seed(5)
+            for i, t in enumerate(model.generate(rd.stats.Ledger(), ids, 260 + 60, rd.BeamShape(W, L),
+                                                 rd.SamplingArgs(temperature, False), rd.SpecialTokens(0, None))):
+                out.append(t)
+                if i + 1 >= steps:
+                    break
+        return out
+
+    out, kernels = _uses_mfma_kernel(loop)
+    assert "attn_mfma_kernel" in kernels and "attn_generic_kernel" not in kernels
+    assert {"row_stats_kernel", "accept_sample_kernel", "residual_probs_kernel"} <= set(kernels)
+    assert len(seen) >= steps
+    for k, st in enumerate(seen):
+        if not st["fragile"]:
+            assert torch.equal(st["n"], st["on"]) and torch.equal(st["s"], st["os"]), (k, st["n"], st["on"])
+        assert st["residual_err"] < 1e-5 and not st["residual_negative"], (k, st["residual_err"])
+    accepted = [int(x) for st in seen for x in st["n"]]
+    print("accepted per row and step:", accepted)
+    assert max(accepted) >= 2 and len(set(accepted)) >= 3  # ragged acceptance happened
+    assert sum(not st["fragile"] for st in seen) >= len(seen) - 1
