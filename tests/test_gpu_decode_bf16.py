@@ -82,14 +82,16 @@ def test_bf16_mfma_decode_loop_teacher_forced_with_accepted_drafts():
     assert sum(r.beams_equal for r in reports) >= len(reports) - 1
 
 
-@pytest.mark.parametrize("one_kernel", [False, True])
-def test_bf16_mfma_decode_loop_teacher_forced_random_weights_forced_acceptance(one_kernel, monkeypatch):
-    # one_kernel: rotation, cache append and attention of a layer as one launch (rd_rope_verify_attention)
+@pytest.mark.parametrize("one_kernel,kv_heads", [(False, 4), (True, 4), (False, 2), (True, 1)])
+def test_bf16_mfma_decode_loop_teacher_forced_random_weights_forced_acceptance(one_kernel, kv_heads, monkeypatch):
+    # one_kernel: rotation, cache append and attention of a layer as one launch (rd_rope_verify_attention);
+    # kv_heads below 4: grouped-query attention (the query heads of a group share cache rows)
     from recurrent_drafting_amd import modeling_llama
     monkeypatch.setattr(modeling_llama.LlamaAttention, "fused_rope_attention", None if one_kernel else False)
-    llama_sd = tm.draw(tm.llama_shapes(CFG), 51)
+    cfg = dict(CFG, num_key_value_heads=kv_heads)
+    llama_sd = tm.draw(tm.llama_shapes(cfg), 51)
     drafter_sd = tm.draw(tm.drafter_shapes(DCFG), 52)
-    llm, drafter = _models(llama_sd, drafter_sd, CFG, DCFG)
+    llm, drafter = _models(llama_sd, drafter_sd, cfg, DCFG)
     ids = tm.prompt(4, 200, 4000, 6, left_pads=[17, 0, 120, 64]).cuda()
     reports, kernels = _uses_mfma_kernel(
         lambda: teacher_forced.run(llm, drafter, ids, 200 + 60, 12, 5, steps=10,
