@@ -292,3 +292,77 @@ def test_update_ids_doc_example(literals):
     assert ids.cpu().tolist() == e["expected_ids"] and cache.sliced[0][0].length == e["max_seq_len"]
     assert torch.equal(cache._cache[:, :, 0, :, 1:6], before[:, :, 0, :, 0:5])
     assert torch.equal(cache._cache[:, :, 1, :, 0:6], before[:, :, 1, :, 1:7])
+
+
+def test_kv_unpack_and_realign_at_the_full_configuration_size():
+    """Configuration 4's cache (32 layers x 2 x batch 8 x 32 heads x 128, bf16, 1500 cached tokens,
+    beam 45 x 5: 7 GB) through Cache.unpack + the re-alignment, and through the fused re-alignment
+    with the rows moved and with the rows kept in place.  Moving rows is the same permutation in
+    every layer, head and column, so the oracle runs on a one-column cache whose values are row
+    numbers, and tells where every live row of the result came from; the full-size result must
+    hold exactly those rows of the full-size input."""
+    from recurrent_drafting_amd import acceptance, kv_cache
+
+    rng = np.random.default_rng(11)
+    B, W, L, NL, H, D, prev = 8, 45, 5, 32, 32, 128, 1500
+    pads = rng.integers(0, 400, size=B)
+    pads[3] = 0
+    ids = rng.integers(1, 32000, size=(B, prev))
+    for b in range(B):
+        ids[b, : pads[b]] = 0
+    beams = T.synthetic_beams(B, W, L, vocab=32000, seed=11) + 1
+    tok, unp, _, _, _ = T.pack(beams, (ids != 0).astype(np.int64))
+    n_sel = tok.shape[1]
+    max_len = prev + W * L + 3
+    n_tok = np.array([4, 0, 1, 2, 3, 0, 1, 2])
+    s_beam = rng.integers(0, W, size=B)
+
+    rows = np.broadcast_to(np.arange(max_len, dtype=np.float32)[None, None, None, None, :, None], (1, 2, B, 1, max_len, 1)).copy()
+    Acc.kv_unpack(rows, prev, unp)
+    unpacked_from = rows[0, 0, :, 0, :, 0].astype(np.int64).copy()  # (B, max_len): source row of every row
+    o_ids, M = Acc.update_kv_and_ids(ids, n_tok, s_beam, beams, rows, 0)
+    final_from = rows[0, 0, :, 0, :, 0].astype(np.int64)
+    new_pads = T.count_left_paddings(o_ids, 0)
+
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cuda").manual_seed(3)
+    before = torch.empty((NL, 2, B, H, max_len, D), dtype=torch.bfloat16, device=dev)
+    before.view(torch.int16).random_(-30000, 30000, generator=g)  # arbitrary bit patterns, made finite below
+    before.nan_to_num_(nan=1.0, posinf=2.0, neginf=-2.0)
+
+    def fresh():
+        c = kv_cache.Cache(B, max_len, NL, H, D, torch.bfloat16, dev)
+        c._cache.copy_(before)
+        c.set_length(prev + n_sel)
+        return c
+
+    def same_rows(c, source, lo_of, hi):
+        for b in range(B):
+            lo = int(lo_of[b])
+            src = torch.tensor(source[b, lo:hi], device=dev)
+            want = before[:, :, b, :, :, :].index_select(3, src)
+            assert torch.equal(c._cache[:, :, b, :, lo:hi, :].view(torch.int16), want.view(torch.int16)), b
+
+    zeros = np.zeros(B, dtype=np.int64)
+    # drop-in sequence
+    c = fresh()
+    c.unpack(prev, _dev(unp))
+    same_rows(c, unpacked_from, zeros, prev + W * L)
+    g_ids = acceptance._update_kv_cache_and_input_ids(_dev(ids), _dev(n_tok), _dev(s_beam), _dev(beams), c, 0)
+    assert np.array_equal(g_ids.cpu().numpy(), o_ids) and c.sliced[0][0].length == M
+    same_rows(c, final_from, new_pads, M)
+    del c
+    # fused: accepted rows straight from their packed slots, rows moved
+    c = fresh()
+    g_ids = acceptance.realign(_dev(ids), _dev(n_tok), _dev(s_beam), _dev(beams), c, 0, unpacker=_dev(unp))
+    assert np.array_equal(g_ids.cpu().numpy(), o_ids)
+    same_rows(c, final_from, new_pads, M)
+    del c
+    # fused, rows kept in place; materialize() then gives the reference's layout
+    c = fresh()
+    c.rows_in_place = True
+    g_ids = acceptance.realign(_dev(ids), _dev(n_tok), _dev(s_beam), _dev(beams), c, 0, unpacker=_dev(unp))
+    assert np.array_equal(g_ids.cpu().numpy(), o_ids)
+    assert c.shift.cpu().tolist() == [int(new_pads[b] - pads[b]) for b in range(B)]
+    c.materialize()
+    same_rows(c, final_from, new_pads, M)
