@@ -63,6 +63,14 @@ RD_API int rd_timing_sample(int every);
  * kernel trace does not.  Synchronises the stream. */
 RD_API int rd_timing_null_kernel_us(int launches, void* stream, float* avg_us);
 RD_API int rd_timing_collect(char* out, size_t out_bytes);
+/* Yardstick for the verification attention's memory side (no counterpart in the reference; used
+ * by kernel_bench.py): `slabs` workgroups of 512 threads each stream `tiles` tiles of 64 rows x
+ * 256 bytes from their slab of k and of v (slab i begins at i * slab_bytes), `depth` (1, 2 or 4)
+ * tiles ahead in registers, through LDS and a barrier per tile -- the loads, staging and barrier
+ * of rd_verify_attention's tile loop without its arithmetic.  sink: slabs * 512 uint32, written
+ * so that the loads cannot be dropped.  Timed under the name "stream_tiles_kernel". */
+RD_API int rd_stream_tiles_probe(const void* k, const void* v, int64_t slab_bytes, int slabs, int tiles,
+                                 int depth, void* sink, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Draft beams -> prefix tree -> packed tokens.

@@ -263,6 +263,27 @@ def case_slope(rows, reps):
     series("kv_append, 8 layers x", "kv_append_kernel", append)
 
 
+def case_stream(rows, reps):
+    """What the memory system delivers to the attention's access pattern (a K and a V slab per
+    (batch row, head), 64-row tiles, one 512-thread workgroup per compute unit) when the tile loop
+    does nothing but load, stage and meet at its barrier: rd_stream_tiles_probe.  The slabs are those
+    of a cache of 2560 + 128 rows, 690 MB together: more than the 256 MB memory-side cache."""
+    slabs, max_len = B * H, 2560 + 128
+    k = torch.randn(slabs, max_len, D, device="cuda").to(torch.bfloat16)
+    v = torch.randn(slabs, max_len, D, device="cuda").to(torch.bfloat16)
+    sink = torch.empty(slabs * 512, dtype=torch.int32, device="cuda")
+    lib = _hip.lib()
+    for keys in (640, 1536, 2560):
+        tiles = keys // 64
+        for depth in (1, 2, 4):
+            fn = lambda: _hip.check(lib.rd_stream_tiles_probe(_hip.ptr(k), _hip.ptr(v), max_len * D * 2, slabs, tiles, depth,
+                                                              _hip.ptr(sink), _hip.stream()))
+            kk = timed(fn, reps)
+            nbytes = 2 * slabs * tiles * 64 * D * 2
+            report(rows, f"stream K/V tiles only, {keys} keys per row, {depth} tile(s) ahead", kk,
+                   {"stream_tiles_kernel": nbytes}, {"stream_tiles_kernel": "GB/s"})
+
+
 def case_rope(rows, reps):
     prev, n = 1500, 181
     cache = kv_cache.Cache(B, prev + n + 8, 1, H, D, torch.bfloat16, torch.device("cuda"))
@@ -304,7 +325,7 @@ def case_traffic(rows, reps):
 
 
 CASES = dict(rope=case_rope, traffic=case_traffic, tree=case_tree, tree_x64=lambda r, n: case_tree(r, n, 64), attention=case_attention, beam=case_beam,
-             logits=case_logits, kv=case_kv, slope=case_slope)
+             logits=case_logits, kv=case_kv, slope=case_slope, stream=case_stream)
 
 
 def main():
@@ -313,7 +334,7 @@ def main():
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
-    names = [n for n in args.only.split(",") if n] or [n for n in CASES if n not in ("traffic", "slope")]
+    names = [n for n in args.only.split(",") if n] or [n for n in CASES if n not in ("traffic", "slope", "stream")]
     rows = []
     for name in names:
         CASES[name](rows, args.reps)

@@ -24,6 +24,7 @@ _P, _I, _L, _Z, _F = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 _PROTOTYPES = {
     "rd_version": (C.c_int, []),
     "rd_last_error": (C.c_char_p, []),
+    "rd_stream_tiles_probe": (_I, [_P, _P, _L, _I, _I, _I, _P, _P]),
     "rd_timing_enable": (_I, [_I]),
     "rd_timing_select": (_I, [C.c_char_p]),
     "rd_timing_sample": (_I, [_I]),
