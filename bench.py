@@ -16,7 +16,8 @@ step (oracle/torch_path.py) timed on this machine's host cores on a bounded samp
 headline, the same step at other points of its operating range, E timed steps each (`long_context`:
 prompts of 1500 and 2500 tokens; `ragged_acceptance`: prompts of 1200 tokens with the acceptance
 decision replaced by random accepted lengths, so that rows shift, accepted rows are appended and
-the trees grow -- random-init models accept nothing by themselves; `rope_attention_launches`: the
+the trees grow -- random-init models accept nothing by themselves; `ragged_prompts`: prompts of 500
+to 2500 tokens in one batch, left-padded; `rope_attention_launches`: the
 headline's step with the opt-in fused rotation + append + attention kernel against the default two).
 """
 
@@ -135,7 +136,7 @@ def timed_decode(model, ids, steps: int, warmup: int, max_new: int, force=None):
         _hip.timing_sample(TIMED_EVERY)
         _hip.timing_enable(True)
         elapsed, timed = 0.0, 0
-        first_len = last_len = None
+        first_len = last_len = first_out = None
         out = None
         while timed < steps:
             torch.cuda.synchronize()
@@ -148,7 +149,8 @@ def timed_decode(model, ids, steps: int, warmup: int, max_new: int, force=None):
                     exhausted = True
                     break
                 seg += 1
-                first_len = out.shape[1] if first_len is None else first_len
+                if first_len is None:
+                    first_len, first_out = out.shape[1], out
                 last_len = out.shape[1]
             torch.cuda.synchronize()
             elapsed += time.perf_counter() - start
@@ -162,14 +164,17 @@ def timed_decode(model, ids, steps: int, warmup: int, max_new: int, force=None):
         _hip.timing_select(None)
         _hip.timing_sample(1)
         attention.shape_log = None
-        final_pads = int((out == 0).long().cumprod(dim=-1).sum()) if out is not None else 0
+        left_pads = lambda ids: int((ids == 0).long().cumprod(dim=-1).sum())  # noqa: E731
+        final_pads = left_pads(out) if out is not None else 0
+        first_pads = left_pads(first_out) if first_out is not None else 0
         stream.close()  # posts the open generation's record
     finally:
         acceptance.greedy_accept = real_accept
     accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
     per_seq_tokens = sum(a + 1 for a in accepted) / max(len(accepted), 1)
     return dict(elapsed=elapsed, steps=timed, per_seq_tokens=per_seq_tokens, tokens=per_seq_tokens * BATCH * timed,
-                dominant=dominant, shapes=shapes, context=(first_len, last_len), final_left_pads=final_pads)
+                dominant=dominant, shapes=shapes, context=(first_len, last_len), final_left_pads=final_pads,
+                first_left_pads=first_pads)
 
 
 def gpu_run(steps: int, warmup: int, extra_steps: int):
@@ -199,6 +204,19 @@ def gpu_run(steps: int, warmup: int, extra_steps: int):
             others[name] = r
             log(f"[bench] {name}: {r['elapsed'] / r['steps'] * 1e3:.2f} ms/step over {r['steps']} steps, "
                 f"context {r['context']}, {r['per_seq_tokens']:.2f} tokens per sequence and step")
+        # prompts of different lengths, left-padded to the longest, as a batch of unrelated requests
+        # has them: the attention's rows then differ in their number of keys and its work items
+        # are cut by the plan's model of the launch
+        ids = prompts(dev, 2500)
+        lens = torch.randint(500, 2501, (BATCH,), generator=torch.Generator().manual_seed(SEED))
+        lens[0] = 2500
+        for b, n in enumerate(lens.tolist()):
+            ids[b, : 2500 - n] = 0
+        r = timed_decode(model, ids, extra_steps, warmup, 64 + 5 * (extra_steps + warmup))
+        r["null_us"] = run["null_us"]
+        r["prompt_tokens"] = sorted(lens.tolist())
+        others["prompts_of_500_to_2500_tokens"] = r
+        log(f"[bench] prompts of {r['prompt_tokens']} tokens: {r['elapsed'] / r['steps'] * 1e3:.2f} ms/step")
         # rotation + cache append + attention of a layer as two launches (the default, and what every
         # other figure of this line is measured on) against one (rd_rope_verify_attention), back to
         # back on the headline's prompts
@@ -255,10 +273,11 @@ def attention_roofline(run):
     shapes = run["shapes"][::TIMED_EVERY][:count] if count else []  # the launches that were timed
     if not count or total_ms <= 0:
         return None
-    # keys: every row from its first real token to its last tree slot.  Left padding only appears
-    # with forced acceptance (rows grow at different rates); its average over the run is taken as
-    # half of what the last step shows, and the tree slots a row does not have are left out.
-    pads = run.get("final_left_pads", 0) / 2.0
+    # keys: every row from its first real token to its last tree slot.  Left padding appears with
+    # prompts of different lengths and with forced acceptance (rows grow at different rates); its
+    # average over the run is taken as the mean of what the first and the last timed step show,
+    # and the tree slots a row does not have are left out.
+    pads = (run.get("first_left_pads", 0) + run.get("final_left_pads", 0)) / 2.0
     keys = [B * (kv - n_q) - pads + rows for (B, n_q, kv, rows) in shapes]
     flops = sum(4.0 * H * D * (rows / B) * k for (B, n_q, kv, rows), k in zip(shapes, keys))
     k_bytes = sum(2.0 * H * D * 2 * k + 2.0 * rows * H * D * 2 for (B, n_q, kv, rows), k in zip(shapes, keys))
@@ -519,6 +538,8 @@ def main():
         # of the 500 -> 2548 trajectory, and random-init models accept no drafted token)
         "long_context": {k: summary_of(r) for k, r in run["others"].items() if k.startswith("context_")},
         "ragged_acceptance": {k: summary_of(r) for k, r in run["others"].items() if k.startswith("ragged_")},
+        "ragged_prompts": {k: dict(summary_of(r), prompt_tokens=r["prompt_tokens"]) for k, r in run["others"].items()
+                           if k.startswith("prompts_of_")},
         # opt-in fused kernel against the default pair of kernels, same prompts, back to back (the
         # fused launch also rotates q and k and appends k and v: its time is not the attention's alone)
         "rope_attention_launches": {

@@ -300,6 +300,7 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
  * the items to one compute unit's share of the whole call.  fix_empty_rows != 0 turns a row that attends to nothing into a row
  * that attends to everything, which is what attention.set_sdpa_fully_masked_rows
  * (attention.py:58-72) does and what a finite-minimum additive bias amounts to.
+ * Limits: batch <= 2048 (rd_tree_attn_prepare: 1024), batch * ceil(kv_len / 512) <= 32768.
  *
  * rd_verify_attention: out = softmax(q k^T * scale, masked) v per (batch row, head).  Replaces
  * repeat_interleave + F.scaled_dot_product_attention(attn_mask=bias) (modeling_llama.py:161-169).

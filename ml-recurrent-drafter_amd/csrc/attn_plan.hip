@@ -56,7 +56,9 @@ __global__ __launch_bounds__(kThreads) void mask_bits_kernel(
 
 // The plan from the span of attended keys of every batch row (s_key_min[b], s_key_end[b], in LDS,
 // written before the call; the call begins with a barrier).  Whole workgroup of kThreads.
-__device__ void build_plan(const int* s_key_min, const int* s_key_end, int B, int n_q, int kv_len,
+// s_rows: 2 * B more ints of LDS (the rows' split counts and first items; global memory is only
+// written here, never read back: a serial loop over rows would pay a trip to memory per row).
+__device__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_rows, int B, int n_q, int kv_len,
                            int words, int min_chunk, int max_splits, int n_heads, int n_cu,
                            const int32_t* __restrict__ kv_shift, int32_t* __restrict__ plan,
                            int32_t* __restrict__ counters, int n_counters) {
@@ -65,39 +67,136 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int B, in
   __shared__ int s_len[rd::kAttnSortLimit];
   for (int i = threadIdx.x; i < n_counters; i += kThreads) counters[i] = 0;
   int32_t* per_row = plan + RD_PLAN_HDR;
+  int* s_splits = s_rows;
+  int* s_first_item = s_rows + B;
+  auto begin_of = [&](int b) { return (s_key_min[b] / 64) * 64; };
   int32_t* items = plan + RD_PLAN_HDR + 4 * B;
   __syncthreads();
   for (int b = threadIdx.x; b < B; b += kThreads) {
-    per_row[4 * b + 0] = (s_key_min[b] / 64) * 64;
+    per_row[4 * b + 0] = begin_of(b);
     per_row[4 * b + 3] = kv_shift ? kv_shift[b] : 0;  // cache row of key c is c - shift
   }
   __syncthreads();
+  __shared__ int s_share;
+  __shared__ bool s_search;
   if (threadIdx.x == 0) {
-    // Keys per work item: one compute unit's even share of all (row, head) work, but never below
-    // min_chunk.  Equal rows on a machine with batch*heads == compute units are then not split at
-    // all (no partials to merge); ragged rows are cut so that the longest item is about one share.
+    // Keys per work item, first guess: one compute unit's even share of all (row, head) work, but
+    // never below min_chunk.  Equal rows on a machine with batch*heads == compute units are then
+    // not split at all (no partials to merge).
     long long total = 0;
-    for (int b = 0; b < B; ++b) total += s_key_end[b] - per_row[4 * b + 0];
+    for (int b = 0; b < B; ++b) total += s_key_end[b] - begin_of(b);
     long long share = (total * n_heads + n_cu - 1) / n_cu;
     share = (share + 63) / 64 * 64;
-    s_chunk = (int)(share > min_chunk ? share : min_chunk);
+    s_share = (int)(share > min_chunk ? share : min_chunk);
+    // The search below is for ragged rows: with no row split at the share and one workgroup per
+    // compute unit at most (every decode step of equal rows) the share stands.  It walks over
+    // every piece of every candidate: only where that is a short walk.
+    const long long smallest = s_share;
+    const int q_tiles = n_q <= 256 ? 1 : (n_q + 255) / 256;
+    bool split_at_share = false;
+    for (int b = 0; b < B && !split_at_share; ++b)
+      split_at_share = (s_key_end[b] - begin_of(b) + s_share - 1 - s_share / 8) / s_share > 1;
+    const bool one_round = (long long)B * n_heads * q_tiles <= n_cu;
+    s_search = B <= 32 && (total / smallest + B) * 32 <= 8192 && !(one_round && !split_at_share);
+  }
+  __syncthreads();
+  // an item may run an eighth over the chunk: a row a little longer than it stays whole (cutting
+  // off a short remainder would cost it the partials, the fences and the merge, and would send
+  // the remainders into a second round of items behind the first)
+  auto splits_of = [&](int live, int chunk) {
+    const int splits = (live + chunk - 1 - chunk / 8) / chunk;
+    return splits < 1 ? 1 : (splits > max_splits ? max_splits : splits);
+  };
+  // Ragged rows: the even share is only a guess, because the items run in rounds (every compute
+  // unit holds one workgroup) and each costs a fixed part on top of its tiles.  A few chunk sizes
+  // from the share upwards are therefore tried on a model of the launch, one thread each: the pieces of
+  // every row, longest first, go to the least loaded of the n_cu / (heads * query tiles) groups
+  // of compute units that an item's workgroups fill together; a piece costs its 64-key tiles plus
+  // kFixed (launch of the item, first tiles, store), a piece of a split row kSplit more (partials,
+  // fence and count: the fences slow the whole XCD, so the price is high), and a split row's
+  // merge kMerge at the end, all in half tiles, fitted to measured launches.  The share stands
+  // unless another size is at least 5 % better.  (Same box, eight rows of 500-2548 keys, 32
+  // heads: 86 -> 67 us at 168 query rows, 63 -> 48 us at 88.)
+  constexpr int kCands = 13, kMaxRows = 32, kMaxGroups = 32;
+  constexpr int kTile = 2, kFixed = 10, kSplit = 20, kMerge = 8;
+  __shared__ int s_est[kCands];
+  __shared__ int s_plen[kCands][2 * kMaxRows], s_pcnt[kCands][2 * kMaxRows], s_load[kCands][kMaxGroups];
+  __shared__ int s_sorted_len[kCands][2 * kMaxRows], s_sorted_cnt[kCands][2 * kMaxRows];
+  auto candidate = [&](int c) {
+    return (int)((long long)s_share * (8 + c) / 8) / 64 * 64;  // share * (1 .. 2.5): smaller ones only split more
+  };
+  if (s_search && threadIdx.x < kCands) {
+    const int c = threadIdx.x, chunk = candidate(c);
+    const int q_tiles = n_q <= 256 ? 1 : (n_q + 255) / 256;
+    const long long per_item = (long long)n_heads * q_tiles;  // workgroups of one item
+    int groups = per_item >= n_cu ? 1 : (int)(n_cu / per_item);
+    groups = groups > kMaxGroups ? kMaxGroups : groups;
+    const int rounds_per_item = per_item >= n_cu ? (int)((per_item + n_cu - 1) / n_cu) : 1;
+    int* plen = s_plen[c];
+    int* pcnt = s_pcnt[c];
+    int n_classes = 0;
+    bool any_split = false;
+    for (int b = 0; b < B; ++b) {  // every row: splits - 1 pieces of `per` keys and the rest
+      const int live = s_key_end[b] - begin_of(b);
+      const int splits = splits_of(live, chunk);
+      int per = (live + splits - 1) / splits;
+      per = (per + 63) / 64 * 64;
+      const int whole = per > 0 ? live / per : 0;  // pieces of full length
+      const int rest = live - whole * per;
+      const int extra = splits > 1 ? kSplit : 0;
+      any_split |= splits > 1;
+      if (whole > 0) { plen[n_classes] = ((per + 63) / 64) * kTile + kFixed + extra; pcnt[n_classes++] = whole; }
+      if (rest > 0) { plen[n_classes] = ((rest + 63) / 64) * kTile + kFixed + extra; pcnt[n_classes++] = 1; }
+    }
+    // longest first: every class finds its rank among the others (independent reads, where an
+    // insertion sort would be a chain of dependent ones)
+    int* slen = s_sorted_len[c];
+    int* scnt = s_sorted_cnt[c];
+    for (int i = 0; i < n_classes; ++i) {
+      const int l = plen[i];
+      int rank = 0;
+      for (int j = 0; j < n_classes; ++j) rank += plen[j] > l || (plen[j] == l && j < i);
+      slen[rank] = l;
+      scnt[rank] = pcnt[i];
+    }
+    int end = 0;
+    {
+      int* load = s_load[c];
+      for (int g = 0; g < groups; ++g) load[g] = 0;
+      for (int i = 0; i < n_classes; ++i)
+        for (int k = 0; k < scnt[i]; ++k) {
+          int least = 0, least_load = load[0];
+          for (int g = 1; g < groups; ++g) {
+            const int l = load[g];
+            if (l < least_load) { least = g; least_load = l; }
+          }
+          least_load += slen[i] * rounds_per_item;
+          load[least] = least_load;
+          end = least_load > end ? least_load : end;
+        }
+    }
+    s_est[c] = end + (any_split ? kMerge : 0);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int chunk = s_share;
+    if (s_search) {
+      const int at_share = s_est[0];  // candidate 0 is the share itself
+      int best = at_share - at_share / 20;  // 5 % better or stay
+      for (int c = 0; c < kCands; ++c)
+        if (s_est[c] < best) { best = s_est[c]; chunk = candidate(c); }
+    }
+    s_chunk = chunk;
   }
   __syncthreads();
   const int chunk = s_chunk;
-  for (int b = threadIdx.x; b < B; b += kThreads) {
-    const int live = s_key_end[b] - per_row[4 * b + 0];
-    // an item may run an eighth over the share: a row a little longer than the share stays whole
-    // (cutting off a short remainder would cost it the partials, the fences and the merge, and
-    // would send the remainders into a second round of items behind the first)
-    int splits = (live + chunk - 1 - chunk / 8) / chunk;
-    per_row[4 * b + 1] = splits < 1 ? 1 : (splits > max_splits ? max_splits : splits);
-  }
+  for (int b = threadIdx.x; b < B; b += kThreads) per_row[4 * b + 1] = s_splits[b] = splits_of(s_key_end[b] - begin_of(b), chunk);
   __syncthreads();
   if (threadIdx.x == 0) {
     int n = 0;
     for (int b = 0; b < B; ++b) {
-      per_row[4 * b + 2] = n;  // first item of this row (before sorting)
-      n += per_row[4 * b + 1];
+      per_row[4 * b + 2] = s_first_item[b] = n;  // first item of this row (before sorting)
+      n += s_splits[b];
     }
     s_n_items = n;
     plan[0] = n; plan[1] = n_q; plan[2] = kv_len; plan[3] = words;
@@ -108,9 +207,9 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int B, in
   // every item computes its own extent and its rank (longest first, ties by index)
   auto extent = [&](int it, int& b, int& s, int& lo, int& hi) {
     b = 0;
-    while (b + 1 < B && per_row[4 * (b + 1) + 2] <= it) ++b;
-    s = it - per_row[4 * b + 2];
-    const int begin = per_row[4 * b + 0], splits = per_row[4 * b + 1], end = s_key_end[b];
+    while (b + 1 < B && s_first_item[b + 1] <= it) ++b;
+    s = it - s_first_item[b];
+    const int begin = begin_of(b), splits = s_splits[b], end = s_key_end[b];
     const int live = end - begin;
     int per = (live + splits - 1) / splits;
     per = (per + 63) / 64 * 64;
@@ -142,9 +241,9 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int B, in
     }
     int32_t* rec = items + RD_ITEM_INTS * rank;
     rec[0] = b; rec[1] = lo; rec[2] = hi; rec[3] = s;
-    rec[4] = per_row[4 * b + 3];
+    rec[4] = kv_shift ? kv_shift[b] : 0;
     rec[5] = s_key_min[b];
-    rec[6] = per_row[4 * b + 1];
+    rec[6] = s_splits[b];
     rec[7] = s_key_end[b];
   }
 }
@@ -158,7 +257,7 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
                                                              int32_t* __restrict__ plan,
                                                              int32_t* __restrict__ counters,
                                                              int n_counters) {
-  extern __shared__ int s_span[];  // [2][B]: first key any query of the row attends to, last such key + 1
+  extern __shared__ int s_span[];  // [4][B]: first key any query of the row attends to, last such key + 1, build_plan's rows
   int* s_key_min = s_span;
   int* s_key_end = s_span + B;
   // per batch row, the span of attended keys: the minimum / maximum over its query rows
@@ -181,7 +280,7 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
       s_key_end[b] = last + 1;
     }
   }
-  build_plan(s_key_min, s_key_end, B, n_q, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan,
+  build_plan(s_key_min, s_key_end, s_span + 2 * B, B, n_q, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan,
              counters, n_counters);
 }
 
@@ -233,7 +332,7 @@ __global__ __launch_bounds__(kThreads) void tree_prepare_kernel(
   if (blockIdx.y == B) {
     // ---- the plan ------------------------------------------------------------------------------
     if (blockIdx.x != 0) return;
-    extern __shared__ int s_span[];  // [2][B]
+    extern __shared__ int s_span[];  // [4][B]
     int* s_key_min = s_span;
     int* s_key_end = s_span + B;
     for (int b = wave; b < B; b += kWaves) {
@@ -250,7 +349,7 @@ __global__ __launch_bounds__(kThreads) void tree_prepare_kernel(
         if (left_pads) left_pads[b] = first;
       }
     }
-    build_plan(s_key_min, s_key_end, B, n, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan,
+    build_plan(s_key_min, s_key_end, s_span + 2 * B, B, n, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan,
                counters, n_counters);
     return;
   }
@@ -321,8 +420,9 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
   RD_REQUIRE(batch > 0 && n_q > 0 && kv_len > 0 && n_heads > 0, RD_EINVAL,
              "rd_attn_prepare: bad sizes (batch %d n_q %d kv_len %d n_heads %d)", batch, n_q, kv_len,
              n_heads);
-  RD_REQUIRE(batch <= 65535 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
-             "rd_attn_prepare: batch %d too large for kv_len %d", batch, kv_len);
+  RD_REQUIRE(batch <= 2048 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
+             "rd_attn_prepare: batch %d too large (2048 rows; %d for kv_len %d)", batch,
+             32768 / rd::attn_max_splits(kv_len), kv_len);
   RD_REQUIRE(mask && bits && plan, RD_EINVAL, "rd_attn_prepare: null pointer");
   RD_REQUIRE(mask_stride_q >= kv_len && mask_stride_b >= 0, RD_EINVAL,
              "rd_attn_prepare: mask_stride_q %lld < kv_len %d", (long long)mask_stride_q, kv_len);
@@ -334,7 +434,7 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
   { rd::ScopedTiming rd_t("mask_bits_kernel", s); hipLaunchKernelGGL(mask_bits_kernel, dim3(n_q, batch), dim3(kThreads), 0, s, mask, mask_stride_b,
                      mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first, row_last); }
   if (int e = rd::check_launch("rd_attn_prepare(bits)")) return e;
-  { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 2 * batch * sizeof(int), s, row_first, row_last, batch, n_q, kv_len,
+  { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 4 * batch * sizeof(int), s, row_first, row_last, batch, n_q, kv_len,
                      words, rd::kAttnChunk, max_splits, n_heads, compute_units(), kv_row_shift, plan,
                      plan + rd::attn_counter_offset(batch, n_q, kv_len), (int)rd::attn_counter_ints(batch, n_q)); }
   return rd::check_launch("rd_attn_prepare(plan)");
@@ -354,8 +454,9 @@ extern "C" int rd_tree_attn_prepare(const int64_t* unpacker, const int64_t* pack
   RD_REQUIRE(prev <= (int64_t)kMaxLeftWords * 64 && prev + n < 2147483647LL, RD_ELIMIT,
              "rd_tree_attn_prepare: prev %lld > %d (use rd_tree_mask + rd_attn_prepare)", (long long)prev, kMaxLeftWords * 64);
   const int kv_len = (int)prev + n;
-  RD_REQUIRE(batch < 65535 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
-             "rd_tree_attn_prepare: batch %d too large for kv_len %d", batch, kv_len);
+  RD_REQUIRE(batch <= 1024 && batch * (int64_t)rd::attn_max_splits(kv_len) <= 32768, RD_ELIMIT,
+             "rd_tree_attn_prepare: batch %d too large (1024 rows; %d for kv_len %d)", batch,
+             32768 / rd::attn_max_splits(kv_len), kv_len);
   RD_REQUIRE(unpacker && packed_token_indices && counts && bits && plan, RD_EINVAL, "rd_tree_attn_prepare: null pointer");
   RD_REQUIRE(prev == 0 || (padding_mask && pm_row_stride >= prev), RD_EINVAL,
              "rd_tree_attn_prepare: padding_mask missing or pm_row_stride %lld < prev %lld", (long long)pm_row_stride, (long long)prev);
@@ -369,7 +470,7 @@ extern "C" int rd_tree_attn_prepare(const int64_t* unpacker, const int64_t* pack
   const int n_counters = (int)rd::attn_counter_ints(batch, n);
 #define RD_LAUNCH_TP(T)                                                                               \
   do { rd::ScopedTiming rd_t("tree_prepare_kernel", s);                                               \
-    hipLaunchKernelGGL(tree_prepare_kernel<T>, grid, dim3(kThreads), 2 * batch * sizeof(int), s, unpacker, \
+    hipLaunchKernelGGL(tree_prepare_kernel<T>, grid, dim3(kThreads), 4 * batch * sizeof(int), s, unpacker, \
                        packed_token_indices, counts, reinterpret_cast<const T*>(padding_mask), pm_row_stride,  \
                        pm_pad_value, prev, batch, width * length, length, n, words, n_heads, compute_units(),  \
                        rd::kAttnChunk, max_splits, kv_row_shift, bits, plan, counters, n_counters, position_ids, \
