@@ -118,7 +118,7 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_ro
   // unless another size is at least 5 % better.  (Same box, eight rows of 500-2548 keys, 32
   // heads: 86 -> 67 us at 168 query rows, 63 -> 48 us at 88.)
   constexpr int kCands = 13, kMaxRows = 32, kMaxGroups = 32;
-  constexpr int kTile = 2, kFixed = 10, kSplit = 20, kMerge = 8;
+  constexpr int kTile = 2, kFixed = 10, kSplit = 16, kMerge = 8;
   __shared__ int s_est[kCands];
   __shared__ int s_plen[kCands][2 * kMaxRows], s_pcnt[kCands][2 * kMaxRows], s_load[kCands][kMaxGroups];
   __shared__ int s_sorted_len[kCands][2 * kMaxRows], s_sorted_cnt[kCands][2 * kMaxRows];

@@ -709,6 +709,12 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // key range as fp32 partials, counts itself in, and the last one to arrive merges the partials
   // of all of them (m in log2 units).  Nobody returns before the count: the barriers below are
   // reached by every wave of the workgroup.
+  // The partials cross from one XCD to another, whose L2s do not see each other's lines.  They are
+  // therefore stored and loaded with device-scope accesses (the sc1 bit: the store goes through
+  // this XCD's L2 to memory, the load does not take a line another XCD may have changed from its
+  // own L2), 16 bytes at a time.  A release fence before the count and an acquire fence behind it
+  // would do the same for ordinary accesses, but each works on the whole L2 of its XCD while the
+  // other workgroups stream through it: rows split four ways ran 8-19 % longer that way.
   const int64_t slot0 = ((int64_t)b * a.H + h) * a.max_splits;
   if (writer) {
     float* po = a.part_o + ((slot0 + split) * a.n_q + q_row) * kD + 4 * g;
@@ -717,28 +723,25 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         f32x4 w = {o[db][4 * i4 + 0], o[db][4 * i4 + 1], o[db][4 * i4 + 2], o[db][4 * i4 + 3]};
-        *reinterpret_cast<f32x4*>(po + 32 * db + 8 * i4) = w;
+        asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(po + 32 * db + 8 * i4), "v"(w) : "memory");
       }
     if (g == 0) {
       float* pm = a.part_ml + ((slot0 + split) * a.n_q + q_row) * 2;
-      pm[0] = m;
-      pm[1] = l;
+      const f32x2 ml = {m, l};
+      asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(pm), "v"(ml) : "memory");
     }
   }
-  // The barrier waits until the partial stores of every wave have left the compute unit; one
-  // wave then does the device-wide part for the whole workgroup: it makes the partials visible
-  // before the item is counted and, if the item is the last, drops stale lines before the others'
-  // partials are read.  (The fences work on the whole L2 of this XCD, so one per workgroup it is,
-  // not one per wave.)
+  // Every wave waits until its stores have arrived, the barrier collects the waves, and one lane
+  // counts the item in: whoever reads n_splits - 1 there knows that the partials of all the others
+  // are in memory.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   int* s_last = reinterpret_cast<int*>(smem);  // (the tile buffers are free by now)
   int32_t* counter = a.counters + ((int64_t)b * rd::kAttnMaxHeads + h) * q_tiles + q_tile;
   if (wave == 0) {
-    __threadfence();
     int last = 0;
     if (lane == 0) last = atomicAdd(counter, 1) == n_splits - 1;
     last = __builtin_amdgcn_readfirstlane(last);
-    if (last) __threadfence();
     if (lane == 0) *s_last = last;
   }
   __syncthreads();
@@ -762,9 +765,13 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       for (int j = 0; j < kPass; ++j) {
         const int q = q0 + kGroups * j < q_end ? q0 + kGroups * j : q_end - 1;  // clamped: loads stay unconditional
         const int64_t row = (slot0 + s) * a.n_q + q;
-        ml[j] = *reinterpret_cast<const f32x2*>(a.part_ml + row * 2);
-        po[j] = *reinterpret_cast<const f32x4*>(a.part_o + row * kD + dq);
+        asm volatile("global_load_dwordx2 %0, %1, off sc1" : "=v"(ml[j]) : "v"(a.part_ml + row * 2) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(po[j]) : "v"(a.part_o + row * kD + dq) : "memory");
       }
+      // (the compiler does not count these loads: one wait for all of them, tied to their registers)
+      static_assert(kPass == 8, "the wait below names eight register pairs");
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(ml[0]), "+v"(ml[1]), "+v"(ml[2]), "+v"(ml[3]), "+v"(ml[4]), "+v"(ml[5]), "+v"(ml[6]), "+v"(ml[7]));
+      asm volatile("" : "+v"(po[0]), "+v"(po[1]), "+v"(po[2]), "+v"(po[3]), "+v"(po[4]), "+v"(po[5]), "+v"(po[6]), "+v"(po[7]));
 #pragma unroll
       for (int j = 0; j < kPass; ++j) {
         const float m_new = fmaxf(mx[j], ml[j][0]);
