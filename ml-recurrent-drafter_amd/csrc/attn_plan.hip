@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kThreads) void mask_bits_kernel(
 // written before the call; the call begins with a barrier).  Whole workgroup of kThreads.
 // s_rows: 2 * B more ints of LDS (the rows' split counts and first items; global memory is only
 // written here, never read back: a serial loop over rows would pay a trip to memory per row).
-__device__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_rows, int B, int n_q, int kv_len,
+__device__ __forceinline__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_rows, int B, int n_q, int kv_len,
                            int words, int min_chunk, int max_splits, int n_heads, int n_cu,
                            const int32_t* __restrict__ kv_shift, int32_t* __restrict__ plan,
                            int32_t* __restrict__ counters, int n_counters) {
@@ -69,7 +69,7 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_ro
   int32_t* per_row = plan + RD_PLAN_HDR;
   int* s_splits = s_rows;
   int* s_first_item = s_rows + B;
-  auto begin_of = [&](int b) { return (s_key_min[b] / 64) * 64; };
+  auto begin_of = [&](int b) __attribute__((always_inline)) { return (s_key_min[b] / 64) * 64; };
   int32_t* items = plan + RD_PLAN_HDR + 4 * B;
   __syncthreads();
   for (int b = threadIdx.x; b < B; b += kThreads) {
@@ -103,7 +103,7 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_ro
   // an item may run an eighth over the chunk: a row a little longer than it stays whole (cutting
   // off a short remainder would cost it the partials, the fences and the merge, and would send
   // the remainders into a second round of items behind the first)
-  auto splits_of = [&](int live, int chunk) {
+  auto splits_of = [&](int live, int chunk) __attribute__((always_inline)) {
     const int splits = (live + chunk - 1 - chunk / 8) / chunk;
     return splits < 1 ? 1 : (splits > max_splits ? max_splits : splits);
   };
@@ -122,21 +122,18 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_ro
   __shared__ int s_est[kCands];
   __shared__ int s_plen[kCands][2 * kMaxRows], s_pcnt[kCands][2 * kMaxRows], s_load[kCands][kMaxGroups];
   __shared__ int s_sorted_len[kCands][2 * kMaxRows], s_sorted_cnt[kCands][2 * kMaxRows];
-  auto candidate = [&](int c) {
+  auto candidate = [&](int c) __attribute__((always_inline)) {
     return (int)((long long)s_share * (8 + c) / 8) / 64 * 64;  // share * (1 .. 2.5): smaller ones only split more
   };
-  if (s_search && threadIdx.x < kCands) {
-    const int c = threadIdx.x, chunk = candidate(c);
-    const int q_tiles = n_q <= 256 ? 1 : (n_q + 255) / 256;
-    const long long per_item = (long long)n_heads * q_tiles;  // workgroups of one item
-    int groups = per_item >= n_cu ? 1 : (int)(n_cu / per_item);
-    groups = groups > kMaxGroups ? kMaxGroups : groups;
-    const int rounds_per_item = per_item >= n_cu ? (int)((per_item + n_cu - 1) / n_cu) : 1;
-    int* plen = s_plen[c];
-    int* pcnt = s_pcnt[c];
-    int n_classes = 0;
-    bool any_split = false;
-    for (int b = 0; b < B; ++b) {  // every row: splits - 1 pieces of `per` keys and the rest
+  // Three short phases instead of one thread per candidate walking through everything: (1) a
+  // thread per (candidate, row) forms the row's two classes of pieces (whole pieces, and the
+  // rest) at fixed slots, (2) a thread per (candidate, class) finds the class's rank by length,
+  // (3) a thread per candidate deals the pieces out, longest first.
+  __shared__ int s_any_split[kCands];
+  if (s_search) {
+    for (int i = threadIdx.x; i < kCands; i += kThreads) s_any_split[i] = 0;
+    for (int idx = threadIdx.x; idx < kCands * B; idx += kThreads) {
+      const int c = idx / B, b = idx - c * B, chunk = candidate(c);
       const int live = s_key_end[b] - begin_of(b);
       const int splits = splits_of(live, chunk);
       int per = (live + splits - 1) / splits;
@@ -144,38 +141,51 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_ro
       const int whole = per > 0 ? live / per : 0;  // pieces of full length
       const int rest = live - whole * per;
       const int extra = splits > 1 ? kSplit : 0;
-      any_split |= splits > 1;
-      if (whole > 0) { plen[n_classes] = ((per + 63) / 64) * kTile + kFixed + extra; pcnt[n_classes++] = whole; }
-      if (rest > 0) { plen[n_classes] = ((rest + 63) / 64) * kTile + kFixed + extra; pcnt[n_classes++] = 1; }
+      s_plen[c][2 * b] = whole > 0 ? ((per + 63) / 64) * kTile + kFixed + extra : 0;
+      s_pcnt[c][2 * b] = whole;
+      s_plen[c][2 * b + 1] = rest > 0 ? ((rest + 63) / 64) * kTile + kFixed + extra : 0;
+      s_pcnt[c][2 * b + 1] = rest > 0 ? 1 : 0;
+      if (splits > 1) s_any_split[c] = 1;  // (every writer writes the same value)
     }
-    // longest first: every class finds its rank among the others (independent reads, where an
-    // insertion sort would be a chain of dependent ones)
-    int* slen = s_sorted_len[c];
-    int* scnt = s_sorted_cnt[c];
-    for (int i = 0; i < n_classes; ++i) {
+  }
+  __syncthreads();
+  if (s_search) {
+    const int n_classes = 2 * B;
+    for (int idx = threadIdx.x; idx < kCands * n_classes; idx += kThreads) {
+      const int c = idx / n_classes, i = idx - c * n_classes;
+      const int* plen = s_plen[c];
       const int l = plen[i];
       int rank = 0;
       for (int j = 0; j < n_classes; ++j) rank += plen[j] > l || (plen[j] == l && j < i);
-      slen[rank] = l;
-      scnt[rank] = pcnt[i];
+      s_sorted_len[c][rank] = l;
+      s_sorted_cnt[c][rank] = s_pcnt[c][i];
     }
+  }
+  __syncthreads();
+  if (s_search && threadIdx.x < kCands) {
+    const int c = threadIdx.x;
+    const int q_tiles = n_q <= 256 ? 1 : (n_q + 255) / 256;
+    const long long per_item = (long long)n_heads * q_tiles;  // workgroups of one item
+    int groups = per_item >= n_cu ? 1 : (int)(n_cu / per_item);
+    groups = groups > kMaxGroups ? kMaxGroups : groups;
+    const int rounds_per_item = per_item >= n_cu ? (int)((per_item + n_cu - 1) / n_cu) : 1;
+    const int* slen = s_sorted_len[c];
+    const int* scnt = s_sorted_cnt[c];
+    int* load = s_load[c];
+    for (int g = 0; g < groups; ++g) load[g] = 0;
     int end = 0;
-    {
-      int* load = s_load[c];
-      for (int g = 0; g < groups; ++g) load[g] = 0;
-      for (int i = 0; i < n_classes; ++i)
-        for (int k = 0; k < scnt[i]; ++k) {
-          int least = 0, least_load = load[0];
-          for (int g = 1; g < groups; ++g) {
-            const int l = load[g];
-            if (l < least_load) { least = g; least_load = l; }
-          }
-          least_load += slen[i] * rounds_per_item;
-          load[least] = least_load;
-          end = least_load > end ? least_load : end;
+    for (int i = 0; i < 2 * B && slen[i] > 0; ++i)
+      for (int k = 0; k < scnt[i]; ++k) {
+        int least = 0, least_load = load[0];
+        for (int g = 1; g < groups; ++g) {
+          const int l = load[g];
+          if (l < least_load) { least = g; least_load = l; }
         }
-    }
-    s_est[c] = end + (any_split ? kMerge : 0);
+        least_load += slen[i] * rounds_per_item;
+        load[least] = least_load;
+        end = least_load > end ? least_load : end;
+      }
+    s_est[c] = end + (s_any_split[c] ? kMerge : 0);
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -205,7 +215,7 @@ __device__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_ro
   __syncthreads();
   const int n_items = s_n_items;
   // every item computes its own extent and its rank (longest first, ties by index)
-  auto extent = [&](int it, int& b, int& s, int& lo, int& hi) {
+  auto extent = [&](int it, int& b, int& s, int& lo, int& hi) __attribute__((always_inline)) {
     b = 0;
     while (b + 1 < B && s_first_item[b + 1] <= it) ++b;
     s = it - s_first_item[b];
