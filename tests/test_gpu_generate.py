@@ -84,3 +84,24 @@ def test_generate_matches_torch_restatement_on_gpu_bigger_model():
     steps, _ = _run(llm, drafter, ids, 300 + 12, 12, 5)
     want = [t.cpu().tolist() for t, _ in P.generate_greedy(llm, drafter, ids.cuda(), 300 + 12, 12, 5, pad=0, eos=None)]
     assert steps == want
+
+
+@pytest.mark.parametrize("batch,W,L,prompt_len,left_pads,markov", [
+    (1, 1, 2, 5, [0], True),          # the smallest beam: one candidate of one drafted token
+    (1, 64, 5, 12, [3], False),       # the widest beam the kernels take, more than the top-50 filter keeps
+    (3, 2, 6, 7, [0, 6, 2], True),    # a row that is almost all padding; beams longer than wide
+    (5, 7, 3, 1, [0, 0, 0, 0, 0], True),  # one-token prompts
+    (2, 45, 5, 40, [0, 17], True),    # the benchmark's beam shape
+])
+def test_generate_edge_shapes_match_the_restatement(batch, W, L, prompt_len, left_pads, markov):
+    """Greedy token streams at the edges of the shape space (float32 tiny models) against the torch
+    restatement on the same GPU, step by step; the last step must be cut at max_length."""
+    seed = 100 + batch + W
+    llama_sd, drafter_sd = tm.markov(seed) if markov else (tm.draw(tm.llama_shapes(), seed), tm.draw(tm.drafter_shapes(), seed + 1000))
+    llm, drafter = _models(llama_sd, drafter_sd)
+    ids = tm.prompt(batch, prompt_len, tm.LLAMA["vocab_size"], seed, left_pads)
+    max_length = prompt_len + 11
+    want = [t.cpu().tolist() for t, _ in P.generate_greedy(llm, drafter, ids.cuda(), max_length, W, L, pad=0, eos=None)]
+    steps, _ = _run(llm, drafter, ids, max_length, W, L)
+    assert steps == want
+    assert len(steps[-1][0]) == max_length and all(len(s[0]) <= max_length for s in steps)
