@@ -53,3 +53,55 @@ def test_cpu_tensors_are_refused():
 
     with pytest.raises(RuntimeError, match="GPU"):
         tree_attention.pack(torch.zeros((1, 2, 3), dtype=torch.long), torch.ones((1, 2), dtype=torch.long))
+
+
+def test_host_side_checks_of_the_attention_and_probe_entry_points():
+    """What the library decides on the host, before any GPU call: which shapes the one-kernel
+    RoPE + attention entry point takes, the size of the attention workspace (closed form), and the
+    argument errors of entry points whose checks come first (no kernel is launched here)."""
+    from recurrent_drafting_amd import _hip
+
+    lib = _hip.lib()
+    BF16, F16, F32 = _hip.RD_BF16, _hip.RD_F16, _hip.RD_F32
+    ok = lib.rd_rope_verify_attention_eligible
+    assert ok(BF16, 32, 128, 168) == 1 and ok(BF16, 128, 128, 256) == 1 and ok(BF16, 1, 128, 1) == 1
+    assert ok(F16, 32, 128, 168) == 0 and ok(F32, 32, 128, 168) == 0      # bf16 only
+    assert ok(BF16, 32, 64, 168) == 0 and ok(BF16, 32, 256, 168) == 0     # head_dim 128 only
+    assert ok(BF16, 129, 128, 168) == 0                                   # the arrival counters are laid out for 128 heads
+    assert ok(BF16, 32, 128, 257) == 0 and ok(BF16, 32, 128, 0) == 0      # a prompt goes through the two kernels
+
+    def align(x):
+        return (x + 255) // 256 * 256
+
+    for batch, heads, n_q, kv, d in [(8, 32, 168, 2716, 128), (1, 1, 1, 1, 128), (3, 5, 40, 512, 128), (2, 8, 300, 513, 64)]:
+        slots = batch * heads * ((kv + 511) // 512)
+        assert lib.rd_attention_workspace_bytes(batch, heads, n_q, kv, d) == align(slots * n_q * d * 4) + align(slots * n_q * 2 * 4)
+    assert lib.rd_attention_workspace_bytes(0, 32, 168, 2716, 128) == 0
+
+    # rd_verify_attention: sizes, head grouping, head_dim, null pointers
+    nulls = [None] * 8
+    assert lib.rd_verify_attention(*nulls, BF16, 0, 32, 32, 168, 700, 128, 1.0, None, None, None, 0, 0, None, None) == -1
+    assert b"bad sizes" in lib.rd_last_error()
+    assert lib.rd_verify_attention(*nulls, BF16, 8, 32, 5, 168, 700, 128, 1.0, None, None, None, 0, 0, None, None) == -1
+    assert b"multiple" in lib.rd_last_error()
+    assert lib.rd_verify_attention(*nulls, BF16, 8, 32, 32, 168, 700, 512, 1.0, None, None, None, 0, 0, None, None) == -2
+    assert lib.rd_verify_attention(*nulls, BF16, 8, 32, 32, 168, 700, 128, 1.0, None, None, None, 0, 0, None, None) == -1
+    assert b"null" in lib.rd_last_error()
+
+    # rd_stream_tiles_probe: host buffers stand in for device pointers, every call returns before a launch
+    buf = (ctypes.c_char * 4096)()
+    base = (ctypes.addressof(buf) + 15) // 16 * 16
+    k, v, sink = ctypes.c_void_p(base), ctypes.c_void_p(base + 1024), ctypes.c_void_p(base + 2048)
+    assert lib.rd_stream_tiles_probe(None, v, 32768, 1, 1, 1, sink, None) == -1
+    assert lib.rd_stream_tiles_probe(k, v, 32768, 0, 1, 1, sink, None) == -1
+    assert lib.rd_stream_tiles_probe(k, v, 16, 1, 8, 1, sink, None) == -1            # a slab too small for its tiles
+    assert lib.rd_stream_tiles_probe(ctypes.c_void_p(base + 4), v, 1 << 20, 1, 8, 1, sink, None) == -1  # alignment
+    assert lib.rd_stream_tiles_probe(k, v, 1 << 20, 1, 8, 3, sink, None) == -2       # depth 1, 2 or 4
+    assert b"depth" in lib.rd_last_error()
+
+    # rd_beam_topk_static: what the built-in scratch cannot hold is refused before the scratch is looked up
+    args = [None, BF16, 0, 0]
+    rest = [32000, None, 50, 0.0, None, 0, None, None, None, None, None, 0, 0, None]
+    assert lib.rd_beam_topk_static(*args, 0, 45, *rest) == -1
+    assert lib.rd_beam_topk_static(*args, 128, 45, *rest) == -2 and b"workspace" in lib.rd_last_error()  # 5760 rows > 4096
+    assert lib.rd_beam_topk_static(*args, 8, 65, *rest) == -2                                            # width > 64
