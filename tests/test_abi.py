@@ -88,7 +88,19 @@ def test_host_side_checks_of_the_attention_and_probe_entry_points():
     assert lib.rd_verify_attention(*nulls, BF16, 8, 32, 32, 168, 700, 128, 1.0, None, None, None, 0, 0, None, None) == -1
     assert b"null" in lib.rd_last_error()
 
-    # rd_stream_tiles_probe: host buffers stand in for device pointers, every call returns before a launch
+    # rd_beam_topk_static: what the built-in scratch cannot hold is refused before the scratch is looked up
+    args = [None, BF16, 0, 0]
+    rest = [32000, None, 50, 0.0, None, 0, None, None, None, None, None, 0, 0, None]
+    assert lib.rd_beam_topk_static(*args, 0, 45, *rest) == -1
+    assert lib.rd_beam_topk_static(*args, 128, 45, *rest) == -2 and b"workspace" in lib.rd_last_error()  # 5760 rows > 4096
+    assert lib.rd_beam_topk_static(*args, 8, 65, *rest) == -2                                            # width > 64
+
+    # rd_stream_tiles_probe: every call returns before a launch; host buffers stand in for the
+    # device pointers, so on a machine with a GPU this part is left out (its GPU test covers it)
+    import torch
+
+    if torch.cuda.device_count() > 0:
+        return
     buf = (ctypes.c_char * 4096)()
     base = (ctypes.addressof(buf) + 15) // 16 * 16
     k, v, sink = ctypes.c_void_p(base), ctypes.c_void_p(base + 1024), ctypes.c_void_p(base + 2048)
@@ -98,10 +110,3 @@ def test_host_side_checks_of_the_attention_and_probe_entry_points():
     assert lib.rd_stream_tiles_probe(ctypes.c_void_p(base + 4), v, 1 << 20, 1, 8, 1, sink, None) == -1  # alignment
     assert lib.rd_stream_tiles_probe(k, v, 1 << 20, 1, 8, 3, sink, None) == -2       # depth 1, 2 or 4
     assert b"depth" in lib.rd_last_error()
-
-    # rd_beam_topk_static: what the built-in scratch cannot hold is refused before the scratch is looked up
-    args = [None, BF16, 0, 0]
-    rest = [32000, None, 50, 0.0, None, 0, None, None, None, None, None, 0, 0, None]
-    assert lib.rd_beam_topk_static(*args, 0, 45, *rest) == -1
-    assert lib.rd_beam_topk_static(*args, 128, 45, *rest) == -2 and b"workspace" in lib.rd_last_error()  # 5760 rows > 4096
-    assert lib.rd_beam_topk_static(*args, 8, 65, *rest) == -2                                            # width > 64
