@@ -81,3 +81,69 @@ def test_rope_and_layer_kernel_limits(lib):
     assert norm(2, 8192) == EINVAL and norm(2, 8196) == ELIMIT        # float32 rows of at most 8192
     assert norm(0, 4100) == ELIMIT and norm(2, 4098) == ELIMIT        # whole 16-byte vectors only
     assert norm(0, 4096, rows=0) == EINVAL and b"bad sizes" in lib.rd_last_error()
+
+
+def test_verification_and_acceptance_limits(lib):
+    def stats(vocab=32000, top_k=50, rows=1448):
+        return lib.rd_verify_row_stats(None, 0, vocab, rows, vocab, top_k, -1e4, 1.0, None, 0, None)
+
+    assert stats() == EINVAL and b"null" in lib.rd_last_error()
+    assert stats(vocab=65536) == EINVAL and stats(vocab=65537) == ELIMIT
+    assert stats(top_k=512) == EINVAL and stats(top_k=513) == ELIMIT
+    assert stats(rows=0) == EINVAL
+
+    def greedy(batch=8, width=45, length=5):
+        return lib.rd_accept_greedy(None, None, 0, None, batch, width, length, None, None, None, None, None)
+
+    assert greedy() == EINVAL and b"null" in lib.rd_last_error()
+    assert greedy(width=65535) == EINVAL and greedy(width=65536) == ELIMIT
+    assert greedy(length=32767) == EINVAL and greedy(length=32768) == ELIMIT
+    assert greedy(batch=0) == EINVAL
+
+    def sample(batch=8, width=45, length=5, vocab=32000):
+        return lib.rd_accept_sample(None, None, None, None, 0, None, None, 0, None, 1.0, None, None, None, batch, width,
+                                    length, vocab, None, None, None)
+
+    assert sample() == EINVAL and b"null" in lib.rd_last_error()
+    assert sample(length=1) == EINVAL and b"null" not in lib.rd_last_error()   # nothing drafted: nothing to accept
+    assert sample(width=65536) == ELIMIT
+
+    def argmax(rows=1448, vocab=32000, stride=32000):
+        return lib.rd_argmax_rows(None, 0, rows, vocab, stride, None, None)
+
+    assert argmax() == EINVAL and b"null" in lib.rd_last_error()
+    assert argmax(stride=31999) == EINVAL and b"null" not in lib.rd_last_error()
+    assert argmax(rows=1 << 31) == ELIMIT
+
+
+def test_mask_and_row_movement_limits(lib):
+    def causal(batch=8, kv_len=500, query_len=500):
+        return lib.rd_causal_mask(None, 8, kv_len, batch, kv_len, query_len, None, None)
+
+    assert causal() == EINVAL and b"null" in lib.rd_last_error()
+    assert causal(query_len=501) == EINVAL and b"null" not in lib.rd_last_error()   # more queries than keys
+    assert causal(batch=65536) == ELIMIT
+
+    def tree_mask(batch=8, width=45, length=5, prev=2548):
+        return lib.rd_tree_mask(None, None, None, None, 8, prev, 0, prev, batch, width, length, None, None)
+
+    assert tree_mask() == EINVAL and b"null" in lib.rd_last_error()
+    assert tree_mask(length=65, width=8) == ELIMIT and tree_mask(width=1024, length=5) == ELIMIT
+    assert tree_mask(batch=65536) == ELIMIT
+    assert tree_mask(prev=-1) == EINVAL
+
+    def unpack(batch=8, n_out=225, n_src=168, row_bytes=8192):
+        return lib.rd_unpack_rows(None, n_src * row_bytes, row_bytes, None, n_out, batch, n_out, n_src, None,
+                                  n_out * row_bytes, row_bytes, None)
+
+    assert unpack() == EINVAL and b"null" in lib.rd_last_error()
+    assert unpack(batch=65536) == ELIMIT
+    assert unpack(row_bytes=0) == EINVAL and b"bad sizes" in lib.rd_last_error()
+
+    def silu_mul(dtype=0, cols=11008, rows=1448):
+        return lib.rd_silu_mul(None, None, 2 * cols, None, cols, dtype, rows, cols, None)
+
+    assert silu_mul() == EINVAL and b"null" in lib.rd_last_error()
+    assert silu_mul(cols=11004) == ELIMIT and silu_mul(dtype=2, cols=11006) == ELIMIT   # whole 16-byte vectors
+    assert silu_mul(dtype=2, cols=11004) == EINVAL
+    assert silu_mul(dtype=5) == EINVAL and b"dtype" in lib.rd_last_error()
