@@ -40,7 +40,11 @@ typedef enum { RD_BF16 = 0, RD_F16 = 1, RD_F32 = 2 } rd_dtype;
 
 #define RD_API __attribute__((visibility("default")))
 
-/* Library version (major*10000 + minor*100 + patch). */
+/* Version of this interface: changes whenever an entry point's arguments, the layout of a buffer
+ * that crosses it (the attention plan, the realignment plan) or a workspace size changes.  A caller
+ * compiled against this header compares rd_version() with RD_ABI_VERSION before its first call, so
+ * that a stale build of the library is refused instead of being called with other arguments. */
+#define RD_ABI_VERSION 103
 RD_API int rd_version(void);
 /* Message of the last failed call on this thread ("" if none). */
 RD_API const char* rd_last_error(void);
@@ -63,14 +67,6 @@ RD_API int rd_timing_sample(int every);
  * kernel trace does not.  Synchronises the stream. */
 RD_API int rd_timing_null_kernel_us(int launches, void* stream, float* avg_us);
 RD_API int rd_timing_collect(char* out, size_t out_bytes);
-/* Yardstick for the verification attention's memory side (no counterpart in the reference; used
- * by kernel_bench.py): `slabs` workgroups of 512 threads each stream `tiles` tiles of 64 rows x
- * 256 bytes from their slab of k and of v (slab i begins at i * slab_bytes), `depth` (1, 2 or 4)
- * tiles ahead in registers, through LDS and a barrier per tile -- the loads, staging and barrier
- * of rd_verify_attention's tile loop without its arithmetic.  sink: slabs * 512 uint32, written
- * so that the loads cannot be dropped.  Timed under the name "stream_tiles_kernel". */
-RD_API int rd_stream_tiles_probe(const void* k, const void* v, int64_t slab_bytes, int slabs, int tiles,
-                                 int depth, void* sink, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Draft beams -> prefix tree -> packed tokens.

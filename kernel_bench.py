@@ -263,22 +263,48 @@ def case_slope(rows, reps):
     series("kv_append, 8 layers x", "kv_append_kernel", append)
 
 
+_bench_lib = None
+
+
+def bench_library():
+    """The bench-only shared object (ml-recurrent-drafter_amd/bench_csrc, built by build_hip.py beside
+    the product library but not part of it or of its C ABI)."""
+    global _bench_lib
+    if _bench_lib is None:
+        import ctypes as C
+
+        path = os.path.join(HERE, "ml-recurrent-drafter_amd", "bench_csrc", "libredrafter_bench.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python ml-recurrent-drafter_amd/build_hip.py`")
+        lib = C.CDLL(path)
+        lib.bench_stream_tiles.restype = C.c_int
+        lib.bench_stream_tiles.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                           C.c_int, C.c_void_p, C.POINTER(C.c_float)]
+        _bench_lib = lib
+    return _bench_lib
+
+
 def case_stream(rows, reps):
     """What the memory system delivers to the attention's access pattern (a K and a V slab per
     (batch row, head), 64-row tiles, one 512-thread workgroup per compute unit) when the tile loop
-    does nothing but load, stage and meet at its barrier: rd_stream_tiles_probe.  The slabs are those
+    does nothing but load, stage and meet at its barrier: bench_stream_tiles.  The slabs are those
     of a cache of 2560 + 128 rows, 690 MB together: more than the 256 MB memory-side cache."""
+    import ctypes as C
+
     slabs, max_len = B * H, 2560 + 128
     k = torch.randn(slabs, max_len, D, device="cuda").to(torch.bfloat16)
     v = torch.randn(slabs, max_len, D, device="cuda").to(torch.bfloat16)
     sink = torch.empty(slabs * 512, dtype=torch.int32, device="cuda")
-    lib = _hip.lib()
+    lib = bench_library()
     for keys in (640, 1536, 2560):
         tiles = keys // 64
         for depth in (1, 2, 4):
-            fn = lambda: _hip.check(lib.rd_stream_tiles_probe(_hip.ptr(k), _hip.ptr(v), max_len * D * 2, slabs, tiles, depth,
-                                                              _hip.ptr(sink), _hip.stream()))
-            kk = timed(fn, reps)
+            us = C.c_float(0.0)
+            for n in (3, reps):  # warm-up, then the timed launches
+                rc = lib.bench_stream_tiles(_hip.ptr(k), _hip.ptr(v), max_len * D * 2, slabs, tiles, depth, _hip.ptr(sink), n,
+                                            _hip.stream(), C.byref(us))
+                assert rc == 0, rc
+            kk = {"stream_tiles_kernel": (1, float(us.value))}
             nbytes = 2 * slabs * tiles * 64 * D * 2
             report(rows, f"stream K/V tiles only, {keys} keys per row, {depth} tile(s) ahead", kk,
                    {"stream_tiles_kernel": nbytes}, {"stream_tiles_kernel": "GB/s"})

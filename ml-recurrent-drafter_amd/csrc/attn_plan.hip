@@ -5,6 +5,7 @@
 //                      of left padding or behind the row's last tree slot are never loaded), split
 //                      of that span into near-equal chunks, and the chunk list sorted longest-first
 #include "attn_plan.h"
+#include "rd_common.h"
 
 namespace {
 
@@ -69,7 +70,7 @@ __device__ __forceinline__ void build_plan(const int* s_key_min, const int* s_ke
   int32_t* per_row = plan + RD_PLAN_HDR;
   int* s_splits = s_rows;
   int* s_first_item = s_rows + B;
-  auto begin_of = [&](int b) __attribute__((always_inline)) { return (s_key_min[b] / 64) * 64; };
+  auto begin_of = [&](int b) __attribute__((always_inline)) { return rd::plan_begin(s_key_min[b]); };
   int32_t* items = plan + RD_PLAN_HDR + 4 * B;
   __syncthreads();
   for (int b = threadIdx.x; b < B; b += kThreads) {
@@ -80,14 +81,10 @@ __device__ __forceinline__ void build_plan(const int* s_key_min, const int* s_ke
   __shared__ int s_share;
   __shared__ bool s_search;
   if (threadIdx.x == 0) {
-    // Keys per work item, first guess: one compute unit's even share of all (row, head) work, but
-    // never below min_chunk.  Equal rows on a machine with batch*heads == compute units are then
-    // not split at all (no partials to merge).
+    // keys per work item, first guess: one compute unit's even share (attn_plan.h)
     long long total = 0;
     for (int b = 0; b < B; ++b) total += s_key_end[b] - begin_of(b);
-    long long share = (total * n_heads + n_cu - 1) / n_cu;
-    share = (share + 63) / 64 * 64;
-    s_share = (int)(share > min_chunk ? share : min_chunk);
+    s_share = rd::plan_share(total, n_heads, n_cu, min_chunk);
     // The search below is for ragged rows: with no row split at the share and one workgroup per
     // compute unit at most (every decode step of equal rows) the share stands.  It walks over
     // every piece of every candidate: only where that is a short walk.
@@ -95,18 +92,12 @@ __device__ __forceinline__ void build_plan(const int* s_key_min, const int* s_ke
     const int q_tiles = n_q <= 256 ? 1 : (n_q + 255) / 256;
     bool split_at_share = false;
     for (int b = 0; b < B && !split_at_share; ++b)
-      split_at_share = (s_key_end[b] - begin_of(b) + s_share - 1 - s_share / 8) / s_share > 1;
+      split_at_share = rd::plan_splits(s_key_end[b] - begin_of(b), s_share, max_splits) > 1;
     const bool one_round = (long long)B * n_heads * q_tiles <= n_cu;
     s_search = B <= 32 && (total / smallest + B) * 32 <= 8192 && !(one_round && !split_at_share);
   }
   __syncthreads();
-  // an item may run an eighth over the chunk: a row a little longer than it stays whole (cutting
-  // off a short remainder would cost it the partials, the fences and the merge, and would send
-  // the remainders into a second round of items behind the first)
-  auto splits_of = [&](int live, int chunk) __attribute__((always_inline)) {
-    const int splits = (live + chunk - 1 - chunk / 8) / chunk;
-    return splits < 1 ? 1 : (splits > max_splits ? max_splits : splits);
-  };
+  auto splits_of = [&](int live, int chunk) __attribute__((always_inline)) { return rd::plan_splits(live, chunk, max_splits); };
   // Ragged rows: the even share is only a guess, because the items run in rounds (every compute
   // unit holds one workgroup) and each costs a fixed part on top of its tiles.  A few chunk sizes
   // from the share upwards are therefore tried on a model of the launch, one thread each: the pieces of
@@ -117,13 +108,13 @@ __device__ __forceinline__ void build_plan(const int* s_key_min, const int* s_ke
   // merge kMerge at the end, all in half tiles, fitted to measured launches.  The share stands
   // unless another size is at least 5 % better.  (Same box, eight rows of 500-2548 keys, 32
   // heads: 86 -> 67 us at 168 query rows, 63 -> 48 us at 88.)
-  constexpr int kCands = 13, kMaxRows = 32, kMaxGroups = 32;
+  constexpr int kCands = rd::kPlanCandidates, kMaxRows = 32, kMaxGroups = 32;
   constexpr int kTile = 2, kFixed = 10, kSplit = 16, kMerge = 8;
   __shared__ int s_est[kCands];
   __shared__ int s_plen[kCands][2 * kMaxRows], s_pcnt[kCands][2 * kMaxRows], s_load[kCands][kMaxGroups];
   __shared__ int s_sorted_len[kCands][2 * kMaxRows], s_sorted_cnt[kCands][2 * kMaxRows];
   auto candidate = [&](int c) __attribute__((always_inline)) {
-    return (int)((long long)s_share * (8 + c) / 8) / 64 * 64;  // share * (1 .. 2.5): smaller ones only split more
+    return rd::plan_candidate(s_share, c);
   };
   // Three short phases instead of one thread per candidate walking through everything: (1) a
   // thread per (candidate, row) forms the row's two classes of pieces (whole pieces, and the
@@ -136,8 +127,7 @@ __device__ __forceinline__ void build_plan(const int* s_key_min, const int* s_ke
       const int c = idx / B, b = idx - c * B, chunk = candidate(c);
       const int live = s_key_end[b] - begin_of(b);
       const int splits = splits_of(live, chunk);
-      int per = (live + splits - 1) / splits;
-      per = (per + 63) / 64 * 64;
+      const int per = rd::plan_per(live, splits);
       const int whole = per > 0 ? live / per : 0;  // pieces of full length
       const int rest = live - whole * per;
       const int extra = splits > 1 ? kSplit : 0;
@@ -219,14 +209,7 @@ __device__ __forceinline__ void build_plan(const int* s_key_min, const int* s_ke
     b = 0;
     while (b + 1 < B && s_first_item[b + 1] <= it) ++b;
     s = it - s_first_item[b];
-    const int begin = begin_of(b), splits = s_splits[b], end = s_key_end[b];
-    const int live = end - begin;
-    int per = (live + splits - 1) / splits;
-    per = (per + 63) / 64 * 64;
-    lo = begin + s * per;
-    hi = lo + per;
-    lo = lo < end ? lo : end;
-    hi = hi < end ? hi : end;
+    rd::plan_extent(begin_of(b), s_key_end[b], s_splits[b], s, &lo, &hi);
   };
   const bool sorted = n_items <= rd::kAttnSortLimit;
   if (sorted) {

@@ -137,7 +137,7 @@ __global__ __launch_bounds__(THREADS) void beam_row_kernel(
   int32_t* c_tok = cand_tok + (int64_t)row * W;
   // (a few more maxima than k_eff: the k-th largest key then sits well above the pivot's key, and
   // a tie between the two, which costs the slow path, takes that many equal values in a row)
-  const float pivot = row_pivot<THREADS, 8 * (sizeof(T) < 4 ? sizeof(T) : 4)>(tmax, k_eff + kPivotMargin < THREADS ? k_eff + kPivotMargin : THREADS, sh);
+  const float pivot = row_pivot<THREADS, Num<T>::kValueBits>(tmax, k_eff + kPivotMargin < THREADS ? k_eff + kPivotMargin : THREADS, sh);
 
   // ---- candidates: entries >= pivot, keyed by their value after the max subtraction ------------
   // t(x) = round_T(x - max) is monotone, so the k-th largest t comes from the list; an entry

@@ -135,5 +135,5 @@ extern "C" int rd_timing_collect(char* out, size_t out_bytes) {
   return RD_OK;
 }
 
-extern "C" int rd_version(void) { return 100; }
+extern "C" int rd_version(void) { return RD_ABI_VERSION; }
 extern "C" const char* rd_last_error(void) { return rd::error_buffer(); }

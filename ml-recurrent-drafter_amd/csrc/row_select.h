@@ -19,15 +19,21 @@ constexpr int kCap = 2048;  // LDS candidate list
 constexpr int kPivotMargin = 16;  // thread maxima taken beyond k when the pivot is chosen
 
 template <typename T> struct Num;
+// kValueBits: the leading bits of the float that can differ between two values of the type (the
+// rest are zero): bf16 is the upper half of a float; a half has 10 mantissa bits behind the float's
+// sign and 8 exponent bits (its subnormals become normal floats of at most 10 mantissa bits).
 template <> struct Num<float> {
+  static constexpr int kValueBits = 32;
   static __device__ float load(const float* p) { return *p; }
   static __device__ float round(float v) { return v; }
 };
 template <> struct Num<__hip_bfloat16> {
+  static constexpr int kValueBits = 16;
   static __device__ float load(const __hip_bfloat16* p) { return __bfloat162float(*p); }
   static __device__ float round(float v) { return __bfloat162float(__float2bfloat16(v)); }
 };
 template <> struct Num<__half> {
+  static constexpr int kValueBits = 19;
   static __device__ float load(const __half* p) { return __half2float(*p); }
   static __device__ float round(float v) { return __half2float(__float2half(v)); }
 };
@@ -200,8 +206,9 @@ __device__ inline void load_row(const T* __restrict__ x_row, int V, float (&x)[I
 // compare, one ballot and one scalar population count -- no LDS traffic, no cross-lane reductions
 // (taking the maxima out one by one, r rounds of wave reductions, cost 2.4 us of the 9 us a quarter
 // row took; ranking all maxima against each other through LDS was bound by the LDS bandwidth once
-// eight workgroups shared a compute unit).  VALUE_BITS: 16 for bf16/fp16 data (the low half of the
-// float is zero), 32 otherwise.
+// eight workgroups shared a compute unit).  VALUE_BITS: Num<T>::kValueBits, the leading bits of the
+// float in which two values of the row's type can differ (with fewer bits the result would still
+// be a valid, only lower, pivot: longer candidate lists).
 template <int THREADS, int VALUE_BITS, typename SH>
 __device__ inline float row_pivot(float tmax, int k_eff, SH& sh) {
   constexpr int WAVES = THREADS / 64;

@@ -29,9 +29,14 @@
 
 #include <type_traits>
 
+#include "attn_addr.h"
 #include "attn_plan.h"
+#include "rd_common.h"
 
 namespace {
+
+// tile sizes, wave layouts, loader roles and every index formula of the MFMA kernel (attn_addr.h)
+using namespace rd::attn;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
@@ -94,41 +99,7 @@ __device__ inline float rope_hi(float x1, float x2, float c, float s) {
 // ---------------------------------------------------------------------------------------------
 // MFMA kernel
 // ---------------------------------------------------------------------------------------------
-constexpr int kD = 128;
-constexpr int kTile = 64;                  // keys per tile
-constexpr int kWaves = 8;
-constexpr int kMfmaThreads = kWaves * 64;  // 512
-// How the 8 waves of a workgroup share its query rows (blocks of 32) and the 64 keys of a tile.
-// A wave is either FULL (it takes both 32-key units of every tile for its row block) or a HALF (it
-// takes one unit; two halves share a row block, each with its own running maximum, sum and
-// accumulators, merged through LDS at the end).  Wave w runs on SIMD w % 4, so the layouts spread
-// the units of a tile evenly over the SIMDs:
-//   kSplit  <= 128 rows  4 blocks, all halves (w, w+4)                      2 units per SIMD
-//   kMix5   <= 160 rows  blocks 0,1 full (w0,w1); 2,3,4 halves (w2+w6, w3+w7, w4+w5)   3,3,2,2
-//   kMix6   <= 192 rows  blocks 0-3 full (w0-w3); 4,5 halves (w4+w5, w6+w7)            3 each
-//   kFull   <= 256 rows  8 blocks, all full                                 4 units per SIMD
-// Without halves, a workgroup with few rows would leave waves idle and let the others serialise
-// their MFMA and softmax phases alone on their SIMDs.
-enum Layout { kSplit = 0, kMix5 = 1, kMix6 = 2, kFull = 3 };
-constexpr int rows_per_wg(int layout) { return layout == kSplit ? 128 : layout == kMix5 ? 160 : layout == kMix6 ? 192 : 256; }
-constexpr int layout_for(int n_q) { return n_q <= 128 ? kSplit : n_q <= 160 ? kMix5 : n_q <= 192 ? kMix6 : kFull; }
-struct WaveRole { int block, part, pair; };  // part: 0/1 = that half of the keys, 2 = full; pair: merge slot of a half
-__device__ inline WaveRole wave_role(int layout, int w) {
-  switch (layout) {
-    case kSplit: return {w & 3, w >> 2, w & 3};
-    case kMix5: {
-      if (w < 2) return {w, 2, 0};
-      if (w == 2 || w == 6) return {2, w == 6, 0};
-      if (w == 3 || w == 7) return {3, w == 7, 1};
-      return {4, w == 5, 2};
-    }
-    case kMix6: return w < 4 ? WaveRole{w, 2, 0} : WaveRole{4 + ((w - 4) >> 1), (w - 4) & 1, (w - 4) >> 1};
-    default: return {w, 2, 0};
-  }
-}
-constexpr int kKBuffers = 3;               // K tiles in LDS: K(t+1) is multiplied while K(t+2) is staged
-constexpr int kVBuffers = 2;               // V tiles in LDS: V(t) is multiplied while V(t+1) is staged
-constexpr int kRing = 2;                   // register stages of tiles on their way from memory
+constexpr int kMfmaThreads = kThreads;  // 512
 
 template <int N, typename F, int I = 0>
 __device__ __attribute__((always_inline)) inline void rd_static_for(F&& f) {
@@ -137,9 +108,6 @@ __device__ __attribute__((always_inline)) inline void rd_static_for(F&& f) {
     rd_static_for<N, F, I + 1>(static_cast<F&&>(f));
   }
 }
-constexpr int kKsStride = kD + 8;          // bf16 elements; 272-byte rows spread 16 lanes over all banks
-constexpr int kVtStride = kTile + 8;       // bf16 elements; 144-byte rows: 16-byte aligned, conflict-free
-
 // max over the two lanes (l, l^32) that share a query row
 __device__ inline float pair_max(float v) {
   const unsigned u = __float_as_uint(v);
@@ -159,10 +127,7 @@ template <int LAYOUT, bool ROPE>
 __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   constexpr int kRowsPerWG = rows_per_wg(LAYOUT);
   constexpr bool kHasFull = LAYOUT != kSplit, kHasHalf = LAYOUT != kFull;
-  constexpr int kKBytes = kKBuffers * kTile * kKsStride * 2, kVBytes = kVBuffers * kD * kVtStride * 2;
-  __shared__ __attribute__((aligned(16))) char smem[kKBytes + kVBytes];
-  __bf16 (*s_k)[kTile * kKsStride] = reinterpret_cast<__bf16 (*)[kTile * kKsStride]>(smem);
-  __bf16 (*s_vt)[kD * kVtStride] = reinterpret_cast<__bf16 (*)[kD * kVtStride]>(smem + kKBytes);
+  __shared__ __attribute__((aligned(16))) char smem[kLdsBytes];
 
   // The item is requested together with the item count (one trip to memory instead of two; the
   // item array has a slot for every blockIdx.y), and every kernel argument is fetched up front:
@@ -193,7 +158,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const int kp = full ? 0 : role.part;                 // key half of a half wave
   const RowSpan rows = row_span(a, b);
   if (q_tile * kRowsPerWG >= rows.n) return;  // (every thread of the workgroup: no barrier is skipped)
-  const int q_row = q_tile * kRowsPerWG + row_wave * 32 + r;
+  const int q_row = q_row_of(q_tile, kRowsPerWG, row_wave, r);
   const bool wave_active = q_tile * kRowsPerWG + row_wave * 32 < rows.n;
   const bool row_valid = q_row < rows.n;
 
@@ -217,9 +182,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // (`finish`) after the last tile load of the prologue has been issued.  The stores are not waited
   // for there either: the first tile that holds new rows is requested many steps into the loop,
   // and the step before that request waits for them (t_sync), ahead of its barrier.
-  const bool writes = ROPE && (hi > a.new_col0 || hi >= key_end);  // (uniform over the workgroup)
-  const int t_lo = lo > a.new_col0 ? lo - a.new_col0 : 0;
-  const int t_hi = !writes ? 0 : (hi >= key_end || hi - a.new_col0 > rows.n ? rows.n : hi - a.new_col0);
+  const NewRows mine = new_rows_of_item(lo, hi, key_end, a.new_col0, rows.n);  // (uniform over the workgroup)
+  const int t_lo = mine.t_lo, t_hi = ROPE ? mine.t_hi : 0;
   const bool has_new = t_lo < t_hi;
   // K tile j is requested in step j - 2 - kRing (the prologue for j < 2 + kRing), V tiles later
   const int first_new_tile = a.new_col0 > lo ? (a.new_col0 - lo) / kTile : 0;
@@ -243,15 +207,13 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   auto new_rows_issue = [&](int round) __attribute__((always_inline)) {
     // every load reads a token that exists (the round's first one stands in where a thread has no
     // task): the loads are then unconditional and the compiler keeps them together
-    const int t0 = t_lo + 128 * round;
+    const int t0 = t_lo + kNewRowsPerRound * round;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int task = tid + kMfmaThreads * i, t = t0 + (task >> 3);
-      const int64_t cache_row = (int64_t)a.new_col0 + t - kv_shift;
-      // (a shift that leaves the slab is not followed: the row is dropped)
-      const bool on = t < t_hi && cache_row >= 0 && cache_row < a.max_len;
+      const int t = rope_k_token(t0, tid, i);
+      const bool on = t < t_hi && new_row_in_slab(a.new_col0, t, kv_shift, a.max_len);
       nr.kt[i] = on ? t : -1;
-      nr.kc[i] = task & 7;
+      nr.kc[i] = rope_k_chunk(tid, i);
       const int tl = on ? t : t0;
       nr.pos[i] = a.position_ids[(int64_t)b * a.pos_sb + tl];
       nr.x1[i] = *reinterpret_cast<const bf16x8*>(kn + (int64_t)tl * a.kn_st + 8 * nr.kc[i]);
@@ -259,11 +221,10 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int task = tid + kMfmaThreads * i, t = t0 + (task >> 4);
-      const int64_t cache_row = (int64_t)a.new_col0 + t - kv_shift;
-      const bool on = t < t_hi && cache_row >= 0 && cache_row < a.max_len;
+      const int t = rope_v_token(t0, tid, i);
+      const bool on = t < t_hi && new_row_in_slab(a.new_col0, t, kv_shift, a.max_len);
       nr.vt[i] = on ? t : -1;
-      nr.vc[i] = task & 15;
+      nr.vc[i] = rope_v_chunk(tid, i);
       nr.vv[i] = *reinterpret_cast<const bf16x8*>(vn + (int64_t)(on ? t : t0) * a.vn_st + 8 * nr.vc[i]);
     }
 #pragma unroll
@@ -300,7 +261,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // than 128 tokens, rare); the rows are in memory after new_rows_wait
   auto new_rows_complete = [&]() __attribute__((always_inline)) {
     new_rows_finish();
-    for (int round = 1; t_lo + 128 * round < t_hi; ++round) {
+    for (int round = 1; t_lo + kNewRowsPerRound * round < t_hi; ++round) {
       new_rows_issue(round);
       new_rows_finish();
     }
@@ -313,8 +274,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // partner of a first-half dim (ks < 4) sits in fragment ks + 4 of the same lane
   bf16x8 qc[8], qs[8];
   {
-    const __bf16* qp = reinterpret_cast<const __bf16*>(a.q) + rows.q_off + (int64_t)h * a.q_sh +
-                       (int64_t)(row_valid ? q_row : 0) * a.q_ss + 8 * g;
+    const __bf16* qp = reinterpret_cast<const __bf16*>(a.q) + rows.q_off +
+                       q_frag_offset(h, a.q_sh, row_valid ? q_row : 0, a.q_ss, g, 0);
     int64_t q_pos = 0;
     if constexpr (ROPE) q_pos = a.position_ids[(int64_t)b * a.pos_sb + (row_valid ? q_row : 0)];
 #pragma unroll
@@ -349,7 +310,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       }
     }
   };
-  const uint64_t* brow = a.bits + ((int64_t)b * a.n_q + (row_valid ? q_row : 0)) * a.words;
+  const uint64_t* brow = a.bits + mask_word_index(b, a.n_q, row_valid ? q_row : 0, a.words, 0);
 
   f32x16 o[4];
 #pragma unroll
@@ -359,19 +320,13 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   float m = -INFINITY, l = 0.f;  // m in log2 units (already scaled)
   const float scale_log2 = a.scale * 1.4426950408889634f;
 
-  // Loader roles: threads [0,256) stage K rows (keys lrow+16*i), threads [256,512) stage V
-  // transposed (keys 4*lrow+i); four 16-byte chunks each per tile.  The V threads map lanes to
-  // (chunk, key quad) so that the 16 lanes of one LDS write cycle hit 16 different bank pairs: lane
-  // bits 0-1 and 4-5 select the chunk, bits 2-3 and 6-7 the key quad.
-  const bool k_loader = wave < kWaves / 2;
-  const int lt = tid & 255;
-  const int chunk = k_loader ? (lt & 15) : ((lt & 3) | (((lt >> 4) & 3) << 2));  // 16-byte column chunk of a row
-  const int lrow = k_loader ? (lt >> 4) : (((lt >> 2) & 3) | ((lt >> 6) << 2));
-  // V^T rows hold the keys of every 16-key group in the order [0-3, 8-11, 4-7, 12-15]: the eight
-  // keys that one lane feeds to a 16-key MFMA step are then 16 contiguous bytes.
-  const int vt_col = 16 * (lrow >> 2) + 4 * (((lrow & 1) << 1) | ((lrow >> 1) & 1));
+  // Loader roles (attn_addr.h: loader_of): waves 0-3 stage K rows, waves 4-7 stage V transposed,
+  // four 16-byte chunks per thread and tile.
+  const bool k_loader = wave < kWaves / 2;  // (== ld.k_loader, and wave-uniform for the compiler)
+  const Loader ld = loader_of(tid);
+  const int chunk = ld.chunk, lrow = ld.lrow;
 
-  const int n_tiles = (hi - lo + kTile - 1) / kTile;
+  const int n_tiles = n_tiles_of(lo, hi);
   // Tiles in flight: a ring of kRing register stages between global memory and LDS; tile j
   // passes through slot j % kRing.  The mask words travel in a ring of their own.
   // Every step issues the same loads on every path (tile indices past the end are clamped to the
@@ -386,24 +341,23 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // address of a 16-byte chunk = wave-uniform part (tile, i) + 32-bit lane part
   const char* base = reinterpret_cast<const char*>(k_loader ? kbase : vbase);
   const int64_t row_bytes = (k_loader ? a.k_ss : a.v_ss) * 2;
-  const int key_step = k_loader ? 16 : 1;   // this thread's keys within a tile: first_key + i * key_step
-  const int first_key = k_loader ? lrow : 4 * lrow;
+  const int key_step = ld.key_step, first_key = ld.first_key;  // this thread's keys within a tile: first_key + i * key_step
   const uint32_t lane_off = (uint32_t)(first_key * row_bytes + 16 * chunk);
   auto fetch_into = [&](bf16x8& c0, bf16x8& c1, bf16x8& c2, bf16x8& c3, int j) __attribute__((always_inline)) {
-    const int key0 = lo + (j < n_tiles ? j : n_tiles - 1) * kTile;
+    const int key0 = tile_key0(lo, j, n_tiles);
     const char* tile = base + (int64_t)key0 * row_bytes;
     const int64_t step_bytes = key_step * row_bytes;
+    // chunk i reads key column tile_chunk_key(ld, key0, i, key_min, key_end): inside the span that
+    // is key0 + first_key + i * key_step ...
     int64_t o0 = lane_off, o1 = step_bytes + lane_off, o2 = 2 * step_bytes + lane_off, o3 = 3 * step_bytes + lane_off;
-    if (key0 + kTile > key_end || key0 < key_min) {
+    if (tile_leaves_span(key0, key_min, key_end)) {
       // the first and the last tile of a row: keys in front of the row's first attended key (left
       // padding) re-read that key, keys behind its last attended key (tree slots that do not exist,
       // the end of the cache) re-read that one.  Nothing outside the row's live cache rows is ever
       // touched: the probabilities of those keys are zero, but zero times whatever lay there
       // could be NaN
       auto clamped = [&](int i) __attribute__((always_inline)) {
-        const int key = key0 + first_key + i * key_step;
-        const int use = (key < key_end ? (key > key_min ? key : key_min) : key_end - 1) - key0;
-        return (int64_t)use * row_bytes + 16 * chunk;
+        return (int64_t)(tile_chunk_key(ld, key0, i, key_min, key_end) - key0) * row_bytes + 16 * chunk;
       };
       o0 = clamped(0); o1 = clamped(1); o2 = clamped(2); o3 = clamped(3);
     }
@@ -416,27 +370,27 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     if constexpr (decltype(slot_c)::value == 0) fetch_into(a0, a1, a2, a3, j); else fetch_into(b0, b1, b2, b3, j);
   };
   auto fetch_word = [&](auto slot_c, int j) __attribute__((always_inline)) {
-    const int key0 = lo + (j < n_tiles ? j : n_tiles - 1) * kTile;
+    const int key0 = tile_key0(lo, j, n_tiles);
     // nothing may touch the loaded value here: an operation on it would make the wave wait for
     // this load, and with it for every tile load issued before it, at this point of every step
     wring[decltype(slot_c)::value] = brow[key0 >> 6];
   };
   auto stage_k_from = [&](bf16x8 c0, bf16x8 c1, bf16x8 c2, bf16x8 c3, int j) __attribute__((always_inline)) {
-    __bf16* dst = s_k[j % kKBuffers] + lrow * kKsStride + 8 * chunk;
+    char* dst = smem + lds_k_stage(ld, j, 0);
     *reinterpret_cast<bf16x8*>(dst) = c0;
-    *reinterpret_cast<bf16x8*>(dst + 16 * kKsStride) = c1;
-    *reinterpret_cast<bf16x8*>(dst + 32 * kKsStride) = c2;
-    *reinterpret_cast<bf16x8*>(dst + 48 * kKsStride) = c3;
+    *reinterpret_cast<bf16x8*>(dst + (lds_k_stage(ld, 0, 1) - lds_k_stage(ld, 0, 0))) = c1;
+    *reinterpret_cast<bf16x8*>(dst + (lds_k_stage(ld, 0, 2) - lds_k_stage(ld, 0, 0))) = c2;
+    *reinterpret_cast<bf16x8*>(dst + (lds_k_stage(ld, 0, 3) - lds_k_stage(ld, 0, 0))) = c3;
   };
   auto stage_k = [&](auto slot_c, int j) __attribute__((always_inline)) {
     if constexpr (decltype(slot_c)::value == 0) stage_k_from(a0, a1, a2, a3, j); else stage_k_from(b0, b1, b2, b3, j);
   };
   auto stage_v_from = [&](bf16x8 p0, bf16x8 p1, bf16x8 p2, bf16x8 p3, int j) __attribute__((always_inline)) {
-    __bf16* dst = s_vt[j % kVBuffers] + 8 * chunk * kVtStride + vt_col;
+    char* dst = smem + lds_v_stage(ld, j, 0);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       bf16x4 t = {p0[e], p1[e], p2[e], p3[e]};
-      *reinterpret_cast<bf16x4*>(dst + e * kVtStride) = t;
+      *reinterpret_cast<bf16x4*>(dst + (lds_v_stage(ld, 0, e) - lds_v_stage(ld, 0, 0))) = t;
     }
   };
   auto stage_v = [&](auto slot_c, int j) __attribute__((always_inline)) {
@@ -447,8 +401,11 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // A wave walks through one or two units per tile: both 32-key halves (a full wave) or its own.
   static_assert(kRing % 2 == 0, "the score registers alternate between two sets per unit");
   f32x16 s_reg[2];
-  auto k_frag = [&](const __bf16* sk, int key_off, int ks) __attribute__((always_inline)) {
-    return *reinterpret_cast<const bf16x8*>(&sk[(key_off + r) * kKsStride + 16 * ks + 8 * g]);
+  // (lds_k_frag is linear in its arguments: the lane's place in the tile's buffer plus the wave-uniform
+  // place of the unit's fragment)
+  auto k_lane = [&](int tile) __attribute__((always_inline)) { return smem + lds_k_frag(tile, 0, r, g, 0); };
+  auto k_frag = [&](const char* sk, int key_off, int ks) __attribute__((always_inline)) {
+    return *reinterpret_cast<const bf16x8*>(sk + lds_k_frag(0, key_off, 0, 0, ks));
   };
 
   // ---- prologue: K of tiles 0 and 1 and V of tile 0 into LDS, the ring filled behind them --------
@@ -498,7 +455,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     for (int i = 0; i < 16; ++i) s_reg[0][i] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks)
-      s_reg[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(s_k[0], kp * 32, ks), qf[ks], s_reg[0], 0, 0, 0);
+      s_reg[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(k_lane(0), kp * 32, ks), qf[ks], s_reg[0], 0, 0, 0);
   }
 
   // ---- one unit per step -----------------------------------------------------------------------
@@ -554,7 +511,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       const float m_use = m == -INFINITY ? 0.f : m;
       // S(next unit) = K Q^T  ||  P = exp2(S * scale - m).  After the last unit the product reads
       // a stale buffer; its result is never used.
-      const __bf16* sk = s_k[next_t % kKBuffers];
+      const char* sk = k_lane(next_t);
       float psum = 0.f;
       constexpr int kDepth = 4;  // K fragments in flight from LDS (a read takes longer than two MFMAs)
       bf16x8 ka[kDepth];
@@ -587,9 +544,9 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     // the second product starts
     constexpr int kVDepth = 4;
     bf16x8 va[kVDepth];
-    const __bf16* sv = s_vt[t % kVBuffers] + key_off + 8 * g;
+    const char* sv = smem + lds_v_frag(t, key_off, r, g, 0);
     auto v_frag = [&](int c) __attribute__((always_inline)) {
-      return *reinterpret_cast<const bf16x8*>(&sv[(32 * (c >> 1) + r) * kVtStride + 16 * (c & 1)]);
+      return *reinterpret_cast<const bf16x8*>(sv + (lds_v_frag(0, 0, 0, 0, c) - lds_v_frag(0, 0, 0, 0, 0)));
     };
     if (busy) {
 #pragma unroll
@@ -657,22 +614,25 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   if (kHasHalf) {
     // merge the two key parts of every row block: part 1 hands (m, l, o) over through LDS (the tile
     // buffers are free: every wave has passed the loop's last barrier)
-    float* x_o = reinterpret_cast<float*>(smem);             // [pair][64 accumulators][lane]
-    float* x_ml = x_o + (kWaves / 2) * 64 * 64;              // [pair][2][lane]
-    static_assert((kWaves / 2) * (64 * 64 + 2 * 64) * 4 <= kKBytes + kVBytes, "merge buffer");
-    const int pair = role.pair;
+    auto x_o = [&](int acc) __attribute__((always_inline)) -> float& {  // [pair][64 accumulators][lane]
+      return *reinterpret_cast<float*>(smem + lds_merge_o(role.pair, acc, lane));
+    };
+    auto x_ml = [&](int which) __attribute__((always_inline)) -> float& {  // [pair][2][lane]
+      return *reinterpret_cast<float*>(smem + lds_merge_ml(role.pair, which, lane));
+    };
+    static_assert(kMergeFloats * 4 <= kLdsBytes, "merge buffer");
     const bool second = !full && kp == 1;
     if (second && wave_active) {
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) x_o[(pair * 64 + 16 * db + i) * 64 + lane] = o[db][i];
-      x_ml[(pair * 2 + 0) * 64 + lane] = m;
-      x_ml[(pair * 2 + 1) * 64 + lane] = l;
+        for (int i = 0; i < 16; ++i) x_o(16 * db + i) = o[db][i];
+      x_ml(0) = m;
+      x_ml(1) = l;
     }
     __syncthreads();
     if (wave_active && !full && !second) {
-      const float m2 = x_ml[(pair * 2 + 0) * 64 + lane], l2 = x_ml[(pair * 2 + 1) * 64 + lane];
+      const float m2 = x_ml(0), l2 = x_ml(1);
       const float m_new = fmaxf(m, m2);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       const float a1 = fast_exp2(m - m_safe), a2 = fast_exp2(m2 - m_safe);  // exp2(-inf) = 0
@@ -681,7 +641,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-          o[db][i] = a1 * o[db][i] + a2 * x_o[(pair * 64 + 16 * db + i) * 64 + lane];
+          o[db][i] = a1 * o[db][i] + a2 * x_o(16 * db + i);
       m = m_new;
     }
   }
@@ -692,8 +652,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     if (!writer) return;
     const bool live = l > 0.f;
     const float inv = live ? 1.f / l : 0.f;
-    __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh +
-                 (int64_t)q_row * a.o_ss + 4 * g;
+    __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + out_offset(h, a.o_sh, q_row, a.o_ss, g, 0, 0);
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -701,7 +660,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
         // (a row without any attended key gets zeros, whatever its accumulators picked up)
         bf16x4 w = {static_cast<__bf16>(live ? o[db][4 * i4 + 0] * inv : 0.f), static_cast<__bf16>(live ? o[db][4 * i4 + 1] * inv : 0.f),
                     static_cast<__bf16>(live ? o[db][4 * i4 + 2] * inv : 0.f), static_cast<__bf16>(live ? o[db][4 * i4 + 3] * inv : 0.f)};
-        *reinterpret_cast<bf16x4*>(op + 32 * db + 8 * i4) = w;
+        *reinterpret_cast<bf16x4*>(op + (out_offset(0, 0, 0, 0, 0, db, i4))) = w;
       }
     return;
   }
@@ -715,9 +674,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // own L2), 16 bytes at a time.  A release fence before the count and an acquire fence behind it
   // would do the same for ordinary accesses, but each works on the whole L2 of its XCD while the
   // other workgroups stream through it: rows split four ways ran 8-19 % longer that way.
-  const int64_t slot0 = ((int64_t)b * a.H + h) * a.max_splits;
   if (writer) {
-    float* po = a.part_o + ((slot0 + split) * a.n_q + q_row) * kD + 4 * g;
+    float* po = a.part_o + partial_row(b, a.H, h, a.max_splits, split, a.n_q, q_row) * kD + 4 * g;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -726,7 +684,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
         asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(po + 32 * db + 8 * i4), "v"(w) : "memory");
       }
     if (g == 0) {
-      float* pm = a.part_ml + ((slot0 + split) * a.n_q + q_row) * 2;
+      float* pm = a.part_ml + partial_row(b, a.H, h, a.max_splits, split, a.n_q, q_row) * 2;
       const f32x2 ml = {m, l};
       asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(pm), "v"(ml) : "memory");
     }
@@ -737,7 +695,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   int* s_last = reinterpret_cast<int*>(smem);  // (the tile buffers are free by now)
-  int32_t* counter = a.counters + ((int64_t)b * rd::kAttnMaxHeads + h) * q_tiles + q_tile;
+  int32_t* counter = a.counters + counter_index(b, rd::kAttnMaxHeads, h, q_tiles, q_tile);
   if (wave == 0) {
     int last = 0;
     if (lane == 0) last = atomicAdd(counter, 1) == n_splits - 1;
@@ -764,14 +722,19 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
 #pragma unroll
       for (int j = 0; j < kPass; ++j) {
         const int q = q0 + kGroups * j < q_end ? q0 + kGroups * j : q_end - 1;  // clamped: loads stay unconditional
-        const int64_t row = (slot0 + s) * a.n_q + q;
+        const int64_t row = partial_row(b, a.H, h, a.max_splits, s, a.n_q, q);
         asm volatile("global_load_dwordx2 %0, %1, off sc1" : "=v"(ml[j]) : "v"(a.part_ml + row * 2) : "memory");
         asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(po[j]) : "v"(a.part_o + row * kD + dq) : "memory");
       }
-      // (the compiler does not count these loads: one wait for all of them, tied to their registers)
-      static_assert(kPass == 8, "the wait below names eight register pairs");
-      asm volatile("s_waitcnt vmcnt(0)" : "+v"(ml[0]), "+v"(ml[1]), "+v"(ml[2]), "+v"(ml[3]), "+v"(ml[4]), "+v"(ml[5]), "+v"(ml[6]), "+v"(ml[7]));
-      asm volatile("" : "+v"(po[0]), "+v"(po[1]), "+v"(po[2]), "+v"(po[3]), "+v"(po[4]), "+v"(po[5]), "+v"(po[6]), "+v"(po[7]));
+      // (the compiler does not count these loads: one wait for all of them, and every destination
+      // register is an operand of that wait, so that none of them can be copied, spilled or read
+      // between its load and the wait)
+      static_assert(kPass == 8, "the wait below names eight register pairs and eight quads");
+      asm volatile("s_waitcnt vmcnt(0)"
+                   : "+v"(ml[0]), "+v"(ml[1]), "+v"(ml[2]), "+v"(ml[3]), "+v"(ml[4]), "+v"(ml[5]), "+v"(ml[6]), "+v"(ml[7]),
+                     "+v"(po[0]), "+v"(po[1]), "+v"(po[2]), "+v"(po[3]), "+v"(po[4]), "+v"(po[5]), "+v"(po[6]), "+v"(po[7])
+                   :
+                   : "memory");
 #pragma unroll
       for (int j = 0; j < kPass; ++j) {
         const float m_new = fmaxf(mx[j], ml[j][0]);
@@ -788,7 +751,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       if (q < q_end) {
         const bool live = ls[j] > 0.f;
         const float inv = live ? 1.f / ls[j] : 0.f;
-        __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + (int64_t)h * a.o_sh + (int64_t)q * a.o_ss + dq;
+        __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + out_offset(h, a.o_sh, q, a.o_ss, 0, 0, 0) + dq;
         bf16x4 w = {static_cast<__bf16>(live ? acc[j][0] * inv : 0.f), static_cast<__bf16>(live ? acc[j][1] * inv : 0.f),
                     static_cast<__bf16>(live ? acc[j][2] * inv : 0.f), static_cast<__bf16>(live ? acc[j][3] * inv : 0.f)};
         *reinterpret_cast<bf16x4*>(op) = w;

@@ -38,7 +38,7 @@ __global__ __launch_bounds__(THREADS) void row_stats_kernel(
   const float mask_z = mask_value / temperature;
   // (a few more maxima than k_eff: the k-th largest key then sits well above the pivot's key, and
   // a tie between the two, which costs the slow path, takes that many equal values in a row)
-  const float pivot = row_pivot<THREADS, 8 * (sizeof(T) < 4 ? sizeof(T) : 4)>(tmax, k_eff + kPivotMargin < THREADS ? k_eff + kPivotMargin : THREADS, sh);
+  const float pivot = row_pivot<THREADS, Num<T>::kValueBits>(tmax, k_eff + kPivotMargin < THREADS ? k_eff + kPivotMargin : THREADS, sh);
   int n_c = -1;
   if (!force_fallback)
     n_c = row_sorted_candidates<ITEMS, VEC, THREADS>(

@@ -12,9 +12,15 @@ import os
 
 import torch
 
-# RD_HIP_LIBRARY names another build of the library (an A/B of two builds on one machine)
-_LIB_PATH = os.environ.get("RD_HIP_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "libredrafter_hip.so")
+import sys
+
+# The library built from csrc/ sits beside this file.  RD_HIP_LIBRARY names another build of it (an
+# A/B of two builds on one machine); whoever loads one is told so on stderr, and the test suite
+# refuses to run on it (tests/conftest.py).
+_DEFAULT_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libredrafter_hip.so")
+_LIB_PATH = os.environ.get("RD_HIP_LIBRARY") or _DEFAULT_LIB_PATH
 _lib = None
+ABI_VERSION = 103  # RD_ABI_VERSION of include/redrafter_hip.h that _PROTOTYPES below was written against
 
 RD_BF16, RD_F16, RD_F32 = 0, 1, 2
 _DTYPES = {torch.bfloat16: RD_BF16, torch.float16: RD_F16, torch.float32: RD_F32}
@@ -24,7 +30,6 @@ _P, _I, _L, _Z, _F = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 _PROTOTYPES = {
     "rd_version": (C.c_int, []),
     "rd_last_error": (C.c_char_p, []),
-    "rd_stream_tiles_probe": (_I, [_P, _P, _L, _I, _I, _I, _P, _P]),
     "rd_timing_enable": (_I, [_I]),
     "rd_timing_select": (_I, [C.c_char_p]),
     "rd_timing_sample": (_I, [_I]),
@@ -93,6 +98,11 @@ def library_path() -> str:
     return _LIB_PATH
 
 
+def is_default_library() -> bool:
+    """False when RD_HIP_LIBRARY points the package at another build of the library."""
+    return os.path.realpath(_LIB_PATH) == os.path.realpath(_DEFAULT_LIB_PATH)
+
+
 def lib():
     """Loads the shared library on first use."""
     global _lib
@@ -104,6 +114,15 @@ def lib():
                 "there is no CPU or PyTorch fallback for the HIP kernels"
             )
         handle = C.CDLL(_LIB_PATH)
+        if not is_default_library():
+            print(f"recurrent_drafting_amd: RD_HIP_LIBRARY is set, using {_LIB_PATH} instead of the in-tree "
+                  "library", file=sys.stderr, flush=True)
+        handle.rd_version.restype = C.c_int
+        found = handle.rd_version()
+        if found != ABI_VERSION:
+            raise RuntimeError(
+                f"{_LIB_PATH} has interface version {found}, this package was written against {ABI_VERSION}: "
+                "rebuild it with `python ml-recurrent-drafter_amd/build_hip.py`")
         for name, (res, args) in _PROTOTYPES.items():
             fn = getattr(handle, name)
             fn.restype = res

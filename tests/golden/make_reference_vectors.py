@@ -113,7 +113,12 @@ def kv_update_cases(rd):
 def beam_search_cases(rd):
     """Tie-free float32 drafter: distinct logits everywhere, so torch.topk's order is determined."""
     out = []
-    for seed, (B, W, L, V, hid) in enumerate([(2, 3, 4, 64, 8), (1, 4, 3, 80, 8), (2, 5, 5, 96, 16)]):
+    # the last two are wider than the top-50 filter (W = 64 > 50 < V): after the first iteration 14
+    # beams are filtered tokens whose scores tie, and torch.topk's choice among them is unspecified;
+    # from the second iteration on 50 live beams offer 2500 candidates, so the final beams (L >= 3)
+    # descend from live beams only and do not depend on that choice
+    for seed, (B, W, L, V, hid) in enumerate([(2, 3, 4, 64, 8), (1, 4, 3, 80, 8), (2, 5, 5, 96, 16),
+                                              (2, 64, 4, 96, 16), (1, 64, 3, 120, 8)]):
         torch.manual_seed(100 + seed)
         cfg = rd.configuration_drafter.DrafterConfig(
             vocab_size=V, hidden_size=hid, exit_dim=2 * hid, num_draft_layers=1, rnn=True)
@@ -174,6 +179,10 @@ def end_to_end_cases(rd):
              dict(seed=21, batch=4, prompt_len=10, left_pads=[0, 4, 1, 0], W=5, L=4, new_tokens=30,
                   markov=True),
              dict(seed=22, batch=2, prompt_len=6, left_pads=[0, 2], W=8, L=6, new_tokens=40,
+                  markov=True),
+             # beams wider than the top-50 filter: ties are certain in the first beam-search iteration
+             dict(seed=31, batch=2, prompt_len=8, left_pads=[0, 3], W=64, L=5, new_tokens=24),
+             dict(seed=32, batch=3, prompt_len=7, left_pads=[2, 0, 1], W=64, L=5, new_tokens=36,
                   markov=True)]
     for c in cases:
         if c.get("markov"):
@@ -351,7 +360,9 @@ def sampling_stream_cases(rd):
              dict(seed=21, batch=3, prompt_len=8, left_pads=[3, 0, 1], W=5, L=5, new_tokens=24,
                   temperature=1.0, rand_seed=78, markov=True),
              dict(seed=23, batch=2, prompt_len=7, left_pads=[0, 2], W=4, L=3, new_tokens=16,
-                  temperature=1.7, rand_seed=79, markov=True)]
+                  temperature=1.7, rand_seed=79, markov=True),
+             dict(seed=33, batch=2, prompt_len=8, left_pads=[1, 0], W=64, L=5, new_tokens=24,
+                  temperature=1.0, rand_seed=80, markov=True)]
     out = []
     real_rand = torch.rand
     for c in cases:

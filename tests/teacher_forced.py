@@ -8,7 +8,17 @@ RecurrentDrafting.generate and, at every step, hands the state the HIP loop went
 with (token ids, drafter context, first token, KV cache contents) to oracle/torch_path on the
 same GPU, then compares what came out:
 
-  beams            oracle beam search on the same context and token (same bf16 torch GEMMs)
+  prefill          before the first step: the cache rows of every layer behind each row's left
+                   padding, the last hidden state and the first token of _comprehend_prompt
+                   (recurrent_drafting.py:391-434) against the float32 restatement of the prefill
+                   (error within `tol` of the scale and within 3x the error of stock torch in the
+                   model's dtype; the token may differ from the float32 argmax only inside the margin)
+  beams            oracle beam search on the same context and token (same bf16 torch GEMMs), reported;
+                   and, asserted, every beam-search iteration on ITS OWN logits: the oracle's
+                   iteration (fp_oracle.beam_search_step, modeling_drafter.py:201-215) fed the logits
+                   and scores the HIP kernel was fed must select the same (parent, token) pairs --
+                   bit for bit where the log-probabilities agree bit for bit, otherwise as
+                   tests/beam_band.py says
   tree             packed tokens, unpacker, position offsets and ids, left pad counts, and the mask
                    (unpacked from the bits the attention consumes) of the HIP beams: bit-exact
   packed logits    against the float32 restatement (bf16 weights upcast), within `tol` of the
@@ -36,7 +46,9 @@ from typing import Callable, List, Optional
 import numpy as np
 import torch
 
+import beam_band
 from oracle import accept_oracle as Acc
+from oracle import fp_oracle as O
 from oracle import torch_path as P
 
 
@@ -48,6 +60,7 @@ class StepReport:
     rows: int
     beams_equal: bool
     beams_shared: float  # share of the HIP beams that are among the restatement's beams of the same row
+    beam_picks_shared: float  # lowest share, over the iterations, of the HIP picks that the oracle makes on the same logits
     logits_err: float  # max |HIP - float32 restatement| / scale
     logits_err_bf16_torch: float  # the same for the bf16 restatement (stock torch ops)
     flips: int  # packed positions whose argmax differs from the float32 argmax
@@ -56,6 +69,17 @@ class StepReport:
     shifts: List[int]  # cache row shifts going into the step
     context_err: float
     kv_err: float
+
+
+@dataclasses.dataclass
+class PrefillReport:
+    seq: int
+    kv_err: float  # max |HIP - float32 restatement| / scale over the cache rows behind the left padding, all layers
+    kv_err_torch: float  # the same for stock torch in the model's dtype
+    state_err: float
+    state_err_torch: float
+    token_flips: int
+    worst_flip_margin: float
 
 
 def _bits_to_mask(bits: torch.Tensor, kv_len: int) -> torch.Tensor:
@@ -100,11 +124,13 @@ def forced_acceptance(seed: int) -> Callable:
 
 def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int = 0,
         tol: float = 2e-2, force: Optional[Callable] = None, check_from: int = 0,
-        log: Optional[Callable] = None) -> List[StepReport]:
-    """Runs `steps` decode steps of the fused loop; steps >= check_from are compared with the
-    restatement.  Raises AssertionError on the first violation; returns the per-step reports."""
+        log: Optional[Callable] = None, prefill_report: Optional[list] = None) -> List[StepReport]:
+    """Runs `steps` decode steps of the fused loop; the prefill and the steps >= check_from are
+    compared with the restatement.  Raises AssertionError on the first violation; returns the
+    per-step reports (the PrefillReport is appended to `prefill_report` when a list is given)."""
     import recurrent_drafting_amd as rd
-    from recurrent_drafting_amd import acceptance, tree_attention
+    from recurrent_drafting_amd import acceptance, modeling_drafter, tree_attention
+    from recurrent_drafting_amd import recurrent_drafting as loop_module
 
     dev = ids.device
     llm32 = copy.deepcopy(llm).float()  # bf16 weights upcast (the drafter is compared in its own dtype)
@@ -113,6 +139,21 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
     real_prepare, real_argmax = tree_attention.prepare_attention, acceptance.argmax_rows
     real_accept, real_realign = acceptance.greedy_accept, acceptance.realign_enqueue
     real_draft = drafter.beam_search_candidates
+    real_prefill, real_topk = loop_module._comprehend_prompt, modeling_drafter.beam_topk_step
+    prefilled = {}
+    iterations = []  # the beam-search iterations of the draft being made
+
+    def w_prefill(llm_, input_ids, cache, sampling_args, pad_token_id):
+        state, token = real_prefill(llm_, input_ids, cache, sampling_args, pad_token_id)
+        S = input_ids.shape[1]
+        prefilled.update(ids=input_ids, rows=cache._cache[:, :, :, :, :S].clone(), state=state.clone(),
+                         token=token.clone())
+        return state, token
+
+    def w_topk(logits, log_p_beam, beams, want_log_probs, force_fallback=False):
+        out = real_topk(logits, log_p_beam, beams, want_log_probs, force_fallback)
+        iterations.append(dict(logits=logits, lpb=log_p_beam, new_lpb=out[0], tok=out[1], par=out[2]))
+        return out
 
     def w_prepare(tree, padding_mask, pad_value=0, n_heads=32, kv_shift=None):
         out = real_prepare(tree, padding_mask, pad_value, n_heads, kv_shift)
@@ -143,8 +184,9 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
     drafts = []  # draft k feeds step k; it is queued while step k-1 is being finished
 
     def w_draft(context, init_token, embeddings, beam_shape, return_log_probs=True):
+        iterations.clear()
         out = real_draft(context, init_token, embeddings, beam_shape, return_log_probs=return_log_probs)
-        drafts.append(dict(context=context.clone(), init=init_token.clone(), beams=out[0]))
+        drafts.append(dict(context=context.clone(), init=init_token.clone(), beams=out[0], iterations=list(iterations)))
         return out
 
     reports: List[StepReport] = []
@@ -153,6 +195,8 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
             mock.patch.object(acceptance, "argmax_rows", w_argmax), \
             mock.patch.object(acceptance, "greedy_accept", w_accept), \
             mock.patch.object(acceptance, "realign_enqueue", w_realign), \
+            mock.patch.object(loop_module, "_comprehend_prompt", w_prefill), \
+            mock.patch.object(modeling_drafter, "beam_topk_step", w_topk), \
             mock.patch.object(drafter, "beam_search_candidates", w_draft):
         stream = model.generate(rd.stats.Ledger(), ids, max_length, rd.BeamShape(W, L),
                                 rd.SamplingArgs(1.0, True), rd.SpecialTokens(pad, None))
@@ -163,6 +207,12 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
             except StopIteration:
                 break
             assert len(drafts) == k + 2
+            if k == 0:
+                with torch.inference_mode():
+                    report = check_prefill(prefilled, llm, llm32, pad, tol)
+                prefilled.clear()
+                if prefill_report is not None:
+                    prefill_report.append(report)
             st = dict(seen)
             if k >= check_from:
                 with torch.inference_mode():
@@ -173,8 +223,65 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
                     log(reports[-1])
             prev_step = dict(snap=st["snap"], tree=st["tree"], unpacker=st["unpacker"], n=st["n"], s=st["s"],
                              ids=st["ids"], prev=st["ids"].shape[1])
+            drafts[k]["iterations"] = None  # (logits of a whole beam-search: not kept)
         stream.close()
     return reports
+
+
+def check_prefill(pf, llm, llm32, pad: int, tol: float) -> PrefillReport:
+    """The prefill of the HIP loop against oracle/torch_path's in float32 on the same token ids."""
+    ids, rows = pf["ids"], pf["rows"]  # rows: (layers, 2, B, Hkv, S, D), the reference's layout
+    dev = ids.device
+    B, S = ids.shape
+    n_layers, _, _, Hkv, _, D = rows.shape
+    pads = P.count_left_pads(ids, pad)
+    mask = P.causal_mask(ids != pad, S)
+    pos = torch.arange(S, device=dev).expand(B, S) - pads[:, None]
+
+    def restate(model, dtype):
+        cache = P.Cache(B, S, n_layers, Hkv, D, dtype, dev)
+        logits, hidden = P.llama_forward(model, ids, mask, pos, cache)
+        return cache.data.float(), hidden[:, -1, :].float(), logits[:, -1, :]
+
+    want_rows, want_state, want_logits = restate(llm32, torch.float32)
+    torch_rows, torch_state, _ = restate(llm, rows.dtype)
+    live = (torch.arange(S, device=dev)[None, :] >= pads[:, None])[None, None, :, None, :, None]
+    zero = torch.zeros((), device=dev)
+    kv_scale = float(torch.where(live, want_rows, zero).abs().max())
+    kv_err = float(torch.where(live, rows.float() - want_rows, zero).abs().max()) / kv_scale
+    kv_yard = float(torch.where(live, torch_rows - want_rows, zero).abs().max()) / kv_scale
+    assert kv_err <= tol, f"prefill: cache rows off by {kv_err:.3g} of their scale"
+    assert kv_err <= 3 * kv_yard + 1e-3, f"prefill: cache rows {kv_err:.3g} off, stock torch only {kv_yard:.3g}"
+    state_scale = float(want_state.abs().max())
+    state_err = float((pf["state"].float() - want_state).abs().max()) / state_scale
+    state_yard = float((torch_state - want_state).abs().max()) / state_scale
+    assert state_err <= tol, f"prefill: last hidden state off by {state_err:.3g} of its scale"
+    assert state_err <= 3 * state_yard + 1e-3, f"prefill: last hidden state {state_err:.3g} off, stock torch only {state_yard:.3g}"
+    o_tok = want_logits.argmax(dim=-1)
+    flipped = (pf["token"] != o_tok).nonzero().flatten()
+    scale = float(want_logits.abs().max())
+    margins = (want_logits[flipped, o_tok[flipped]] - want_logits[flipped, pf["token"][flipped]]) / scale
+    worst = float(margins.max()) if flipped.numel() else 0.0
+    assert worst <= tol, f"prefill: first token flipped with float32 margin {worst:.3g} of the scale"
+    return PrefillReport(S, kv_err, kv_yard, state_err, state_yard, int(flipped.numel()), worst)
+
+
+def _check_beam_iterations(k, iterations) -> float:
+    """Every iteration of the HIP beam search against the oracle's iteration on the same logits and
+    scores (modeling_drafter.py:201-215).  Returns the lowest share of common picks."""
+    lowest = 1.0
+    for it, rec in enumerate(iterations):
+        logits, lpb = rec["logits"].cpu(), rec["lpb"].cpu()
+        o_lpb, o_tok, o_par, o_logp = O.beam_search_step(logits, lpb)
+        live = o_logp.float() > -1000
+        # one rounding step of a log-probability in the drafter's dtype (float32: of the score near 50000)
+        tol = 2e-2 * float(o_logp.float()[live].abs().max()) if logits.dtype != torch.float32 else 1e-2
+        try:
+            shared = beam_band.check_selection(o_logp, lpb, o_lpb, o_tok, o_par, rec["new_lpb"], rec["tok"], rec["par"], tol)
+        except AssertionError as e:
+            raise AssertionError(f"step {k}, beam-search iteration {it}: {e}") from e
+        lowest = min(lowest, shared)
+    return lowest
 
 
 def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafter, W, L, pad, tol, prev_step,
@@ -197,6 +304,9 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
     # so the two searches may keep different candidates at the margin; the share in common is reported
     beams_shared = float((beams[:, :, None, :] == o_beams[:, None, :, :]).all(-1).any(-1).float().mean())
     assert torch.equal(beams[:, :, 0], draft_in["init"][:, None].expand(B, W))
+    assert len(draft_in["iterations"]) == L - 1
+    beam_picks_shared = _check_beam_iterations(k, draft_in["iterations"])
+    assert beam_picks_shared >= 0.9, f"step {k}: only {beam_picks_shared:.2f} of the HIP picks are the oracle's on the same logits"
 
     # -- tree of the HIP beams: bit-exact ----------------------------------------------------------
     o_packed, o_unpacker, o_mask, o_off = P.pack(beams, (ids != pad).to(ids.dtype))
@@ -293,5 +403,5 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
                 assert torch.equal(snap[:, :, b, :, lo + keep + j], p["snap"][:, :, b, :, src]), \
                     f"step {k}: accepted cache row {j} of row {b}"
             assert lo + keep + int(p["n"][b]) + 1 == prev
-    return StepReport(k, prev, n_q, total, beams_equal, beams_shared, logits_err, yard, int(flipped.numel()), worst,
+    return StepReport(k, prev, n_q, total, beams_equal, beams_shared, beam_picks_shared, logits_err, yard, int(flipped.numel()), worst,
                       n.tolist(), st["shift"].tolist(), context_err, kv_err)

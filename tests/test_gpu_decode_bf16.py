@@ -13,7 +13,13 @@ which bar).
    4096/8192 with two blocks), batch 8, about 1500 tokens of context with ragged left padding,
    beam 45 x 5: forced ragged acceptance for a few steps, then teacher-forced steps;
 4. speculative sampling at temperature 1 on the pair of 1: every step's acceptance and residual
-   distribution against the oracle on the step's own logits, drafter log-probabilities and uniforms.
+   distribution against the oracle on the step's own logits, drafter log-probabilities and uniforms;
+5. all 32 layers of the 7B shape, batch 8, ragged prompts of about 600 tokens, beam 45 x 5: the
+   prefill and two teacher-forced steps after forced ragged acceptance (the composition of the layers:
+   error growth through the residual stream, docs/parity_check.md:77-98).
+
+Every case also checks the prefill (cache rows, last hidden state, first token) against the float32
+restatement, and every beam-search iteration against the oracle's iteration on the same logits.
 """
 import os
 import sys
@@ -58,9 +64,16 @@ def _uses_mfma_kernel(fn):
     return out, kernels
 
 
+def _prefill_summary(pre):
+    r = pre[0]
+    return (f"prefill: S {r.seq} cache rows {r.kv_err:.2e} (torch {r.kv_err_torch:.2e}) last state {r.state_err:.2e} "
+            f"(torch {r.state_err_torch:.2e}) first-token flips {r.token_flips} (margin {r.worst_flip_margin:.1e})")
+
+
 def _summary(reports):
     return "\n".join(
         f"step {r.step}: prev {r.prev} n_q {r.n_q} rows {r.rows} beams_equal {r.beams_equal} shared {r.beams_shared:.2f} "
+        f"picks on the same logits {r.beam_picks_shared:.3f} "
         f"logits {r.logits_err:.2e} (torch bf16 {r.logits_err_bf16_torch:.2e}) flips {r.flips} "
         f"(margin {r.worst_flip_margin:.1e}) n {r.n_tokens} shift {r.shifts} ctx {r.context_err:.1e} "
         f"kv {r.kv_err:.1e}" for r in reports)
@@ -70,8 +83,10 @@ def test_bf16_mfma_decode_loop_teacher_forced_with_accepted_drafts():
     llama_sd, drafter_sd = tm.markov(41, llama_cfg=CFG, drafter_cfg=DCFG, mix=0.05)
     llm, drafter = _models(llama_sd, drafter_sd, CFG, DCFG)
     ids = tm.prompt(4, 300, 4000, 5, left_pads=[0, 131, 3, 250]).cuda()
+    pre = []
     reports, kernels = _uses_mfma_kernel(
-        lambda: teacher_forced.run(llm, drafter, ids, 300 + 40, 12, 5, steps=12))
+        lambda: teacher_forced.run(llm, drafter, ids, 300 + 40, 12, 5, steps=12, prefill_report=pre))
+    print(_prefill_summary(pre))
     print(_summary(reports))
     assert "attn_mfma_kernel" in kernels and "attn_generic_kernel" not in kernels
     assert len(reports) >= 8
@@ -93,9 +108,11 @@ def test_bf16_mfma_decode_loop_teacher_forced_random_weights_forced_acceptance(o
     drafter_sd = tm.draw(tm.drafter_shapes(DCFG), 52)
     llm, drafter = _models(llama_sd, drafter_sd, cfg, DCFG)
     ids = tm.prompt(4, 200, 4000, 6, left_pads=[17, 0, 120, 64]).cuda()
+    pre = []
     reports, kernels = _uses_mfma_kernel(
         lambda: teacher_forced.run(llm, drafter, ids, 200 + 60, 12, 5, steps=10,
-                                   force=teacher_forced.forced_acceptance(9)))
+                                   force=teacher_forced.forced_acceptance(9), prefill_report=pre))
+    print(_prefill_summary(pre))
     print(_summary(reports))
     assert "attn_mfma_kernel" in kernels and "attn_generic_kernel" not in kernels
     assert ("rope_append_kernel" in kernels) == (not one_kernel), sorted(kernels)
@@ -116,15 +133,51 @@ def test_bf16_7b_shape_one_layer_teacher_forced_steps_at_long_context():
     for b, n in enumerate([0, 700, 13, 250, 999, 64, 1, 420]):
         ids[b, :n] = 0
     ids = ids.cuda()
+    pre = []
     reports, kernels = _uses_mfma_kernel(
         lambda: teacher_forced.run(llm, drafter, ids, S + 64, 45, 5, steps=7, check_from=4,
-                                   force=teacher_forced.forced_acceptance(4)))
+                                   force=teacher_forced.forced_acceptance(4), prefill_report=pre))
+    print(_prefill_summary(pre))
     print(_summary(reports))
     assert "attn_mfma_kernel" in kernels and "attn_generic_kernel" not in kernels
-    assert len(reports) == 3
+    assert len(reports) == 3 and pre[0].seq == S
     assert all(r.prev >= 1500 and r.n_q >= 100 for r in reports)
-    assert all(r.beams_shared >= 0.5 for r in reports)
+    # (beams_shared compares with a beam search on logits from GEMMs of other shapes and is only
+    # reported; what is asserted is every iteration's selection on the same logits)
+    assert all(r.beam_picks_shared >= 0.9 for r in reports)
     assert any(any(x != 0 for x in r.shifts) for r in reports)
+
+
+def test_bf16_7b_shape_all_32_layers_prefill_and_teacher_forced_steps():
+    """Configuration 4 at full depth: 32 layers of the 7B shape in bf16, batch 8, beam 45 x 5, ragged
+    left-padded prompts of 600 tokens; the prefill and two steps (after two steps of forced ragged
+    acceptance, so rows have shifted) against the float32 restatement of all 32 layers.  The bar is
+    teacher_forced's, with the logit error also held against stock torch's bf16 error on the same
+    inputs (at most three times that)."""
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+
+    torch.manual_seed(0)
+    llm, drafter = bench.build_models("cuda:0", torch.bfloat16, 32, 11)
+    B, S = 8, 600
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(1, 32000, (B, S), generator=g)
+    for b, n in enumerate([0, 310, 7, 120, 455, 64, 1, 200]):
+        ids[b, :n] = 0
+    ids = ids.cuda()
+    pre = []
+    reports, kernels = _uses_mfma_kernel(
+        lambda: teacher_forced.run(llm, drafter, ids, S + 48, 45, 5, steps=4, check_from=2, tol=4e-2,
+                                   force=teacher_forced.forced_acceptance(6), prefill_report=pre))
+    print(_prefill_summary(pre))
+    print(_summary(reports))
+    assert "attn_mfma_kernel" in kernels and "attn_generic_kernel" not in kernels
+    assert len(reports) == 2 and pre[0].seq == S
+    assert all(r.prev >= 600 and r.n_q >= 100 for r in reports)
+    assert all(r.beam_picks_shared >= 0.9 for r in reports)
+    assert any(any(x != 0 for x in r.shifts) for r in reports)
+    # the composition of 32 layers stays as close to float32 as stock torch's bf16 ops do
+    assert all(r.logits_err <= 3 * r.logits_err_bf16_torch + 1e-3 for r in reports)
 
 
 def test_bf16_mfma_sampling_loop_accepts_as_the_oracle_does_on_the_same_logits():

@@ -90,7 +90,7 @@ def upstream_shaped_loop(llm, drafter, input_ids, max_length, beam_shape, sampli
                                   "base_forward", "choose_from_candidates", "update_kv_cache_and_input_ids"}
 
 
-@pytest.mark.parametrize("case_index", [1, 3, 4])
+@pytest.mark.parametrize("case_index", [1, 3, 4, 5, 6])  # 5, 6: beam 64 x 5
 def test_upstream_shaped_greedy_loop_reproduces_the_reference_streams(ref_vectors, case_index):
     import recurrent_drafting_amd as rd
 
@@ -118,7 +118,7 @@ def _rand_stream(seed):
     return draw
 
 
-@pytest.mark.parametrize("case_index", [0, 1, 2])
+@pytest.mark.parametrize("case_index", [0, 1, 2, 3])  # 3: beam 64 x 5
 def test_sampling_loops_reproduce_the_reference_streams(ref_vectors, case_index):
     """torch.rand a fixed CPU stream and Categorical the mode, exactly as when the reference wrote
     the vectors: the upstream-shaped loop on the drop-ins and the fused loop give its tokens."""

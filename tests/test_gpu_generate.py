@@ -39,7 +39,7 @@ def _run(llm, drafter, ids, max_length, W, L, eos=None):
     return steps, ledger
 
 
-@pytest.mark.parametrize("case_index", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("case_index", [0, 1, 2, 3, 4, 5, 6])  # 5, 6: beam 64 x 5, certain ties in the first iteration
 def test_generate_matches_reference_token_streams(ref_vectors, case_index):
     case = ref_vectors["end_to_end"][case_index]
     c = case["config"]

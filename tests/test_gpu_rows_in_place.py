@@ -207,13 +207,19 @@ def test_timing_sample_times_every_nth_launch():
 
 
 def test_stream_tiles_probe_reads_what_it_is_given_and_refuses_the_rest():
-    """The memory-side yardstick of the attention (rd_stream_tiles_probe): every depth folds the same
-    tiles into the same checksum, a slab shorter than its tiles is refused before anything runs."""
-    import ctypes as C
+    """The memory-side yardstick of the attention (bench_stream_tiles of the bench-only library that
+    kernel_bench.py loads): every depth folds the same tiles into the same checksum, a slab shorter
+    than its tiles is refused before anything runs."""
+    import os
+    import sys
+
+    import numpy as np
     from recurrent_drafting_amd import _hip
 
-    lib = _hip.lib()
-    import numpy as np
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import kernel_bench
+
+    lib = kernel_bench.bench_library()
 
     slabs, tiles, rows = 6, 8, 8 * 64 + 7  # (a whole number of rounds for every depth: the probe repeats its last tile otherwise)
     k = torch.randint(-2**31, 2**31 - 1, (slabs, rows, 64), dtype=torch.int32, device="cuda")  # 256-byte rows
@@ -222,10 +228,11 @@ def test_stream_tiles_probe_reads_what_it_is_given_and_refuses_the_rest():
     want = np.bitwise_xor.reduce(words, axis=1)
     for depth in (1, 2, 4):
         sink = torch.zeros(slabs * 512, dtype=torch.int32, device="cuda")
-        _hip.check(lib.rd_stream_tiles_probe(_hip.ptr(k), _hip.ptr(v), rows * 256, slabs, tiles, depth, _hip.ptr(sink), _hip.stream()))
+        assert lib.bench_stream_tiles(_hip.ptr(k), _hip.ptr(v), rows * 256, slabs, tiles, depth, _hip.ptr(sink), 1, _hip.stream(), None) == 0
+        torch.cuda.synchronize()
         got = np.bitwise_xor.reduce(sink.view(slabs, 512).cpu().numpy(), axis=1)
         assert np.array_equal(got, want), depth
     sink = torch.zeros(slabs * 512, dtype=torch.int32, device="cuda")
-    assert lib.rd_stream_tiles_probe(_hip.ptr(k), _hip.ptr(v), tiles * 64 * 256 - 16, slabs, tiles, 2, _hip.ptr(sink), None) == -1
-    assert lib.rd_stream_tiles_probe(_hip.ptr(k), _hip.ptr(v), rows * 256, slabs, tiles, 3, _hip.ptr(sink), None) == -2
-    assert lib.rd_stream_tiles_probe(None, _hip.ptr(v), rows * 256, slabs, tiles, 2, _hip.ptr(sink), None) == -1
+    assert lib.bench_stream_tiles(_hip.ptr(k), _hip.ptr(v), tiles * 64 * 256 - 16, slabs, tiles, 2, _hip.ptr(sink), 1, None, None) == -1
+    assert lib.bench_stream_tiles(_hip.ptr(k), _hip.ptr(v), rows * 256, slabs, tiles, 3, _hip.ptr(sink), 1, None, None) == -2
+    assert lib.bench_stream_tiles(None, _hip.ptr(v), rows * 256, slabs, tiles, 2, _hip.ptr(sink), 1, None, None) == -1

@@ -91,7 +91,7 @@ def _models(llama_sd, drafter_sd):
     return llm.eval(), drafter.eval()
 
 
-@pytest.mark.parametrize("case_index", [0, 1, 2])
+@pytest.mark.parametrize("case_index", [0, 1, 2, 3])  # 3: beam 64 x 5, wider than the top-50 filter
 def test_sampling_streams_match_the_reference(ref_vectors, case_index):
     """The reference's own sampling decode loop (CPU, float32; torch.rand a fixed stream, the
     categorical draw replaced by the mode) produced these token streams."""

@@ -96,9 +96,12 @@ def test_beam_search_matches_chain_oracle():
     assert torch.equal(beams, o_beams) and torch.allclose(hist, o_hist, atol=1e-6)
 
 
-@pytest.mark.parametrize("case_index", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("case_index", [0, 1, 2, 3, 4, 5, 6])
 def test_generate_matches_reference_token_streams(ref_vectors, case_index):
-    """The reference's own greedy decode loop (CPU, float32) produced these streams."""
+    """The reference's own greedy decode loop (CPU, float32) produced these streams.  Cases 5 and 6
+    have beams wider than the top-50 filter (64 x 5): the first beam-search iteration then ends in
+    certain ties among filtered tokens, whose order torch.topk leaves open -- the streams must not
+    depend on it (the tied beams are gone after the second iteration)."""
     case = ref_vectors["end_to_end"][case_index]
     c = case["config"]
     if c.get("markov"):
