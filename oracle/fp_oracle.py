@@ -13,6 +13,15 @@ rounded after the max subtraction, the mask value -50000 becomes -49920, log_sof
 output to the input dtype, and only the beam score is float32 (the running score is created as
 float32 at modeling_drafter.py:170-172, and bf16 + fp32 promotes to fp32).
 
+log_softmax of a 16-bit tensor is a library routine whose last bit depends on the device: torch's
+GPU kernel forms x - (max + log(sum)) in float32 and rounds the result once, its CPU kernel rounds
+max + log(sum) to the 16-bit type first and the difference again (31 % of the surviving entries of
+a flat row end up one bf16 step away from the correctly rounded value).  The reference runs its
+16-bit models on a GPU, so `log_softmax_rounded_once` below takes the GPU kernel's rule: float32
+arithmetic, one rounding.  Pinned by a float64 computation rounded once
+(tests/test_oracle_fp.py) and, on the GPU box, by torch's own GPU log_softmax on the same tensor
+(tests/test_gpu_beam.py).
+
 Tie rule.  torch.topk leaves the order of equal elements unspecified and equal scores are certain
 here (every filtered entry of a row has the same score).  The oracle, like the HIP kernel, breaks
 ties by the LOWEST flat index (beam * V + token); comparisons with any other implementation are on
@@ -78,6 +87,11 @@ def warp_logits(x: torch.Tensor, top_k: int = 50, mask_value: float = LOG_0) -> 
     return torch.where(x < thr, torch.tensor(mask_value, dtype=x.dtype), x)
 
 
+def log_softmax_rounded_once(x: torch.Tensor) -> torch.Tensor:
+    """log_softmax over the last axis in float32, rounded once to x's dtype (torch's GPU kernel)."""
+    return x.float().log_softmax(dim=-1).to(x.dtype)
+
+
 def stable_topk(scores: torch.Tensor, k: int):
     """Top-k along the last dim, sorted descending, equal scores in increasing index order."""
     order = torch.sort(scores, dim=-1, descending=True, stable=True)
@@ -90,7 +104,7 @@ def beam_search_step(logits: torch.Tensor, log_p_beam: torch.Tensor):
     Returns (new_log_p_beam (B,W) f32 sorted descending, token (B,W) i64, parent (B,W) i64,
     log_p_new_token (B,W,V) in logits' dtype)."""
     B, W, V = logits.shape
-    logp = warp_logits(maintain_logits(logits)).log_softmax(dim=-1)
+    logp = log_softmax_rounded_once(warp_logits(maintain_logits(logits)))
     scores = logp + log_p_beam.unsqueeze(-1)  # promotes to float32
     top, idx = stable_topk(scores.reshape(B, W * V), W)
     return top, idx % V, idx // V, logp

@@ -69,6 +69,8 @@ class StepReport:
     shifts: List[int]  # cache row shifts going into the step
     context_err: float
     kv_err: float
+    context_err_bf16_torch: float = 0.0  # the same two figures for the restatement in the model's dtype
+    kv_err_bf16_torch: float = 0.0
 
 
 @dataclasses.dataclass
@@ -209,7 +211,7 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
             assert len(drafts) == k + 2
             if k == 0:
                 with torch.inference_mode():
-                    report = check_prefill(prefilled, llm, llm32, pad, tol)
+                    report = check_prefill(prefilled, llm, llm32, pad, tol, log=print)
                 prefilled.clear()
                 if prefill_report is not None:
                     prefill_report.append(report)
@@ -228,7 +230,7 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
     return reports
 
 
-def check_prefill(pf, llm, llm32, pad: int, tol: float) -> PrefillReport:
+def check_prefill(pf, llm, llm32, pad: int, tol: float, log: Optional[Callable] = None) -> PrefillReport:
     """The prefill of the HIP loop against oracle/torch_path's in float32 on the same token ids."""
     ids, rows = pf["ids"], pf["rows"]  # rows: (layers, 2, B, Hkv, S, D), the reference's layout
     dev = ids.device
@@ -247,15 +249,25 @@ def check_prefill(pf, llm, llm32, pad: int, tol: float) -> PrefillReport:
     torch_rows, torch_state, _ = restate(llm, rows.dtype)
     live = (torch.arange(S, device=dev)[None, :] >= pads[:, None])[None, None, :, None, :, None]
     zero = torch.zeros((), device=dev)
-    kv_scale = float(torch.where(live, want_rows, zero).abs().max())
-    kv_err = float(torch.where(live, rows.float() - want_rows, zero).abs().max()) / kv_scale
-    kv_yard = float(torch.where(live, torch_rows - want_rows, zero).abs().max()) / kv_scale
-    assert kv_err <= tol, f"prefill: cache rows off by {kv_err:.3g} of their scale"
-    assert kv_err <= 3 * kv_yard + 1e-3, f"prefill: cache rows {kv_err:.3g} off, stock torch only {kv_yard:.3g}"
+    # per layer (errors grow through the residual stream), each against the layer's own scale
+    per_layer = lambda x: torch.where(live, x, zero).abs().amax(dim=(1, 2, 3, 4, 5))
+    layer_scale = per_layer(want_rows)
+    layer_err = per_layer(rows.float() - want_rows) / layer_scale
+    layer_yard = per_layer(torch_rows - want_rows) / layer_scale
+    kv_err, kv_yard = float(layer_err.max()), float(layer_yard.max())
     state_scale = float(want_state.abs().max())
     state_err = float((pf["state"].float() - want_state).abs().max()) / state_scale
     state_yard = float((torch_state - want_state).abs().max()) / state_scale
-    assert state_err <= tol, f"prefill: last hidden state off by {state_err:.3g} of its scale"
+    if log is not None:
+        log("prefill cache rows, error by layer (HIP / stock torch in the model's dtype): " + " ".join(
+            f"{i}:{float(layer_err[i]):.1e}/{float(layer_yard[i]):.1e}" for i in sorted({0, n_layers // 4, n_layers // 2, 3 * n_layers // 4, n_layers - 1})))
+        log(f"prefill last hidden state {state_err:.2e} (stock torch {state_yard:.2e})")
+    # `tol` of the scale, or what stock torch's own ops in this dtype make of the same inputs (at
+    # depth the rounding of 16-bit residual streams is the larger of the two)
+    assert bool((layer_err <= torch.clamp(3 * layer_yard + 1e-3, min=tol)).all()), \
+        f"prefill: cache rows off by {kv_err:.3g} of their scale, stock torch {kv_yard:.3g}"
+    assert bool((layer_err <= 3 * layer_yard + 1e-3).all()), f"prefill: cache rows {kv_err:.3g} off, stock torch only {kv_yard:.3g}"
+    assert state_err <= max(tol, 3 * state_yard + 1e-3), f"prefill: last hidden state off by {state_err:.3g} of its scale"
     assert state_err <= 3 * state_yard + 1e-3, f"prefill: last hidden state {state_err:.3g} off, stock torch only {state_yard:.3g}"
     o_tok = want_logits.argmax(dim=-1)
     flipped = (pf["token"] != o_tok).nonzero().flatten()
@@ -274,8 +286,8 @@ def _check_beam_iterations(k, iterations) -> float:
         logits, lpb = rec["logits"].cpu(), rec["lpb"].cpu()
         o_lpb, o_tok, o_par, o_logp = O.beam_search_step(logits, lpb)
         live = o_logp.float() > -1000
-        # one rounding step of a log-probability in the drafter's dtype (float32: of the score near 50000)
-        tol = 2e-2 * float(o_logp.float()[live].abs().max()) if logits.dtype != torch.float32 else 1e-2
+        # one rounding step of a log-probability in the drafter's dtype (float32: of a score near 50000)
+        tol = 2.0 ** -7 * float(o_logp.float()[live].abs().max()) if logits.dtype != torch.float32 else 1e-2
         try:
             shared = beam_band.check_selection(o_logp, lpb, o_lpb, o_tok, o_par, rec["new_lpb"], rec["tok"], rec["par"], tol)
         except AssertionError as e:
@@ -306,7 +318,7 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
     assert torch.equal(beams[:, :, 0], draft_in["init"][:, None].expand(B, W))
     assert len(draft_in["iterations"]) == L - 1
     beam_picks_shared = _check_beam_iterations(k, draft_in["iterations"])
-    assert beam_picks_shared >= 0.9, f"step {k}: only {beam_picks_shared:.2f} of the HIP picks are the oracle's on the same logits"
+    assert beam_picks_shared >= 0.97, f"step {k}: only {beam_picks_shared:.3f} of the HIP picks are the oracle's on the same logits"
 
     # -- tree of the HIP beams: bit-exact ----------------------------------------------------------
     o_packed, o_unpacker, o_mask, o_off = P.pack(beams, (ids != pad).to(ids.dtype))
@@ -333,7 +345,7 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
         return logits.flatten(0, 1)[slot_of_row], hidden.flatten(0, 1)[slot_of_row], cache
 
     want, want_hidden, o_cache = restate(llm32, torch.float32)
-    torch_bf16, _, _ = restate(llm, snap.dtype)
+    torch_bf16, torch_hidden, torch_cache = restate(llm, snap.dtype)
     got = st["logits"][:total].float()
     scale = float(want.abs().max())
     logits_err = float((got - want).abs().max()) / scale
@@ -378,6 +390,8 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
     ctx_want = ctx_want[b_idx * n_q + st["last_slot"]]
     ctx_scale = float(want_hidden.abs().max())
     context_err = float((draft_next["context"].float() - ctx_want).abs().max()) / ctx_scale
+    ctx_torch = torch_hidden.new_zeros((B * n_q, torch_hidden.shape[1])).index_copy_(0, slot_of_row, torch_hidden)
+    context_yard = float((ctx_torch[b_idx * n_q + st["last_slot"]].float() - ctx_want).abs().max()) / ctx_scale
     assert context_err <= tol, f"step {k}: drafter context off by {context_err:.3g}"
 
     # -- KV cache: the rows the HIP forward wrote against the restatement's; the rows kept and moved ----
@@ -386,6 +400,8 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
     live = (torch.arange(n_q, device=dev)[None, :] < counts[:, None])[None, None, :, None, :, None]
     kv_scale = float(o_new.abs().max())
     kv_err = float(torch.where(live, hip_new - o_new, torch.zeros_like(o_new)).abs().max()) / kv_scale
+    kv_yard = float(torch.where(live, torch_cache.data[:, :, :, :, prev : prev + n_q].float() - o_new,
+                                torch.zeros_like(o_new)).abs().max()) / kv_scale
     assert kv_err <= tol, f"step {k}: appended K/V rows off by {kv_err:.3g}"
     if prev_step is not None:
         # what the previous step kept: its live columns, then the accepted rows of its chosen beam,
@@ -404,4 +420,4 @@ def _check_step(k, st, draft_in, draft_next, out, max_length, llm, llm32, drafte
                     f"step {k}: accepted cache row {j} of row {b}"
             assert lo + keep + int(p["n"][b]) + 1 == prev
     return StepReport(k, prev, n_q, total, beams_equal, beams_shared, beam_picks_shared, logits_err, yard, int(flipped.numel()), worst,
-                      n.tolist(), st["shift"].tolist(), context_err, kv_err)
+                      n.tolist(), st["shift"].tolist(), context_err, kv_err, context_yard, kv_yard)

@@ -107,14 +107,21 @@ def test_step_bf16_rounding_points_ties_by_lowest_index_rule(B, W, V, t, spread,
     o_lpb, o_tok, o_par, o_logp = O.beam_search_step(logits, lpb)
     live = o_logp.float() > -1000
     diff = (logp - o_logp.float()).abs()
-    step = 2e-2 * o_logp.float()[live].abs().max().item()
+    step = 2.0 ** -7 * o_logp.float()[live].abs().max().item()  # one bf16 step of the largest magnitude
     assert diff.max() <= step
     # the filtered class stays one finite constant per row, about -49920 - log(sum)
     assert logp[0, 0].min().item() < -49000
+    # one rounding of the float32 result: all but a few entries (those whose float32 value sits within
+    # a float32 step of a bf16 rounding boundary) have the oracle's bits -- and the bits that torch's own
+    # GPU log_softmax gives for the same tensor, which is the reference's op on this device
+    assert (diff[live] > 0).float().mean() <= 1e-3, (diff[live] > 0).float().mean()
+    y = O.warp_logits(O.maintain_logits(logits))
+    torch_gpu = torch.log_softmax(y.cuda(), dim=-1).float().cpu()
+    assert (torch_gpu[live] != logp[live]).float().mean() <= 1e-3
     if diff.max() == 0:
         assert torch.equal(tok, o_tok) and torch.equal(par, o_par) and torch.equal(new_lpb, o_lpb)
     shared = beam_band.check_selection(o_logp, lpb, o_lpb, o_tok, o_par, new_lpb, tok, par, tol=step)
-    assert shared >= 0.9, shared
+    assert shared >= 0.97, shared
     rows = torch.arange(B)[:, None]
     assert torch.equal(new_beams[..., :-1], beams[rows, par]) and torch.equal(new_beams[..., -1], tok)
 
@@ -133,10 +140,10 @@ def test_step_fp16_values_differ_below_the_upper_half_of_the_float(force_fallbac
     new_lpb, tok, par, new_beams, logp = _step(logits, lpb, beams, True, force_fallback)
     o_lpb, o_tok, o_par, o_logp = O.beam_search_step(logits, lpb)
     live = o_logp.float() > -1000
-    step = 2e-3 * o_logp.float()[live].abs().max().item()
+    step = 2.0 ** -10 * o_logp.float()[live].abs().max().item()  # one fp16 step of the largest magnitude
     assert (logp - o_logp.float()).abs()[live].max() <= step
     shared = beam_band.check_selection(o_logp, lpb, o_lpb, o_tok, o_par, new_lpb, tok, par, tol=step)
-    assert shared >= 0.9, shared
+    assert shared >= 0.97, shared
 
 
 def test_step_many_ties_by_lowest_index_rule_overflow_to_exact_path():

@@ -76,7 +76,7 @@ def _summary(reports):
         f"picks on the same logits {r.beam_picks_shared:.3f} "
         f"logits {r.logits_err:.2e} (torch bf16 {r.logits_err_bf16_torch:.2e}) flips {r.flips} "
         f"(margin {r.worst_flip_margin:.1e}) n {r.n_tokens} shift {r.shifts} ctx {r.context_err:.1e} "
-        f"kv {r.kv_err:.1e}" for r in reports)
+        f"(torch {r.context_err_bf16_torch:.1e}) kv {r.kv_err:.1e} (torch {r.kv_err_bf16_torch:.1e})" for r in reports)
 
 
 def test_bf16_mfma_decode_loop_teacher_forced_with_accepted_drafts():
@@ -144,7 +144,7 @@ def test_bf16_7b_shape_one_layer_teacher_forced_steps_at_long_context():
     assert all(r.prev >= 1500 and r.n_q >= 100 for r in reports)
     # (beams_shared compares with a beam search on logits from GEMMs of other shapes and is only
     # reported; what is asserted is every iteration's selection on the same logits)
-    assert all(r.beam_picks_shared >= 0.9 for r in reports)
+    assert all(r.beam_picks_shared >= 0.97 for r in reports)
     assert any(any(x != 0 for x in r.shifts) for r in reports)
 
 
@@ -167,17 +167,22 @@ def test_bf16_7b_shape_all_32_layers_prefill_and_teacher_forced_steps():
     ids = ids.cuda()
     pre = []
     reports, kernels = _uses_mfma_kernel(
-        lambda: teacher_forced.run(llm, drafter, ids, S + 48, 45, 5, steps=4, check_from=2, tol=4e-2,
+        lambda: teacher_forced.run(llm, drafter, ids, S + 48, 45, 5, steps=4, check_from=2, tol=0.15,
                                    force=teacher_forced.forced_acceptance(6), prefill_report=pre))
     print(_prefill_summary(pre))
     print(_summary(reports))
     assert "attn_mfma_kernel" in kernels and "attn_generic_kernel" not in kernels
     assert len(reports) == 2 and pre[0].seq == S
     assert all(r.prev >= 600 and r.n_q >= 100 for r in reports)
-    assert all(r.beam_picks_shared >= 0.9 for r in reports)
+    assert all(r.beam_picks_shared >= 0.97 for r in reports)
     assert any(any(x != 0 for x in r.shifts) for r in reports)
-    # the composition of 32 layers stays as close to float32 as stock torch's bf16 ops do
-    assert all(r.logits_err <= 3 * r.logits_err_bf16_torch + 1e-3 for r in reports)
+    # The composition of 32 layers stays as close to float32 as stock torch's bf16 ops do: at this
+    # depth the bar is not a fixed share of the scale (the run above only caps the error at 0.15 of it)
+    # but three times what the same op sequence in stock torch bf16 makes of the same inputs
+    for r in reports:
+        assert r.logits_err <= 3 * r.logits_err_bf16_torch + 1e-3, (r.logits_err, r.logits_err_bf16_torch)
+        assert r.kv_err <= 3 * r.kv_err_bf16_torch + 1e-3, (r.kv_err, r.kv_err_bf16_torch)
+        assert r.context_err <= 3 * r.context_err_bf16_torch + 1e-3, (r.context_err, r.context_err_bf16_torch)
 
 
 def test_bf16_mfma_sampling_loop_accepts_as_the_oracle_does_on_the_same_logits():

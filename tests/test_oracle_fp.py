@@ -134,3 +134,18 @@ def test_beam_search_matches_reference_vectors(ref_vectors):
         assert torch.allclose(picked, torch.tensor(c["log_prob_of_drafted"]), atol=1e-5)
         assert torch.allclose(hist.max(-1).values, torch.tensor(c["log_prob_row_max"]), atol=1e-5)
         assert torch.allclose(hist.min(-1).values, torch.tensor(c["log_prob_row_min"]), atol=1e-2)
+
+
+def test_log_softmax_of_16_bit_rows_is_rounded_once():
+    """The float64 value rounded once to bf16 / fp16 is what the oracle returns (torch's GPU rule);
+    torch's CPU kernel for 16-bit types, which rounds max + log(sum) first, is up to a step away."""
+    torch.manual_seed(0)
+    for dtype in (torch.bfloat16, torch.float16):
+        x = O.warp_logits(O.maintain_logits((torch.randn(6, 4000) * 0.05).to(dtype)))
+        want = (x.double() - torch.logsumexp(x.double(), dim=-1, keepdim=True)).to(dtype)
+        got = O.log_softmax_rounded_once(x)
+        live = want.float() > -1000
+        assert got.dtype == dtype and torch.equal(got[live], want[live])
+        assert torch.allclose(got.float(), want.float(), rtol=1e-6, atol=0)  # (the filtered class: sums near 50000)
+    x32 = torch.randn(3, 100)
+    assert torch.equal(O.log_softmax_rounded_once(x32), x32.log_softmax(-1))
