@@ -18,7 +18,10 @@ prompts of 1500 and 2500 tokens; `ragged_acceptance`: prompts of 1200 tokens wit
 decision replaced by random accepted lengths, so that rows shift, accepted rows are appended and
 the trees grow -- random-init models accept nothing by themselves; `ragged_prompts`: prompts of 500
 to 2500 tokens in one batch, left-padded; `rope_attention_launches`: the
-headline's step with the opt-in fused rotation + append + attention kernel against the default two).
+headline's step with the opt-in fused rotation + append + attention kernel against the default two;
+`sampling`: speculative sampling at temperature 1 on the headline's models and prompts, and on the
+Llama-2-13B shape at batch 16, prompt 256, beam 64 x 5 -- step time, synchronised stage times and
+the event times of the kernels of the sampling path).
 """
 
 from __future__ import annotations
@@ -51,17 +54,24 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_models(device: str, dtype: torch.dtype, n_layers: int, seed: int):
+# configuration 5 of the benchmark plan: Llama-2-13B shape, batch 16, prompt 256, beam 64 x 5, T = 1
+LLAMA_13B = dict(LLAMA_7B, hidden_size=5120, intermediate_size=13824, num_hidden_layers=40,
+                 num_attention_heads=40, num_key_value_heads=40)
+DRAFTER_13B = dict(DRAFTER_7B, hidden_size=5120, exit_dim=10240)
+
+
+def build_models(device: str, dtype: torch.dtype, n_layers: int, seed: int, llama_cfg=None, drafter_cfg=None):
     """Random-init pair; every weight N(0, 0.02) from one seeded generator, norm gains 1."""
     import recurrent_drafting_amd as rd
     from transformers.models.llama.configuration_llama import LlamaConfig
 
+    llama_cfg, drafter_cfg = llama_cfg or LLAMA_7B, drafter_cfg or DRAFTER_7B
     prev = torch.get_default_dtype()
     torch.set_default_dtype(dtype)
     try:
         with torch.device(device):
-            llm = rd.modeling_llama.LlamaForCausalLM(LlamaConfig(**dict(LLAMA_7B, num_hidden_layers=n_layers)))
-            drafter = rd.modeling_drafter.Drafter(rd.configuration_drafter.DrafterConfig(**DRAFTER_7B))
+            llm = rd.modeling_llama.LlamaForCausalLM(LlamaConfig(**dict(llama_cfg, num_hidden_layers=n_layers)))
+            drafter = rd.modeling_drafter.Drafter(rd.configuration_drafter.DrafterConfig(**drafter_cfg))
     finally:
         torch.set_default_dtype(prev)
     gen = torch.Generator(device=device).manual_seed(seed)
@@ -75,9 +85,9 @@ def build_models(device: str, dtype: torch.dtype, n_layers: int, seed: int):
     return llm.eval(), drafter.eval()
 
 
-def prompts(device: str, length: int = PROMPT) -> torch.Tensor:
+def prompts(device: str, length: int = PROMPT, batch: int = BATCH) -> torch.Tensor:
     gen = torch.Generator(device="cpu").manual_seed(SEED)
-    return torch.randint(1, LLAMA_7B["vocab_size"], (BATCH, length), generator=gen).to(device)
+    return torch.randint(1, LLAMA_7B["vocab_size"], (batch, length), generator=gen).to(device)
 
 
 # -------------------------------------------------------------------------------------------------
@@ -104,10 +114,12 @@ def forced_acceptance(seed: int):
     return force
 
 
-def timed_decode(model, ids, steps: int, warmup: int, max_new: int, force=None):
+def timed_decode(model, ids, steps: int, warmup: int, max_new: int, force=None, temperature=None,
+                 beam=(WIDTH, LENGTH)):
     """Runs warmup + steps decode steps of one generation (a new one is started, prefill untimed,
     whenever the cap is reached) and returns the timing of the `steps` steps, the shapes of the
-    attention launches in them and the HIP-event time of every TIMED_EVERY-th of those launches."""
+    attention launches in them and the HIP-event time of every TIMED_EVERY-th of those launches.
+    temperature None: greedy; a number: speculative sampling at that temperature."""
     import recurrent_drafting_amd as rd
     from recurrent_drafting_amd import _hip, acceptance, attention
 
@@ -119,8 +131,8 @@ def timed_decode(model, ids, steps: int, warmup: int, max_new: int, force=None):
         ledger = rd.stats.Ledger(sync=False)
 
         def new_stream():
-            return model.generate(ledger, ids, max_length, rd.BeamShape(WIDTH, LENGTH),
-                                  rd.SamplingArgs(1.0, True), rd.SpecialTokens(0, None))
+            sampling = rd.SamplingArgs(1.0, True) if temperature is None else rd.SamplingArgs(float(temperature), False)
+            return model.generate(ledger, ids, max_length, rd.BeamShape(*beam), sampling, rd.SpecialTokens(0, None))
 
         stream = new_stream()
         for _ in range(warmup):
@@ -172,9 +184,46 @@ def timed_decode(model, ids, steps: int, warmup: int, max_new: int, force=None):
         acceptance.greedy_accept = real_accept
     accepted = [a for rec in ledger.records for a in rec.get("avg_num_accepted", [])]
     per_seq_tokens = sum(a + 1 for a in accepted) / max(len(accepted), 1)
-    return dict(elapsed=elapsed, steps=timed, per_seq_tokens=per_seq_tokens, tokens=per_seq_tokens * BATCH * timed,
+    cfg = model.llm.config
+    return dict(elapsed=elapsed, steps=timed, per_seq_tokens=per_seq_tokens, tokens=per_seq_tokens * ids.shape[0] * timed,
                 dominant=dominant, shapes=shapes, context=(first_len, last_len), final_left_pads=final_pads,
-                first_left_pads=first_pads)
+                first_left_pads=first_pads, heads=cfg.num_attention_heads,
+                head_dim=cfg.hidden_size // cfg.num_attention_heads)
+
+
+def synchronised_steps(model, ids, max_length, beam, temperature, warm: int = 2, steps: int = 4):
+    """A few steps under the reference's synchronised stage timers, with every kernel of the library
+    event-timed: -> (mean seconds per stage, {kernel: (launches, total ms)}, the ledger)."""
+    import recurrent_drafting_amd as rd
+    from recurrent_drafting_amd import _hip
+
+    ledger = rd.stats.Ledger(sync=True)
+    sampling = rd.SamplingArgs(1.0, True) if temperature is None else rd.SamplingArgs(float(temperature), False)
+    stream = model.generate(ledger, ids, max_length, rd.BeamShape(*beam), sampling, rd.SpecialTokens(0, None))
+    for _ in range(warm):
+        next(stream)
+    _hip.timing_enable(True)
+    for _ in range(steps):
+        next(stream)
+    torch.cuda.synchronize()
+    kernels = _hip.timing_collect()
+    _hip.timing_enable(False)
+    stream.close()
+    rec = ledger.records[0]
+    for key in ("step", "input_id_length", "avg_num_accepted"):  # drop the warm-up steps
+        rec[key] = rec[key][warm:]
+    rec["wall_times"] = {k: v[warm:] for k, v in rec["wall_times"].items()}
+    stage = {k: sum(v) / len(v) for k, v in rec["wall_times"].items()}
+    return stage, kernels, ledger
+
+
+def sampling_point(model, ids, extra_steps: int, warmup: int, beam):
+    """Speculative sampling at temperature 1 on the given models and prompts: the free-running step
+    time, then the synchronised stage times and the kernels of the sampling path on a few more steps."""
+    run = timed_decode(model, ids, extra_steps, warmup, 64 + 5 * (extra_steps + warmup), temperature=1.0, beam=beam)
+    stage, kernels, _ = synchronised_steps(model, ids, ids.shape[1] + 64, beam, 1.0)
+    run.update(stage=stage, kernels=kernels)
+    return run
 
 
 def gpu_run(steps: int, warmup: int, extra_steps: int):
@@ -232,29 +281,35 @@ def gpu_run(steps: int, warmup: int, extra_steps: int):
         finally:
             modeling_llama.LlamaAttention.fused_rope_attention = default
 
+        # speculative sampling at temperature 1 on the headline's models and prompts (the kernels of
+        # recurrent_drafting.py:75-111, :499-556: row statistics of the packed logits, acceptance,
+        # residual distribution; the float32 log-probability history of the drafter)
+        r = sampling_point(model, prompts(dev, PROMPT), extra_steps, warmup, (WIDTH, LENGTH))
+        r["null_us"] = run["null_us"]
+        others["sampling_temperature_1"] = r
+        log(f"[bench] sampling at temperature 1: {r['elapsed'] / r['steps'] * 1e3:.2f} ms/step, "
+            f"{r['per_seq_tokens']:.2f} tokens per sequence and step")
+
     # ---- stage breakdown with the reference's synchronised timers, on a few extra steps ---------------
-    ledger2 = rd.stats.Ledger(sync=True)
-    ids = prompts(dev, PROMPT)
-    s2 = model.generate(ledger2, ids, PROMPT + NEW_TOKENS, rd.BeamShape(WIDTH, LENGTH),
-                        rd.SamplingArgs(1.0, True), rd.SpecialTokens(0, None))
-    next(s2)
-    next(s2)
-    _hip.timing_enable(True)  # every kernel of the library, on four steps
-    for _ in range(4):
-        next(s2)
-    torch.cuda.synchronize()
-    kernels = _hip.timing_collect()
-    _hip.timing_enable(False)
-    s2.close()
-    rec = ledger2.records[0]
-    for key in ("step", "input_id_length", "avg_num_accepted"):  # drop the two warm-up steps
-        rec[key] = rec[key][2:]
-    rec["wall_times"] = {k: v[2:] for k, v in rec["wall_times"].items()}
-    stage = {k: sum(v) / len(v) for k, v in rec["wall_times"].items()}
+    stage, kernels, ledger2 = synchronised_steps(model, prompts(dev, PROMPT), PROMPT + NEW_TOKENS, (WIDTH, LENGTH), None)
     table, _ = rd.stats.summarize(ledger2, BATCH, LENGTH - 1)  # the reference's own summary (stats.py:158-215)
     run.update(kernels=kernels, stage=stage, ref_style_tokens_per_second=table.tokens_per_second, others=others)
     del model, llm, drafter
     torch.cuda.empty_cache()
+
+    # ---- configuration 5: Llama-2-13B shape, batch 16, prompt 256, beam 64 x 5, sampling at T = 1 -------
+    if extra_steps > 0:
+        t0 = time.perf_counter()
+        llm, drafter = build_models(dev, torch.bfloat16, LLAMA_13B["num_hidden_layers"], SEED + 1, LLAMA_13B, DRAFTER_13B)
+        model = rd.RecurrentDrafting(llm, drafter)
+        torch.cuda.synchronize()
+        log(f"[bench] 13B-shaped models in {time.perf_counter() - t0:.1f}s")
+        r = sampling_point(model, prompts(dev, 256, batch=16), extra_steps, warmup, (64, 5))
+        r["null_us"] = run["null_us"]
+        others["llama_13b_shape_batch_16_beam_64x5_sampling"] = r
+        log(f"[bench] 13B shape, batch 16, beam 64x5, sampling: {r['elapsed'] / r['steps'] * 1e3:.2f} ms/step")
+        del model, llm, drafter
+        torch.cuda.empty_cache()
     return run
 
 
@@ -267,7 +322,7 @@ def attention_roofline(run):
     TIMED_EVERY-th launch of the timed region (the shapes are those of the same launches).
     Arithmetic intensity below the machine balance (2500 TFLOP/s / 8 TB/s = 312 FLOP/B) means the
     HBM roof binds, above it the MFMA roof."""
-    H, D = LLAMA_7B["num_attention_heads"], LLAMA_7B["hidden_size"] // LLAMA_7B["num_attention_heads"]
+    H, D = run.get("heads", LLAMA_7B["num_attention_heads"]), run.get("head_dim", 128)
     count, total_ms = run["dominant"].get("attn_mfma_kernel", (0, 0.0))
     launched = len(run["shapes"])
     shapes = run["shapes"][::TIMED_EVERY][:count] if count else []  # the launches that were timed
@@ -314,6 +369,20 @@ def attention_roofline(run):
         mean_query_rows=round(sum(r for (_, _, _, r) in shapes) / len(shapes), 1),
         mean_kv_len=round(sum(kv for (_, _, kv, _) in shapes) / len(shapes), 1),
     )
+    return out
+
+
+SAMPLING_KERNELS = ("row_stats_kernel", "accept_sample_kernel", "residual_probs_kernel", "gather_rows_kernel",
+                    "beam_row_kernel", "beam_merge_kernel", "attn_mfma_kernel")
+
+
+def sampling_summary(run):
+    """A sampling operating point: summary_of plus the synchronised times of the sampling-only stages
+    and the event times of the kernels on the sampling path."""
+    out = summary_of(run)
+    out["stage_seconds_synchronised"] = {k: round(v, 6) for k, v in run["stage"].items()}
+    out["kernel_avg_us"] = {k: round(ms * 1e3 / n, 2) for k, (n, ms) in sorted(run["kernels"].items())
+                            if k in SAMPLING_KERNELS and n}
     return out
 
 
@@ -540,6 +609,9 @@ def main():
         "ragged_acceptance": {k: summary_of(r) for k, r in run["others"].items() if k.startswith("ragged_")},
         "ragged_prompts": {k: dict(summary_of(r), prompt_tokens=r["prompt_tokens"]) for k, r in run["others"].items()
                            if k.startswith("prompts_of_")},
+        # speculative sampling (temperature 1): the headline's models and prompts, and the Llama-2-13B
+        # shape at batch 16 with beam 64 x 5 (configuration 5 of the benchmark plan)
+        "sampling": {k: sampling_summary(r) for k, r in run["others"].items() if "sampling" in k},
         # opt-in fused kernel against the default pair of kernels, same prompts, back to back (the
         # fused launch also rotates q and k and appends k and v: its time is not the attention's alone)
         "rope_attention_launches": {
