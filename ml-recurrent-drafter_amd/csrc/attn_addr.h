@@ -25,9 +25,12 @@ constexpr int kKBuffers = 3;               // K tiles in LDS: K(t+1) is multipli
 constexpr int kVBuffers = 2;               // V tiles in LDS: V(t) is multiplied while V(t+1) is staged
 constexpr int kRing = 2;                   // register stages of tiles on their way from memory
 constexpr int kKsStride = kD + 8;          // bf16 elements; 272-byte rows spread 16 lanes over all banks
-constexpr int kVtStride = kTile + 8;       // bf16 elements; 144-byte rows: 16-byte aligned, conflict-free
+// V tiles lie in LDS as they lie in memory, one key per row; the V^T fragments of the second product
+// come out of transposing reads (ds_read_b64_tr_b16).  320-byte rows: the four keys and 32 dims
+// that the 32 lanes of one read cycle touch fall into 64 different banks.
+constexpr int kVsStride = kD + 32;         // bf16 elements
 constexpr int kKBytes = kKBuffers * kTile * kKsStride * 2;
-constexpr int kVBytes = kVBuffers * kD * kVtStride * 2;
+constexpr int kVBytes = kVBuffers * kTile * kVsStride * 2;
 constexpr int kLdsBytes = kKBytes + kVBytes;
 
 // How the 8 waves of a workgroup share its query rows (blocks of 32) and the 64 keys of a tile.
@@ -60,10 +63,8 @@ RD_HD WaveRole wave_role(int layout, int w) {
 }
 
 // ---- tile loads ------------------------------------------------------------------------------
-// Threads [0,256) stage K rows (keys lrow + 16*i), threads [256,512) stage V transposed (keys
-// 4*lrow + i); four 16-byte chunks each per tile.  The V threads map lanes to (chunk, key quad) so
-// that the 16 lanes of one LDS write cycle hit 16 different bank pairs: lane bits 0-1 and 4-5
-// select the chunk, bits 2-3 and 6-7 the key quad.
+// Threads [0,256) stage the K tile, threads [256,512) the V tile, both the same way: a thread
+// carries the 16-byte chunk `chunk` of the rows lrow + 16*i, i = 0..3 (16 lanes per 256-byte row).
 struct Loader {
   bool k_loader;
   int chunk;      // 16-byte column chunk of a row (0..15)
@@ -75,10 +76,10 @@ RD_HD Loader loader_of(int tid) {
   Loader ld;
   ld.k_loader = tid < kThreads / 2;
   const int lt = tid & 255;
-  ld.chunk = ld.k_loader ? (lt & 15) : ((lt & 3) | (((lt >> 4) & 3) << 2));
-  ld.lrow = ld.k_loader ? (lt >> 4) : (((lt >> 2) & 3) | ((lt >> 6) << 2));
-  ld.key_step = ld.k_loader ? 16 : 1;
-  ld.first_key = ld.k_loader ? ld.lrow : 4 * ld.lrow;
+  ld.chunk = lt & 15;
+  ld.lrow = lt >> 4;
+  ld.key_step = 16;
+  ld.first_key = ld.lrow;
   return ld;
 }
 RD_HD int n_tiles_of(int lo, int hi) { return (hi - lo + kTile - 1) / kTile; }
@@ -97,30 +98,54 @@ RD_HD int tile_chunk_key(const Loader& ld, int key0, int i, int key_min, int key
   return tile_leaves_span(key0, key_min, key_end) ? key_in_span(key, key_min, key_end) : key;
 }
 
+// L2 touch: beyond the tiles that travel in the register ring, every loader thread reads four bytes
+// of a tile further ahead, so that the line is on its way into the L2 long before the ring asks for
+// it (256 threads, the 128 lines of a tile's 64 rows of 256 bytes: two threads per line).
+RD_HD int touch_row(int tid) { return (tid & 255) >> 2; }
+RD_HD int touch_byte(int tid) { return ((tid >> 1) & 1) * 128; }
+RD_HD int touch_key(int tid, int key0, int key_min, int key_end) { return key_in_span(key0 + touch_row(tid), key_min, key_end); }
+
 // ---- LDS -------------------------------------------------------------------------------------
-// byte offsets from the start of the workgroup's LDS; K buffers first, then the V^T buffers
+// byte offsets from the start of the workgroup's LDS; K buffers first, then the V buffers
 RD_HD int lds_k_stage(const Loader& ld, int j, int i) {  // chunk i of the K tile j
   return ((j % kKBuffers) * kTile * kKsStride + (ld.lrow + 16 * i) * kKsStride + 8 * ld.chunk) * 2;
 }
-// V^T rows hold the keys of every 16-key group in the order [0-3, 8-11, 4-7, 12-15]: the eight
-// keys that one lane feeds to a 16-key MFMA step are then 16 contiguous bytes.
-RD_HD int vt_col(int lrow) { return 16 * (lrow >> 2) + 4 * (((lrow & 1) << 1) | ((lrow >> 1) & 1)); }
-RD_HD int lds_v_stage(const Loader& ld, int j, int e) {  // the four keys of element e (0..7) of the thread's chunk
-  return kKBytes + ((j % kVBuffers) * kD * kVtStride + (8 * ld.chunk + e) * kVtStride + vt_col(ld.lrow)) * 2;
+RD_HD int lds_v_stage(const Loader& ld, int j, int i) {  // chunk i of the V tile j
+  return kKBytes + ((j % kVBuffers) * kTile * kVsStride + (ld.lrow + 16 * i) * kVsStride + 8 * ld.chunk) * 2;
 }
 // K fragment ks (0..7) of lane (r, g) for the unit at key_off (0 or 32) of tile j: 8 elements
 RD_HD int lds_k_frag(int j, int key_off, int r, int g, int ks) {
   return ((j % kKBuffers) * kTile * kKsStride + (key_off + r) * kKsStride + 16 * ks + 8 * g) * 2;
 }
-// V^T fragment c (0..7) of lane (r, g) for the unit at key_off of tile j: 8 elements
-RD_HD int lds_v_frag(int j, int key_off, int r, int g, int c) {
-  return kKBytes + ((j % kVBuffers) * kD * kVtStride + (32 * (c >> 1) + r) * kVtStride + 16 * (c & 1) + key_off + 8 * g) * 2;
+// V^T fragment c (0..7: dims 32 * (c / 2) .., keys 16 * (c % 2) .. of the unit) for the unit at
+// key_off of tile j.  The lane (r = lane % 32, g = lane / 32) needs, as k-slot s = 0..7 of the
+// MFMA's A operand, V[key_off + 16 * (c % 2) + 4 * g + s % 4 + 8 * (s / 4)][32 * (c / 2) + r]: the
+// keys that its P^T operand holds in the same slots.  Two transposing reads deliver them, `half`
+// = s / 4 each four slots.  A transposing read works on groups of 16 lanes: lane i of a group
+// receives, as element e, element i % 4 of the 8 bytes that lane i / 4 + 4 * e of the group points
+// at.  So the lane's OWN address is that of four dims of one key: key ((lane % 16) / 4) of the
+// four, dims 4 * (lane % 4) .. of the group's sixteen (lanes 16-31 and 48-63: the upper sixteen
+// dims of the 32).
+RD_HD int lds_v_frag(int j, int key_off, int lane, int c, int half) {
+  const int g = lane >> 5;
+  const int key = key_off + 16 * (c & 1) + 4 * g + 8 * half + ((lane & 15) >> 2);
+  const int dim = 32 * (c >> 1) + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  return kKBytes + ((j % kVBuffers) * kTile * kVsStride + key * kVsStride + dim) * 2;
 }
-// merge of the two key halves of a row block after the loop: [pair][64 accumulators][lane] floats,
-// then [pair][2][lane]
-constexpr int kMergeFloats = (kWaves / 2) * (64 * 64 + 2 * 64);
+// Merge of the two key halves of a row block after the loop.  Each wave of the pair ends up with
+// one half of the head dimension: the wave with key part 0 keeps dims 0-63 (accumulator blocks 0,
+// 1) and hands its blocks 2, 3 over, part 1 keeps dims 64-127 and hands blocks 0, 1 over; both
+// leave their (m, l).  [pair][64 accumulators][lane] floats (accumulator 16 * block + i, written by
+// the wave that does NOT keep that block), then [pair][key part][m | l][lane].
+constexpr int kMergeFloats = (kWaves / 2) * (64 * 64 + 4 * 64);
 RD_HD int lds_merge_o(int pair, int acc, int lane) { return ((pair * 64 + acc) * 64 + lane) * 4; }
-RD_HD int lds_merge_ml(int pair, int which, int lane) { return ((kWaves / 2) * 64 * 64 + (pair * 2 + which) * 64 + lane) * 4; }
+RD_HD int lds_merge_ml(int pair, int part, int which, int lane) {
+  return ((kWaves / 2) * 64 * 64 + ((pair * 2 + part) * 2 + which) * 64 + lane) * 4;
+}
+// accumulator blocks (32 dims each) that a wave normalises and stores: all four for a full wave,
+// two for a half wave
+RD_HD int first_block_kept(int part) { return part == 1 ? 2 : 0; }
+RD_HD int blocks_kept(int part) { return part == 2 ? 4 : 2; }
 
 // ---- query rows, outputs, mask words ---------------------------------------------------------
 RD_HD int q_row_of(int q_tile, int rows_per_workgroup, int row_block, int r) { return q_tile * rows_per_workgroup + row_block * 32 + r; }

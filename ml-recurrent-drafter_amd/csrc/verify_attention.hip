@@ -10,8 +10,10 @@
 //   attn_mfma_kernel      bf16, head_dim 128: S^T = K Q^T and O^T = V^T P^T on
 //                         v_mfma_f32_32x32x16_bf16.  512 threads = 8 waves; a wave owns 32 query
 //                         rows (with at most 128 rows per workgroup, two waves share a row block
-//                         and split every tile's keys).  64-key K tiles and transposed V tiles
-//                         travel global -> register ring -> LDS and are shared by the waves.  The
+//                         and split every tile's keys).  64-key K and V tiles travel global ->
+//                         register ring -> LDS as they lie in memory and are shared by the waves;
+//                         the V^T operand of the second product comes out of transposing LDS
+//                         reads (ds_read_b64_tr_b16).  The
 //                         loop is a software pipeline over 32-key units: while the vector ALU turns
 //                         the scores of one unit into probabilities (online softmax in fp32, lazy
 //                         rescale), the matrix pipeline already multiplies the next unit's keys.
@@ -156,14 +158,76 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const int row_wave = role.block;                     // row block of this wave
   const bool full = kHasFull && (!kHasHalf || role.part == 2);  // wave-uniform
   const int kp = full ? 0 : role.part;                 // key half of a half wave
+  const __bf16* kbase = reinterpret_cast<const __bf16*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh - (int64_t)kv_shift * a.k_ss;
+  const __bf16* vbase = reinterpret_cast<const __bf16*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh - (int64_t)kv_shift * a.v_ss;
+
+  // Loader roles (attn_addr.h: loader_of): waves 0-3 stage the K tile, waves 4-7 the V tile, four
+  // 16-byte chunks per thread and tile.
+  const bool k_loader = wave < kWaves / 2;  // (== ld.k_loader, and wave-uniform for the compiler)
+  const Loader ld = loader_of(tid);
+  const int chunk = ld.chunk, lrow = ld.lrow;
+
+  const int n_tiles = n_tiles_of(lo, hi);
+  // Tiles in flight: a ring of kRing register stages between global memory and LDS; tile j
+  // passes through slot j % kRing.  The mask words travel in a ring of their own.
+  // Every step issues the same loads on every path (tile indices past the end are clamped to the
+  // last tile, keys past kv_len to the last key): with loads under divergent or data-dependent
+  // branches the compiler can no longer count which loads are still in flight and waits for all
+  // of them at every use, which would cap the ring at one tile.
+  static_assert(kRing == 2, "two named register stages");
+  // the four 16-byte chunks a thread carries per tile, for ring slots 0 (a) and 1 (b); plain
+  // variables: grouped in arrays or structs they are left in scratch memory
+  bf16x8 a0, a1, a2, a3, b0, b1, b2, b3;
+  uint64_t wring[kRing];
+  // address of a 16-byte chunk = wave-uniform part (tile, i) + 32-bit lane part
+  const char* base = reinterpret_cast<const char*>(k_loader ? kbase : vbase);
+  const int64_t row_bytes = (k_loader ? a.k_ss : a.v_ss) * 2;
+  const int key_step = ld.key_step, first_key = ld.first_key;  // this thread's keys within a tile: first_key + i * key_step
+  const uint32_t lane_off = (uint32_t)(first_key * row_bytes + 16 * chunk);
+  auto fetch_into = [&](bf16x8& c0, bf16x8& c1, bf16x8& c2, bf16x8& c3, int j) __attribute__((always_inline)) {
+    const int key0 = tile_key0(lo, j, n_tiles);
+    const char* tile = base + (int64_t)key0 * row_bytes;
+    const int64_t step_bytes = key_step * row_bytes;
+    // chunk i reads key column tile_chunk_key(ld, key0, i, key_min, key_end): inside the span that
+    // is key0 + first_key + i * key_step ...
+    int64_t o0 = lane_off, o1 = step_bytes + lane_off, o2 = 2 * step_bytes + lane_off, o3 = 3 * step_bytes + lane_off;
+    if (tile_leaves_span(key0, key_min, key_end)) {
+      // the first and the last tile of a row: keys in front of the row's first attended key (left
+      // padding) re-read that key, keys behind its last attended key (tree slots that do not exist,
+      // the end of the cache) re-read that one.  Nothing outside the row's live cache rows is ever
+      // touched: the probabilities of those keys are zero, but zero times whatever lay there
+      // could be NaN
+      auto clamped = [&](int i) __attribute__((always_inline)) {
+        return (int64_t)(tile_chunk_key(ld, key0, i, key_min, key_end) - key0) * row_bytes + 16 * chunk;
+      };
+      o0 = clamped(0); o1 = clamped(1); o2 = clamped(2); o3 = clamped(3);
+    }
+    // Non-temporal loads: every K and V row is read once per launch (twice when two query tiles or
+    // grouped heads share it, back to back), so it should not push the L2's other lines out on its
+    // way through.  In the decode step this alone takes the launch from 28.8 to 27.3 us at 600 keys
+    // per row and from 85 to 70 us at 2500.
+    c0 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(tile + o0));
+    c1 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(tile + o1));
+    c2 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(tile + o2));
+    c3 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(tile + o3));
+  };
+  auto fetch_tile = [&](auto slot_c, int j) __attribute__((always_inline)) {
+    if constexpr (decltype(slot_c)::value == 0) fetch_into(a0, a1, a2, a3, j); else fetch_into(b0, b1, b2, b3, j);
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1 % kRing>;
+  // The first tiles are requested as soon as the work item is known: they need nothing but the
+  // item (everything else on the way to the first product -- the row's query rows, Q, the mask
+  // words -- hangs on one more trip to memory, which these loads no longer wait for).
+  if constexpr (!ROPE) {
+    fetch_tile(S0{}, 0);
+    if (k_loader) fetch_tile(S1{}, 1);
+  }
   const RowSpan rows = row_span(a, b);
   if (q_tile * kRowsPerWG >= rows.n) return;  // (every thread of the workgroup: no barrier is skipped)
   const int q_row = q_row_of(q_tile, kRowsPerWG, row_wave, r);
   const bool wave_active = q_tile * kRowsPerWG + row_wave * 32 < rows.n;
   const bool row_valid = q_row < rows.n;
-
-  const __bf16* kbase = reinterpret_cast<const __bf16*>(a.k) + (int64_t)b * a.k_sb + (int64_t)hk * a.k_sh - (int64_t)kv_shift * a.k_ss;
-  const __bf16* vbase = reinterpret_cast<const __bf16*>(a.v) + (int64_t)b * a.v_sb + (int64_t)hk * a.v_sh - (int64_t)kv_shift * a.v_ss;
 
   // ---- new cache rows and rotated queries (ROPE) ---------------------------------------------------
   // The new keys and values of this (batch row, kv head) go to their cache rows before anybody's
@@ -320,55 +384,6 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   float m = -INFINITY, l = 0.f;  // m in log2 units (already scaled)
   const float scale_log2 = a.scale * 1.4426950408889634f;
 
-  // Loader roles (attn_addr.h: loader_of): waves 0-3 stage K rows, waves 4-7 stage V transposed,
-  // four 16-byte chunks per thread and tile.
-  const bool k_loader = wave < kWaves / 2;  // (== ld.k_loader, and wave-uniform for the compiler)
-  const Loader ld = loader_of(tid);
-  const int chunk = ld.chunk, lrow = ld.lrow;
-
-  const int n_tiles = n_tiles_of(lo, hi);
-  // Tiles in flight: a ring of kRing register stages between global memory and LDS; tile j
-  // passes through slot j % kRing.  The mask words travel in a ring of their own.
-  // Every step issues the same loads on every path (tile indices past the end are clamped to the
-  // last tile, keys past kv_len to the last key): with loads under divergent or data-dependent
-  // branches the compiler can no longer count which loads are still in flight and waits for all
-  // of them at every use, which would cap the ring at one tile.
-  static_assert(kRing == 2, "two named register stages");
-  // the four 16-byte chunks a thread carries per tile, for ring slots 0 (a) and 1 (b); plain
-  // variables: grouped in arrays or structs they are left in scratch memory
-  bf16x8 a0, a1, a2, a3, b0, b1, b2, b3;
-  uint64_t wring[kRing];
-  // address of a 16-byte chunk = wave-uniform part (tile, i) + 32-bit lane part
-  const char* base = reinterpret_cast<const char*>(k_loader ? kbase : vbase);
-  const int64_t row_bytes = (k_loader ? a.k_ss : a.v_ss) * 2;
-  const int key_step = ld.key_step, first_key = ld.first_key;  // this thread's keys within a tile: first_key + i * key_step
-  const uint32_t lane_off = (uint32_t)(first_key * row_bytes + 16 * chunk);
-  auto fetch_into = [&](bf16x8& c0, bf16x8& c1, bf16x8& c2, bf16x8& c3, int j) __attribute__((always_inline)) {
-    const int key0 = tile_key0(lo, j, n_tiles);
-    const char* tile = base + (int64_t)key0 * row_bytes;
-    const int64_t step_bytes = key_step * row_bytes;
-    // chunk i reads key column tile_chunk_key(ld, key0, i, key_min, key_end): inside the span that
-    // is key0 + first_key + i * key_step ...
-    int64_t o0 = lane_off, o1 = step_bytes + lane_off, o2 = 2 * step_bytes + lane_off, o3 = 3 * step_bytes + lane_off;
-    if (tile_leaves_span(key0, key_min, key_end)) {
-      // the first and the last tile of a row: keys in front of the row's first attended key (left
-      // padding) re-read that key, keys behind its last attended key (tree slots that do not exist,
-      // the end of the cache) re-read that one.  Nothing outside the row's live cache rows is ever
-      // touched: the probabilities of those keys are zero, but zero times whatever lay there
-      // could be NaN
-      auto clamped = [&](int i) __attribute__((always_inline)) {
-        return (int64_t)(tile_chunk_key(ld, key0, i, key_min, key_end) - key0) * row_bytes + 16 * chunk;
-      };
-      o0 = clamped(0); o1 = clamped(1); o2 = clamped(2); o3 = clamped(3);
-    }
-    c0 = *reinterpret_cast<const bf16x8*>(tile + o0);
-    c1 = *reinterpret_cast<const bf16x8*>(tile + o1);
-    c2 = *reinterpret_cast<const bf16x8*>(tile + o2);
-    c3 = *reinterpret_cast<const bf16x8*>(tile + o3);
-  };
-  auto fetch_tile = [&](auto slot_c, int j) __attribute__((always_inline)) {
-    if constexpr (decltype(slot_c)::value == 0) fetch_into(a0, a1, a2, a3, j); else fetch_into(b0, b1, b2, b3, j);
-  };
   auto fetch_word = [&](auto slot_c, int j) __attribute__((always_inline)) {
     const int key0 = tile_key0(lo, j, n_tiles);
     // nothing may touch the loaded value here: an operation on it would make the wave wait for
@@ -385,13 +400,12 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   auto stage_k = [&](auto slot_c, int j) __attribute__((always_inline)) {
     if constexpr (decltype(slot_c)::value == 0) stage_k_from(a0, a1, a2, a3, j); else stage_k_from(b0, b1, b2, b3, j);
   };
-  auto stage_v_from = [&](bf16x8 p0, bf16x8 p1, bf16x8 p2, bf16x8 p3, int j) __attribute__((always_inline)) {
+  auto stage_v_from = [&](bf16x8 c0, bf16x8 c1, bf16x8 c2, bf16x8 c3, int j) __attribute__((always_inline)) {
     char* dst = smem + lds_v_stage(ld, j, 0);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      bf16x4 t = {p0[e], p1[e], p2[e], p3[e]};
-      *reinterpret_cast<bf16x4*>(dst + (lds_v_stage(ld, 0, e) - lds_v_stage(ld, 0, 0))) = t;
-    }
+    *reinterpret_cast<bf16x8*>(dst) = c0;
+    *reinterpret_cast<bf16x8*>(dst + (lds_v_stage(ld, 0, 1) - lds_v_stage(ld, 0, 0))) = c1;
+    *reinterpret_cast<bf16x8*>(dst + (lds_v_stage(ld, 0, 2) - lds_v_stage(ld, 0, 0))) = c2;
+    *reinterpret_cast<bf16x8*>(dst + (lds_v_stage(ld, 0, 3) - lds_v_stage(ld, 0, 0))) = c3;
   };
   auto stage_v = [&](auto slot_c, int j) __attribute__((always_inline)) {
     if constexpr (decltype(slot_c)::value == 0) stage_v_from(a0, a1, a2, a3, j); else stage_v_from(b0, b1, b2, b3, j);
@@ -409,20 +423,15 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   };
 
   // ---- prologue: K of tiles 0 and 1 and V of tile 0 into LDS, the ring filled behind them --------
-  using S0 = std::integral_constant<int, 0>;
-  using S1 = std::integral_constant<int, 1 % kRing>;
   // K runs one tile further ahead than V (K(t+1) is multiplied during step t); both roles keep
   // the tile that step t stages in ring slot (t + 1) % kRing, so that one piece of code, with
   // the same registers, serves both.
   const int ahead = k_loader ? 2 : 1;
   if constexpr (!ROPE) {
-    if (k_loader) {
-      fetch_tile(S0{}, 0);
-      fetch_tile(S1{}, 1);
+    if (k_loader) {  // (requested at the kernel's entry)
       stage_k(S0{}, 0);
       stage_k(S1{}, 1);
     } else {
-      fetch_tile(S0{}, 0);
       stage_v(S0{}, 0);
     }
   } else {
@@ -439,23 +448,43 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       stage_v(S0{}, 0);
     }
   }
-  // The ring is filled in the order in which the steps refill it (tile, then mask word, slot by
+  // The ring is filled in the order in which the steps refill it (mask word, then tile, slot by
   // slot): the loads in flight at the top of the first step are then the same as at the top of
   // every later one, and the compiler's count of them stays exact around the loop.  The mask word
   // of tile j sits in wring[j % kRing] from two steps before its tile until the tile's last unit;
   // it is never copied to another variable (a copy right after the load would be a wait for it).
   rd_static_for<kRing>([&](auto j) __attribute__((always_inline)) {
     constexpr int J = decltype(j)::value;
-    fetch_tile(std::integral_constant<int, (J + 1) % kRing>{}, ahead + J);
     fetch_word(std::integral_constant<int, J>{}, J);
+    fetch_tile(std::integral_constant<int, (J + 1) % kRing>{}, ahead + J);
   });
   __syncthreads();
+  // The scores of a unit are masked, and their row maximum taken, as soon as they exist: in the
+  // step before the one that turns them into probabilities, under that step's second product
+  // (the matrix pipeline is busy there and the vector ALU is not).  tmax: that maximum, in log2
+  // units, of the unit whose scores wait in the score registers; here for the first unit.
+  // Rows past n_q take an all-ones word: their results are never used.
+  auto unit_bits = [&](uint64_t word, int key_off) __attribute__((always_inline)) {  // the unit's 32 keys
+    return row_valid ? (uint32_t)(word >> key_off) : ~0u;
+  };
+  auto masked = [&](float score, uint32_t w, int i) __attribute__((always_inline)) {
+    // accumulator i is key 8*(i/4) + 4*g + i%4 of the unit; w: the unit's bits shifted down by 4*g
+    return ((w >> (8 * (i >> 2) + (i & 3))) & 1u) ? score : -INFINITY;
+  };
+  float tmax = -INFINITY;
   if (wave_active) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) s_reg[0][i] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks)
       s_reg[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(k_lane(0), kp * 32, ks), qf[ks], s_reg[0], 0, 0, 0);
+    const uint32_t w = unit_bits(wring[0], kp * 32) >> (4 * g);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      s_reg[0][i] = masked(s_reg[0][i], w, i);
+      tmax = fmaxf(tmax, s_reg[0][i]);
+    }
+    tmax = pair_max(tmax) * scale_log2;
   }
 
   // ---- one unit per step -----------------------------------------------------------------------
@@ -475,22 +504,14 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     f32x16& s_next = s_reg[CUR ^ 1];
     const bool busy = wave_active && run;
     bf16x8 pf[2];  // P^T of the unit, the B operand of the second product
+    if (kLast) {
+      // This tile's mask word is done with (its last unit was masked in the step before): the word
+      // of tile t+kRing takes its slot.  Requested ahead of this step's tile, so that the step that
+      // uses it waits for no tile it has not staged.
+      fetch_word(std::integral_constant<int, J>{}, t + kRing);
+    }
     if (busy) {
-      // mask, running maximum, lazy rescale: short, not overlapped
-      // rows past n_q take an all-ones word: no masking work, and their results are never used
-      const uint32_t mine = row_valid ? (uint32_t)(wring[J] >> key_off) : ~0u;
-      if (!__all(mine == ~0u)) {
-        const uint32_t w = mine >> (4 * g);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const bool on = (w >> (8 * (i >> 2) + (i & 3))) & 1u;
-          s_cur[i] = on ? s_cur[i] : -INFINITY;
-        }
-      }
-      float tmax = -INFINITY;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s_cur[i]);
-      tmax = pair_max(tmax) * scale_log2;
+      // lazy rescale (the unit's scores were masked and their maximum taken in the wave's previous step)
       // The running maximum only has to bound the exponents, not equal the true maximum: it is
       // raised (and O, l rescaled) only when a unit exceeds it by more than kSlack, so most units
       // skip the 64-register rescale.  p <= 2^kSlack stays far inside bf16/fp32 range.
@@ -544,9 +565,17 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     // the second product starts
     constexpr int kVDepth = 4;
     bf16x8 va[kVDepth];
-    const char* sv = smem + lds_v_frag(t, key_off, r, g, 0);
+    // (lds_v_frag is linear: the lane's own place in the tile's buffer plus the wave-uniform place
+    // of the fragment's keys and dims; a fragment is two transposing reads of four keys each)
+    typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+    typedef __attribute__((address_space(3))) char lds_char;
+    lds_char* sv = (lds_char*)smem + lds_v_frag(t, key_off, lane, 0, 0);
     auto v_frag = [&](int c) __attribute__((always_inline)) {
-      return *reinterpret_cast<const bf16x8*>(sv + (lds_v_frag(0, 0, 0, 0, c) - lds_v_frag(0, 0, 0, 0, 0)));
+      const bf16x4 first = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+          (lds_bf16x4*)(sv + (lds_v_frag(0, 0, 0, c, 0) - lds_v_frag(0, 0, 0, 0, 0))));
+      const bf16x4 second = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+          (lds_bf16x4*)(sv + (lds_v_frag(0, 0, 0, c, 1) - lds_v_frag(0, 0, 0, 0, 0))));
+      return __builtin_shufflevector(first, second, 0, 1, 2, 3, 4, 5, 6, 7);
     };
     if (busy) {
 #pragma unroll
@@ -559,17 +588,36 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       fetch_tile(Slot{}, t + ahead + kRing);
     }
     if (busy) {
-      // O^T += V^T P^T ; k-slot j of lane group g is key 16*tt + 4*g + (j%4) + 8*(j/4) of the unit,
-      // stored at columns 16*tt + 8*g + j of the V^T row
+      // O^T += V^T P^T ; k-slot j of lane group g is key 16*tt + 4*g + (j%4) + 8*(j/4) of the unit.
+      // Behind each MFMA, two scores of the NEXT unit (complete since the first product above) are
+      // folded into that unit's row maximum.  Its mask word has been in the ring since the step
+      // before (requested before that step's tile: using it waits for no tile that this step has
+      // not already staged).
+      uint64_t next_word = wring[(J + 1) % kRing];  // the next unit lies in the next tile ...
+      if constexpr (!kLast) next_word = next_t == t ? wring[J] : next_word;  // ... or is this tile's other half
+      const uint32_t next_bits = unit_bits(next_word, next_off);
+      float next_max = -INFINITY;
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         o[c >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[c % kVDepth], pf[c & 1], o[c >> 1], 0, 0, 0);
         if (c + kVDepth < 8) va[c % kVDepth] = v_frag(c + kVDepth);
+        next_max = fmaxf(next_max, fmaxf(s_next[2 * c], s_next[2 * c + 1]));
+        __builtin_amdgcn_sched_barrier(0);
       }
+      // Most units lie in front of the tree, where every key is attended.  The others (the tree's
+      // tiles, a tile with left padding) are masked now and their maximum is taken again.
+      if (!__all(next_bits == ~0u)) {
+        const uint32_t wn = next_bits >> (4 * g);
+        next_max = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          s_next[i] = masked(s_next[i], wn, i);
+          next_max = fmaxf(next_max, s_next[i]);
+        }
+      }
+      tmax = pair_max(next_max) * scale_log2;
     }
     if (kLast) {
-      // this tile's mask word is done with: the word of tile t+kRing takes its slot
-      fetch_word(std::integral_constant<int, J>{}, t + kRing);
       if constexpr (ROPE) {
         if (t == t_sync) new_rows_wait();  // (uniform) the next step may request a tile with new rows
       }
@@ -611,50 +659,81 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   if (t0 < n_tiles) tile_step(S0{}, t0);
 
   l = pair_sum(l);
+  // accumulator i of block db is d = 32*db + 8*(i/4) + 4*g + i%4
+  static_assert(kMergeFloats * 4 <= kLdsBytes, "merge buffer");
   if (kHasHalf) {
-    // merge the two key parts of every row block: part 1 hands (m, l, o) over through LDS (the tile
-    // buffers are free: every wave has passed the loop's last barrier)
-    auto x_o = [&](int acc) __attribute__((always_inline)) -> float& {  // [pair][64 accumulators][lane]
+    // Merge of the two key parts of every row block through LDS (the tile buffers are free: every
+    // wave has passed the loop's last barrier).  The two waves of a pair exchange halves: each hands
+    // over the two accumulator blocks it does not keep and its (m, l), and merges the partner's
+    // part of the two blocks it keeps -- half the LDS traffic per wave of handing everything to one
+    // wave, and both waves normalise and store.  Both evaluate the same expressions on the same
+    // operands in the same order (part 0's term first), so they agree on m and l to the bit.
+    auto x_o = [&](int acc) __attribute__((always_inline)) -> float& {
       return *reinterpret_cast<float*>(smem + lds_merge_o(role.pair, acc, lane));
     };
-    auto x_ml = [&](int which) __attribute__((always_inline)) -> float& {  // [pair][2][lane]
-      return *reinterpret_cast<float*>(smem + lds_merge_ml(role.pair, which, lane));
+    auto x_ml = [&](int part, int which) __attribute__((always_inline)) -> float& {
+      return *reinterpret_cast<float*>(smem + lds_merge_ml(role.pair, part, which, lane));
     };
-    static_assert(kMergeFloats * 4 <= kLdsBytes, "merge buffer");
-    const bool second = !full && kp == 1;
-    if (second && wave_active) {
+    auto hand_over = [&](auto first_c) __attribute__((always_inline)) {  // the blocks this wave does not keep
+      constexpr int kFirst = decltype(first_c)::value;
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = kFirst; db < kFirst + 2; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) x_o(16 * db + i) = o[db][i];
-      x_ml(0) = m;
-      x_ml(1) = l;
+    };
+    auto take_over = [&](auto first_c, float a0, float a1) __attribute__((always_inline)) {  // the blocks it keeps
+      constexpr int kFirst = decltype(first_c)::value;
+#pragma unroll
+      for (int db = kFirst; db < kFirst + 2; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const float theirs = x_o(16 * db + i);
+          // (part 0's term first, whoever computes it)
+          o[db][i] = kFirst == 0 ? a0 * o[db][i] + a1 * theirs : a0 * theirs + a1 * o[db][i];
+        }
+    };
+    const bool half = !full && wave_active;  // (wave-uniform)
+    if (half) {
+      if (kp == 0) hand_over(std::integral_constant<int, 2>{}); else hand_over(std::integral_constant<int, 0>{});
+      x_ml(kp, 0) = m;
+      x_ml(kp, 1) = l;
     }
     __syncthreads();
-    if (wave_active && !full && !second) {
-      const float m2 = x_ml(0), l2 = x_ml(1);
-      const float m_new = fmaxf(m, m2);
+    if (half) {
+      const float m0 = kp == 0 ? m : x_ml(0, 0), l0 = kp == 0 ? l : x_ml(0, 1);
+      const float m1 = kp == 1 ? m : x_ml(1, 0), l1 = kp == 1 ? l : x_ml(1, 1);
+      const float m_new = fmaxf(m0, m1);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float a1 = fast_exp2(m - m_safe), a2 = fast_exp2(m2 - m_safe);  // exp2(-inf) = 0
-      l = a1 * l + a2 * l2;
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-          o[db][i] = a1 * o[db][i] + a2 * x_o(16 * db + i);
+      const float a0 = fast_exp2(m0 - m_safe), a1 = fast_exp2(m1 - m_safe);  // exp2(-inf) = 0
+      {
+#pragma clang fp contract(off)
+        l = a0 * l0 + a1 * l1;
+      }
+      if (kp == 0) take_over(std::integral_constant<int, 0>{}, a0, a1); else take_over(std::integral_constant<int, 2>{}, a0, a1);
       m = m_new;
     }
   }
-  const bool second_half = kHasHalf && !full && kp == 1;  // has handed its part to its partner
-  const bool writer = wave_active && row_valid && !second_half;
-  // accumulator i of block db is d = 32*db + 8*(i/4) + 4*g + i%4
+  const bool writer = wave_active && row_valid;
+  // What a wave writes: the accumulator blocks it keeps (attn_addr.h: first_block_kept,
+  // blocks_kept), named at compile time in each of the three cases (a block index that is only
+  // known at run time would put the accumulators into scratch memory).
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  using B2 = std::integral_constant<int, 2>;
+  using B3 = std::integral_constant<int, 3>;
+#define RD_FOR_KEPT_BLOCKS(body)                                         \
+  do {                                                                   \
+    if (full || !kHasHalf) { body(B0{}); body(B1{}); body(B2{}); body(B3{}); } \
+    else if (kp == 0) { body(B0{}); body(B1{}); }                        \
+    else { body(B2{}); body(B3{}); }                                     \
+  } while (0)
   if (n_splits == 1) {
     if (!writer) return;
     const bool live = l > 0.f;
     const float inv = live ? 1.f / l : 0.f;
     __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + out_offset(h, a.o_sh, q_row, a.o_ss, g, 0, 0);
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
+    auto store_block = [&](auto db_c) __attribute__((always_inline)) {
+      constexpr int db = decltype(db_c)::value;
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         // (a row without any attended key gets zeros, whatever its accumulators picked up)
@@ -662,6 +741,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
                     static_cast<__bf16>(live ? o[db][4 * i4 + 2] * inv : 0.f), static_cast<__bf16>(live ? o[db][4 * i4 + 3] * inv : 0.f)};
         *reinterpret_cast<bf16x4*>(op + (out_offset(0, 0, 0, 0, 0, db, i4))) = w;
       }
+    };
+    RD_FOR_KEPT_BLOCKS(store_block);
     return;
   }
   // The keys of this batch row are split over n_splits work items: each leaves (m, l, O) of its
@@ -676,14 +757,17 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // other workgroups stream through it: rows split four ways ran 8-19 % longer that way.
   if (writer) {
     float* po = a.part_o + partial_row(b, a.H, h, a.max_splits, split, a.n_q, q_row) * kD + 4 * g;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
+    auto store_partial = [&](auto db_c) __attribute__((always_inline)) {
+      constexpr int db = decltype(db_c)::value;
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
-        f32x4 w = {o[db][4 * i4 + 0], o[db][4 * i4 + 1], o[db][4 * i4 + 2], o[db][4 * i4 + 3]};
-        asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(po + 32 * db + 8 * i4), "v"(w) : "memory");
+        const f32x4 w = {o[db][4 * i4 + 0], o[db][4 * i4 + 1], o[db][4 * i4 + 2], o[db][4 * i4 + 3]};
+        float* const dst = po + 32 * db + 8 * i4;  // (a local: an asm operand cannot name a captured variable here)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(w) : "memory");
       }
-    if (g == 0) {
+    };
+    RD_FOR_KEPT_BLOCKS(store_partial);
+    if (g == 0 && (full || kp == 0)) {  // (both waves of a pair hold the same m and l)
       float* pm = a.part_ml + partial_row(b, a.H, h, a.max_splits, split, a.n_q, q_row) * 2;
       const f32x2 ml = {m, l};
       asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(pm), "v"(ml) : "memory");
@@ -759,6 +843,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     }
   }
   if (tid == 0) *counter = 0;  // ready for the next launch on this plan
+#undef RD_FOR_KEPT_BLOCKS
 }
 
 // ---------------------------------------------------------------------------------------------

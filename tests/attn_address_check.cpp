@@ -78,58 +78,78 @@ struct Item { int b, lo, hi, split, n_splits; };
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-// LDS: every staging write and fragment read inside its region, aligned, staging writes of a tile
-// disjoint, and fragment reads only of bytes that the staging wrote.
+// LDS: every staging write and fragment read inside its region and aligned, the staging writes of
+// a tile disjoint, and every fragment read delivers the elements the MFMA operand layout asks for.
+// The staging is modelled by what it writes: element (key, dim) of the tile is tagged key * 128 + dim
+// at the place its loader thread puts it; the fragment reads are then emulated on that model -- for
+// V with the lane exchange of the transposing read (lane i of a group of 16 receives, as element e,
+// element i % 4 of the 8 bytes that lane i / 4 + 4 * e of its group points at).
 void check_lds(Failure& f) {
   for (int j = 0; j < 12; ++j) {
-    std::vector<char> k_written(kKBytes, 0), v_written(kVBytes, 0);
+    std::vector<int> k_tag(kKBytes / 2, -1), v_tag(kVBytes / 2, -1);
     for (int tid = 0; tid < kThreads; ++tid) {
       const Loader ld = loader_of(tid);
       CHECK(ld.k_loader == (tid / 64 < kWaves / 2), "loader role of thread %d", tid);
       CHECK(ld.chunk >= 0 && ld.chunk < 16 && ld.lrow >= 0 && ld.lrow < 16, "loader lane map of thread %d", tid);
-      if (ld.k_loader) {
-        for (int i = 0; i < 4; ++i) {
-          const int off = lds_k_stage(ld, j, i);
-          CHECK(off >= 0 && off + 16 <= kKBytes && off % 16 == 0, "K stage offset %d (thread %d tile %d chunk %d)", off, tid, j, i);
-          for (int x = 0; x < 16; ++x) {
-            CHECK(!k_written[off + x], "K stage writes overlap at byte %d", off + x);
-            k_written[off + x] = 1;
-          }
-        }
-      } else {
-        for (int e = 0; e < 8; ++e) {
-          const int off = lds_v_stage(ld, j, e);
-          CHECK(off >= kKBytes && off + 8 <= kLdsBytes && off % 8 == 0, "V stage offset %d (thread %d tile %d element %d)", off, tid, j, e);
-          for (int x = 0; x < 8; ++x) {
-            CHECK(!v_written[off - kKBytes + x], "V stage writes overlap at byte %d", off + x);
-            v_written[off - kKBytes + x] = 1;
-          }
+      for (int i = 0; i < 4; ++i) {
+        const int key = ld.first_key + i * ld.key_step;  // the tile row this chunk was loaded from
+        CHECK(key >= 0 && key < kTile, "loader thread %d chunk %d: key %d of the tile", tid, i, key);
+        const int off = ld.k_loader ? lds_k_stage(ld, j, i) : lds_v_stage(ld, j, i);
+        const int lo = ld.k_loader ? 0 : kKBytes, hi = ld.k_loader ? kKBytes : kLdsBytes;
+        CHECK(off >= lo && off + 16 <= hi && off % 16 == 0, "stage offset %d (thread %d tile %d chunk %d)", off, tid, j, i);
+        std::vector<int>& tag = ld.k_loader ? k_tag : v_tag;
+        for (int x = 0; x < 8; ++x) {
+          int& t = tag[(off - lo) / 2 + x];
+          CHECK(t == -1, "stage writes overlap at byte %d", off + 2 * x);
+          t = key * kD + 8 * ld.chunk + x;
         }
       }
     }
     for (int key_off = 0; key_off <= 32; key_off += 32)
-      for (int r = 0; r < 32; ++r)
-        for (int g = 0; g < 2; ++g)
-          for (int c = 0; c < 8; ++c) {
-            const int ko = lds_k_frag(j, key_off, r, g, c);
-            CHECK(ko >= 0 && ko + 16 <= kKBytes && ko % 16 == 0, "K fragment offset %d", ko);
-            for (int x = 0; x < 16; ++x) CHECK(k_written[ko + x], "K fragment reads byte %d that no staging write fills", ko + x);
-            const int vo = lds_v_frag(j, key_off, r, g, c);
-            CHECK(vo >= kKBytes && vo + 16 <= kLdsBytes && vo % 16 == 0, "V fragment offset %d", vo);
-            for (int x = 0; x < 16; ++x) CHECK(v_written[vo - kKBytes + x], "V fragment reads byte %d that no staging write fills", vo + x);
+      for (int c = 0; c < 8; ++c) {
+        for (int lane = 0; lane < 64; ++lane) {
+          const int r = lane & 31, g = lane >> 5;
+          // K fragment ks = c: B^T operand of S^T = K Q^T: lane (r, g) holds K[key_off + r][16 c + 8 g ..]
+          const int ko = lds_k_frag(j, key_off, r, g, c);
+          CHECK(ko >= 0 && ko + 16 <= kKBytes && ko % 16 == 0, "K fragment offset %d", ko);
+          for (int x = 0; x < 8; ++x)
+            CHECK(k_tag[ko / 2 + x] == (key_off + r) * kD + 16 * c + 8 * g + x, "K fragment %d of lane %d: element %d is %d", c, lane, x, k_tag[ko / 2 + x]);
+        }
+        // V^T fragment c: two transposing reads; k-slot s of lane (r, g) must be
+        // V[key_off + 16 (c % 2) + 4 g + s % 4 + 8 (s / 4)][32 (c / 2) + r]
+        for (int half = 0; half < 2; ++half)
+          for (int lane = 0; lane < 64; ++lane) {
+            const int own = lds_v_frag(j, key_off, lane, c, half);
+            CHECK(own >= kKBytes && own + 8 <= kLdsBytes && own % 8 == 0, "V fragment offset %d (lane %d)", own, lane);
+            const int r = lane & 31, g = lane >> 5, i = lane & 15, group = lane & ~15;
+            for (int e = 0; e < 4; ++e) {
+              const int src = lds_v_frag(j, key_off, group + (i >> 2) + 4 * e, c, half);
+              const int got = v_tag[(src - kKBytes) / 2 + (i & 3)];
+              const int s_slot = 4 * half + e;
+              const int want = (key_off + 16 * (c & 1) + 4 * g + (s_slot & 3) + 8 * (s_slot >> 2)) * kD + 32 * (c >> 1) + r;
+              CHECK(got == want, "V fragment %d half %d of lane %d: slot %d holds element %d, the operand wants %d", c, half, lane, s_slot, got, want);
+            }
           }
+      }
   }
   for (int pair = 0; pair < kWaves / 2; ++pair)
     for (int lane = 0; lane < 64; ++lane) {
       for (int acc = 0; acc < 64; ++acc) {
         const int off = lds_merge_o(pair, acc, lane);
-        CHECK(off >= 0 && off + 4 <= kLdsBytes && off + 4 <= lds_merge_ml(0, 0, 0), "merge accumulator offset %d", off);
+        CHECK(off >= 0 && off + 4 <= kLdsBytes && off + 4 <= lds_merge_ml(0, 0, 0, 0), "merge accumulator offset %d", off);
       }
-      for (int which = 0; which < 2; ++which) {
-        const int off = lds_merge_ml(pair, which, lane);
-        CHECK(off >= 0 && off + 4 <= kLdsBytes && off + 4 <= kMergeFloats * 4, "merge (m, l) offset %d", off);
-      }
+      for (int part = 0; part < 2; ++part)
+        for (int which = 0; which < 2; ++which) {
+          const int off = lds_merge_ml(pair, part, which, lane);
+          CHECK(off >= lds_merge_o(kWaves / 2 - 1, 63, 63) + 4 && off + 4 <= kLdsBytes && off + 4 <= kMergeFloats * 4, "merge (m, l) offset %d", off);
+        }
     }
+  // the two waves of a pair hand over disjoint accumulator blocks and keep the other two: every
+  // block of the head dimension is kept by exactly one of them
+  for (int part = 0; part < 2; ++part) {
+    CHECK(blocks_kept(part) == 2 && first_block_kept(part) == 2 * part, "blocks kept by key part %d", part);
+  }
+  CHECK(blocks_kept(2) == 4 && first_block_kept(2) == 0, "blocks kept by a full wave");
   // every layout gives every row block either one full wave or two halves with distinct key parts,
   // and halves of different blocks distinct merge slots
   for (int layout = kSplit; layout <= kFull; ++layout) {
@@ -205,7 +225,6 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
           const int q_row = q_row_of(q_tile, rows_wg, role.block, r);
           const bool row_valid = q_row < rows_n;
           const bool wave_active = q_tile * rows_wg + role.block * 32 < rows_n;
-          const bool second_half = role.part == 1;
           // Q fragments and mask words (rows past the count read row 0 of the batch row)
           const int q_use = row_valid ? q_row : 0;
           if (row_valid)
@@ -232,9 +251,9 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
             }
           }
           // results
-          const bool writer = wave_active && row_valid && !second_half;
+          const bool writer = wave_active && row_valid;  // every wave stores the accumulator blocks it keeps
           if (writer) {
-            for (int db = 0; db < 4; ++db)
+            for (int db = first_block_kept(role.part); db < first_block_kept(role.part) + blocks_kept(role.part); ++db)
               for (int i4 = 0; i4 < 4; ++i4) {
                 const int64_t off = o_off + out_offset(h, L.o_sh, q_row, L.o_ss, g, db, i4);
                 CHECK(off >= 0 && off + 4 <= L.o_elems, "output element %lld of %lld (row %d head %d query %d)", (long long)off, (long long)L.o_elems, b, h, q_row);
