@@ -44,7 +44,7 @@ typedef enum { RD_BF16 = 0, RD_F16 = 1, RD_F32 = 2 } rd_dtype;
  * that crosses it (the attention plan, the realignment plan) or a workspace size changes.  A caller
  * compiled against this header compares rd_version() with RD_ABI_VERSION before its first call, so
  * that a stale build of the library is refused instead of being called with other arguments. */
-#define RD_ABI_VERSION 103
+#define RD_ABI_VERSION 104
 RD_API int rd_version(void);
 /* Message of the last failed call on this thread ("" if none). */
 RD_API const char* rd_last_error(void);
@@ -122,19 +122,25 @@ RD_API int rd_tree_mask(const int64_t* unpacker, const int64_t* packed_token_ind
  * Rows are row_bytes long; strides are in bytes (packed, out) / elements (index); output row t of
  * batch row b starts at out + b*out_batch_stride_bytes + t*out_row_stride_bytes.  An index outside
  * [0, n_src) leaves its output row untouched.
+ * row_start (batch + 1 int32 on the device, or NULL): with it `packed` holds only the rows that
+ * exist, batch row after batch row (rd_tree_build's row_start): row r of batch row b is row
+ * row_start[b] + r of packed, packed_batch_stride_bytes is not used, and an index at or beyond the
+ * batch row's count row_start[b+1] - row_start[b] leaves its output row untouched.
  * ------------------------------------------------------------------------------------------ */
 RD_API int rd_unpack_rows(const void* packed, int64_t packed_batch_stride_bytes, int64_t row_bytes,
                           const int64_t* index, int64_t index_batch_stride, int batch, int n_out,
                           int n_src, void* out, int64_t out_batch_stride_bytes,
-                          int64_t out_row_stride_bytes, void* stream);
+                          int64_t out_row_stride_bytes, const int32_t* row_start, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * First maximal index of every row of a (rows, vocab) matrix; NaN counts as the largest value.
  * Replaces torch.argmax(logits_by_llm, dim=-1) (recurrent_drafting.py:52, :425).
- * row_stride in elements.
+ * row_stride in elements.  out_index (rows int64 on the device, or NULL): with it the result of
+ * row r goes to out[out_index[r]] instead of out[r] -- the argmax of packed rows written straight
+ * to their (batch, slot) places; elements of out that no row names are left as they are.
  * ------------------------------------------------------------------------------------------ */
 RD_API int rd_argmax_rows(const void* x, int dtype, int64_t rows, int64_t vocab, int64_t row_stride,
-                          int64_t* out, void* stream);
+                          int64_t* out, const int64_t* out_index, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Greedy acceptance.  Replaces _greedy_choose_from_candidates (recurrent_drafting.py:468-496) and
@@ -184,13 +190,17 @@ RD_API int rd_position_ids(const int64_t* input_ids, int64_t ids_row_stride, int
  * left_pads (batch int32 on the device, or NULL): the leading pad run of every row of input_ids when
  * the caller has it already (rd_tree_attn_prepare and rd_count_left_paddings write it); saves the
  * launch that counts them.
+ * step_out (2 int32 on the device, or NULL): receives the new length M and the number of accepted
+ * tokens summed over the rows (what the reference's loop reports as avg_num_accepted * batch,
+ * recurrent_drafting.py:691-697), so that a caller can fetch both with whatever else it reads.
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_realign_plan_ints(int batch, int length);
 RD_API int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride, int64_t prev,
                            const int64_t* n_tokens_in_seq, const int64_t* seq_in_beam,
                            const int64_t* beams, const int64_t* unpacker, int batch, int width,
                            int length, int64_t pad_token_id, int32_t* plan, int64_t* new_ids,
-                           int32_t* kv_row_shift, const int32_t* left_pads, void* stream);
+                           int32_t* kv_row_shift, const int32_t* left_pads, int32_t* step_out,
+                           void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * KV cache, shape (n_layers, 2, batch, n_heads, max_len, head_dim), rows of row_bytes bytes.

@@ -231,6 +231,15 @@ def case_slope(rows, reps):
             return (lambda: op(logits)), B * mult * n * V * 2
         return make
 
+    def beam(mult):
+        # one beam-search iteration at 1x, 2x and 4x the decode step's batch (360, 720, 1440 rows of
+        # 32000 logits): the row kernel reads every row once
+        logits = (torch.randn(B * mult, W, V, device="cuda") * 2).to(torch.bfloat16)
+        lpb = -torch.rand(B * mult, W, device="cuda") * 4
+        beams = torch.randint(0, V, (B * mult, W, 2), device="cuda")
+        return (lambda: modeling_drafter.beam_topk_step(logits, lpb, beams, False)), B * mult * W * V * 2
+
+    series("beam_topk bf16 (batch x width rows of 32000)", "beam_row_kernel", beam)
     series("argmax packed bf16 logits", "argmax_rows_kernel", logits_case(acceptance.argmax_rows))
     series("verify_row_stats packed bf16 logits", "row_stats_kernel", logits_case(lambda x: acceptance.verify_row_stats(x, 1.0)))
 

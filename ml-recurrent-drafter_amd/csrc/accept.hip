@@ -33,7 +33,8 @@ __device__ inline bool better(float v, int64_t i, float bv, int64_t bi) {
 template <typename T, int VEC>
 __global__ __launch_bounds__(kThreads) void argmax_rows_kernel(const T* __restrict__ x,
                                                                int64_t row_stride, int64_t V,
-                                                               int64_t* __restrict__ out) {
+                                                               int64_t* __restrict__ out,
+                                                               const int64_t* __restrict__ out_index) {
   const T* row = x + (int64_t)blockIdx.x * row_stride;
   float bv = -INFINITY;
   int64_t bi = INT64_MAX;
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(kThreads) void argmax_rows_kernel(const T* __restri
   if (threadIdx.x == 0) {
     for (int w = 1; w < kWaves; ++w)
       if (better(s_v[w], s_i[w], bv, bi)) { bv = s_v[w]; bi = s_i[w]; }
-    out[blockIdx.x] = bi == INT64_MAX ? 0 : bi;
+    out[out_index ? out_index[blockIdx.x] : (int64_t)blockIdx.x] = bi == INT64_MAX ? 0 : bi;
   }
 }
 
@@ -178,22 +179,26 @@ __global__ __launch_bounds__(kThreads) void realign_plan_kernel(
     const int64_t* __restrict__ n_tokens_in_seq, const int64_t* __restrict__ seq_in_beam,
     const int64_t* __restrict__ beams, const int64_t* __restrict__ unpacker, int B, int W, int L,
     int64_t pad, const int32_t* __restrict__ pads, int32_t* __restrict__ plan,
-    int64_t* __restrict__ new_ids, int32_t* __restrict__ kv_shift) {
+    int64_t* __restrict__ new_ids, int32_t* __restrict__ kv_shift, int32_t* __restrict__ step_out) {
   const int b = blockIdx.x;
-  int m = 0;
+  int m = 0, accepted = 0;
   for (int r = threadIdx.x; r < B; r += kThreads) {
-    const int sl = (int)prev - pads[r] + clampi((int)n_tokens_in_seq[r], 0, L - 1) + 1;
+    const int n = clampi((int)n_tokens_in_seq[r], 0, L - 1);
+    const int sl = (int)prev - pads[r] + n + 1;
     m = sl > m ? sl : m;
+    accepted += n;
   }
   for (int off = 32; off > 0; off >>= 1) {
     const int o = __shfl_xor(m, off);
     m = o > m ? o : m;
+    accepted += __shfl_xor(accepted, off);
   }
-  __shared__ int s_m[kWaves];
-  if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
+  __shared__ int s_m[kWaves], s_accepted[kWaves];
+  if ((threadIdx.x & 63) == 0) { s_m[threadIdx.x >> 6] = m; s_accepted[threadIdx.x >> 6] = accepted; }
   __syncthreads();
   m = 0;
-  for (int w = 0; w < kWaves; ++w) m = s_m[w] > m ? s_m[w] : m;
+  accepted = 0;
+  for (int w = 0; w < kWaves; ++w) { m = s_m[w] > m ? s_m[w] : m; accepted += s_accepted[w]; }
 
   const int old_pads = pads[b];
   // out-of-range inputs are clamped so that no access below can leave its buffer
@@ -207,7 +212,10 @@ __global__ __launch_bounds__(kThreads) void realign_plan_kernel(
   // behind the live ones) and the shift takes up the change of the left padding instead.
   const int shift = kv_shift ? kv_shift[b] : 0;
   if (threadIdx.x == 0) {
-    if (b == 0) { plan[0] = m; plan[1] = (int)prev; plan[2] = L; plan[3] = 0; }
+    if (b == 0) {
+      plan[0] = m; plan[1] = (int)prev; plan[2] = L; plan[3] = 0;
+      if (step_out) { step_out[0] = m; step_out[1] = accepted; }
+    }
     row_plan[0] = old_pads - shift;
     row_plan[1] = (kv_shift ? old_pads : new_pads) - shift;
     row_plan[2] = n_new; row_plan[3] = live;
@@ -228,22 +236,22 @@ __global__ __launch_bounds__(kThreads) void realign_plan_kernel(
 
 template <typename T>
 int launch_argmax(const void* x, int64_t rows, int64_t V, int64_t row_stride, int64_t* out,
-                  hipStream_t s) {
+                  const int64_t* out_index, hipStream_t s) {
   constexpr int VEC = 16 / sizeof(T);
   const bool vec_ok = ((uintptr_t)x % 16 == 0) && (row_stride % VEC == 0);
   if (vec_ok)
     { rd::ScopedTiming rd_t("argmax_rows_kernel", s); hipLaunchKernelGGL((argmax_rows_kernel<T, VEC>), dim3(rows), dim3(kThreads), 0, s,
-                       reinterpret_cast<const T*>(x), row_stride, V, out); }
+                       reinterpret_cast<const T*>(x), row_stride, V, out, out_index); }
   else
     { rd::ScopedTiming rd_t("argmax_rows_kernel", s); hipLaunchKernelGGL((argmax_rows_kernel<T, 1>), dim3(rows), dim3(kThreads), 0, s,
-                       reinterpret_cast<const T*>(x), row_stride, V, out); }
+                       reinterpret_cast<const T*>(x), row_stride, V, out, out_index); }
   return rd::check_launch("rd_argmax_rows");
 }
 
 }  // namespace
 
 extern "C" int rd_argmax_rows(const void* x, int dtype, int64_t rows, int64_t vocab,
-                              int64_t row_stride, int64_t* out, void* stream) {
+                              int64_t row_stride, int64_t* out, const int64_t* out_index, void* stream) {
   RD_REQUIRE(rows > 0 && vocab > 0 && row_stride >= vocab, RD_EINVAL,
              "rd_argmax_rows: rows %lld vocab %lld row_stride %lld", (long long)rows,
              (long long)vocab, (long long)row_stride);
@@ -251,9 +259,9 @@ extern "C" int rd_argmax_rows(const void* x, int dtype, int64_t rows, int64_t vo
   RD_REQUIRE(x && out, RD_EINVAL, "rd_argmax_rows: null pointer");
   hipStream_t s = rd::as_stream(stream);
   switch (dtype) {
-    case RD_F32: return launch_argmax<float>(x, rows, vocab, row_stride, out, s);
-    case RD_BF16: return launch_argmax<__hip_bfloat16>(x, rows, vocab, row_stride, out, s);
-    case RD_F16: return launch_argmax<__half>(x, rows, vocab, row_stride, out, s);
+    case RD_F32: return launch_argmax<float>(x, rows, vocab, row_stride, out, out_index, s);
+    case RD_BF16: return launch_argmax<__hip_bfloat16>(x, rows, vocab, row_stride, out, out_index, s);
+    case RD_F16: return launch_argmax<__half>(x, rows, vocab, row_stride, out, out_index, s);
     default: return rd::fail(RD_EINVAL, "rd_argmax_rows: unknown dtype %d", dtype);
   }
 }
@@ -287,7 +295,8 @@ extern "C" int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride,
                                const int64_t* n_tokens_in_seq, const int64_t* seq_in_beam,
                                const int64_t* beams, const int64_t* unpacker, int batch, int width,
                                int length, int64_t pad_token_id, int32_t* plan, int64_t* new_ids,
-                               int32_t* kv_row_shift, const int32_t* left_pads, void* stream) {
+                               int32_t* kv_row_shift, const int32_t* left_pads, int32_t* step_out,
+                               void* stream) {
   RD_REQUIRE(batch > 0 && width > 0 && length > 0 && prev >= 0, RD_EINVAL,
              "rd_realign_plan: bad sizes (batch %d width %d length %d prev %lld)", batch, width,
              length, (long long)prev);
@@ -306,7 +315,7 @@ extern "C" int rd_realign_plan(const int64_t* input_ids, int64_t ids_row_stride,
   }
   { rd::ScopedTiming rd_t("realign_plan_kernel", s); hipLaunchKernelGGL(realign_plan_kernel, dim3(batch), dim3(kThreads), 0, s, input_ids,
                      ids_row_stride, prev, n_tokens_in_seq, seq_in_beam, beams, unpacker, batch,
-                     width, length, pad_token_id, pads, plan, new_ids, kv_row_shift); }
+                     width, length, pad_token_id, pads, plan, new_ids, kv_row_shift, step_out); }
   return rd::check_launch("rd_realign_plan");
 }
 

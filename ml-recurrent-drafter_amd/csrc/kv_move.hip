@@ -15,11 +15,15 @@ typedef unsigned int vec16 __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(kThreads) void gather_rows_kernel(
     const char* __restrict__ src, int64_t src_batch_stride, int64_t row_bytes,
     const int64_t* __restrict__ index, int64_t index_batch_stride, int n_src,
-    char* __restrict__ dst, int64_t dst_batch_stride, int64_t dst_row_stride, int vec_bytes) {
+    char* __restrict__ dst, int64_t dst_batch_stride, int64_t dst_row_stride, int vec_bytes,
+    const int32_t* __restrict__ row_start) {
   const int t = blockIdx.x, b = blockIdx.y;
   const int64_t r = index[(int64_t)b * index_batch_stride + t];
-  if (r < 0 || r >= n_src) return;  // a corrupt index must not leave the buffer
-  const char* s = src + (int64_t)b * src_batch_stride + r * row_bytes;
+  // packed source rows (row_start): batch row b owns rows [row_start[b], row_start[b + 1])
+  const int64_t first = row_start ? row_start[b] : 0;
+  const int64_t limit = row_start ? row_start[b + 1] - first : n_src;
+  if (r < 0 || r >= limit || r >= n_src) return;  // a corrupt index must not leave the buffer
+  const char* s = src + (row_start ? first * row_bytes : (int64_t)b * src_batch_stride) + r * row_bytes;
   char* d = dst + (int64_t)b * dst_batch_stride + (int64_t)t * dst_row_stride;
   if (vec_bytes == 16) {
     const int64_t n = row_bytes >> 4;
@@ -203,7 +207,7 @@ extern "C" int rd_unpack_rows(const void* packed, int64_t packed_batch_stride_by
                               int64_t row_bytes, const int64_t* index, int64_t index_batch_stride,
                               int batch, int n_out, int n_src, void* out,
                               int64_t out_batch_stride_bytes, int64_t out_row_stride_bytes,
-                              void* stream) {
+                              const int32_t* row_start, void* stream) {
   RD_REQUIRE(batch > 0 && n_out > 0 && n_src > 0 && row_bytes > 0, RD_EINVAL,
              "rd_unpack_rows: bad sizes (batch %d n_out %d n_src %d row_bytes %lld)", batch, n_out,
              n_src, (long long)row_bytes);
@@ -215,16 +219,16 @@ extern "C" int rd_unpack_rows(const void* packed, int64_t packed_batch_stride_by
              (long long)out_row_stride_bytes, (long long)row_bytes);
   RD_REQUIRE(out_batch_stride_bytes >= (int64_t)(n_out - 1) * out_row_stride_bytes + row_bytes,
              RD_EINVAL, "rd_unpack_rows: out_batch_stride_bytes too small");
-  RD_REQUIRE(packed_batch_stride_bytes >= (int64_t)n_src * row_bytes, RD_EINVAL,
+  RD_REQUIRE(row_start || packed_batch_stride_bytes >= (int64_t)n_src * row_bytes, RD_EINVAL,
              "rd_unpack_rows: packed_batch_stride_bytes too small");
   const uintptr_t all = (uintptr_t)packed | (uintptr_t)out | (uintptr_t)row_bytes |
-                        (uintptr_t)packed_batch_stride_bytes | (uintptr_t)out_batch_stride_bytes |
+                        (uintptr_t)(row_start ? 0 : packed_batch_stride_bytes) | (uintptr_t)out_batch_stride_bytes |
                         (uintptr_t)out_row_stride_bytes;
   const int vec = (all % 16 == 0) ? 16 : (all % 4 == 0 ? 4 : 1);
   { rd::ScopedTiming rd_t("gather_rows_kernel", rd::as_stream(stream)); hipLaunchKernelGGL(gather_rows_kernel, dim3(n_out, batch), dim3(kThreads), 0,
                      rd::as_stream(stream), reinterpret_cast<const char*>(packed),
                      packed_batch_stride_bytes, row_bytes, index, index_batch_stride, n_src,
-                     reinterpret_cast<char*>(out), out_batch_stride_bytes, out_row_stride_bytes, vec); }
+                     reinterpret_cast<char*>(out), out_batch_stride_bytes, out_row_stride_bytes, vec, row_start); }
   return rd::check_launch("rd_unpack_rows");
 }
 

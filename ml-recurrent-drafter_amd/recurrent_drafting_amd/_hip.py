@@ -20,7 +20,7 @@ import sys
 _DEFAULT_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libredrafter_hip.so")
 _LIB_PATH = os.environ.get("RD_HIP_LIBRARY") or _DEFAULT_LIB_PATH
 _lib = None
-ABI_VERSION = 103  # RD_ABI_VERSION of include/redrafter_hip.h that _PROTOTYPES below was written against
+ABI_VERSION = 104  # RD_ABI_VERSION of include/redrafter_hip.h that _PROTOTYPES below was written against
 
 RD_BF16, RD_F16, RD_F32 = 0, 1, 2
 _DTYPES = {torch.bfloat16: RD_BF16, torch.float16: RD_F16, torch.float32: RD_F32}
@@ -38,13 +38,13 @@ _PROTOTYPES = {
     "rd_tree_workspace_bytes": (_Z, [_I, _I, _I]),
     "rd_tree_build": (_I, [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "rd_tree_mask": (_I, [_P, _P, _P, _P, _I, _L, _L, _L, _I, _I, _I, _P, _P]),
-    "rd_unpack_rows": (_I, [_P, _L, _L, _P, _L, _I, _I, _I, _P, _L, _L, _P]),
-    "rd_argmax_rows": (_I, [_P, _I, _L, _L, _L, _P, _P]),
+    "rd_unpack_rows": (_I, [_P, _L, _L, _P, _L, _I, _I, _I, _P, _L, _L, _P, _P]),
+    "rd_argmax_rows": (_I, [_P, _I, _L, _L, _L, _P, _P, _P]),
     "rd_accept_greedy": (_I, [_P, _P, _L, _P, _I, _I, _I, _P, _P, _P, _P, _P]),
     "rd_count_left_paddings": (_I, [_P, _L, _L, _I, _L, _P, _P]),
     "rd_position_ids": (_I, [_P, _L, _L, _I, _L, _P, _L, _I, _P, _P]),
     "rd_realign_plan_ints": (_Z, [_I, _I]),
-    "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P, _P, _P]),
+    "rd_realign_plan": (_I, [_P, _L, _L, _P, _P, _P, _P, _I, _I, _I, _L, _P, _P, _P, _P, _P, _P]),
     "rd_kv_unpack": (_I, [_P, _I, _I, _I, _L, _L, _L, _P, _I, _I, _P]),
     "rd_kv_compact": (_I, [_P, _I, _I, _I, _L, _L, _L, _I, _P, _P]),
     "rd_kv_append": (_I, [_P, _I, _I, _I, _L, _L, _I, _P, _P]),

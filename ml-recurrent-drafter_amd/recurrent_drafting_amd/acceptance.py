@@ -23,21 +23,31 @@ def _select_one_per_row(x: torch.Tensor, batch_index: torch.Tensor) -> torch.Ten
     return out.view((B,) + tuple(rest))
 
 
-def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
-    """torch.argmax(logits, dim=-1) with the first-maximum rule, one pass over the logits."""
+def argmax_rows(logits: torch.Tensor, rows=None) -> torch.Tensor:
+    """torch.argmax(logits, dim=-1) with the first-maximum rule, one pass over the logits.
+
+    rows (a packed_rows.PackedRows): logits holds one row per packed row, and the result comes back
+    as (batch, n) with the argmax of every slot that exists at its place -- the kernel writes it
+    there; the slots that do not exist hold whatever the allocation held (nothing reads them: the
+    unpacker only names slots that exist)."""
     V = logits.shape[-1]
     lead = logits.shape[:-1]
     x = logits.reshape(-1, V)
     if x.stride(1) != 1:
         x = x.contiguous()
-    out = torch.empty(x.shape[0], dtype=torch.long, device=x.device)
+    if rows is None:
+        n_rows, out, where = x.shape[0], torch.empty(x.shape[0], dtype=torch.long, device=x.device), None
+    else:
+        assert x.shape[0] == rows.rows
+        n_rows, where = rows.total, rows.index
+        out = torch.empty(rows.batch * rows.n, dtype=torch.long, device=x.device)
     _hip.check(
         _hip.lib().rd_argmax_rows(
-            _hip.ptr(x), _hip.dtype_code(x.dtype), x.shape[0], V, x.stride(0), _hip.ptr(out),
+            _hip.ptr(x), _hip.dtype_code(x.dtype), n_rows, V, x.stride(0), _hip.ptr(out), _hip.ptr(where),
             _hip.stream(),
         )
     )
-    return out.view(lead)
+    return out.view(lead) if rows is None else out.view(rows.batch, rows.n)
 
 
 def _count_left_paddings(tokens: torch.Tensor, pad_token_id: int) -> torch.Tensor:
@@ -161,16 +171,20 @@ def realign_enqueue(
     pad_token_id: int,
     unpacker: Optional[torch.Tensor] = None,
     left_pads: Optional[torch.Tensor] = None,
+    step_out: Optional[torch.Tensor] = None,
 ) -> PendingRealign:
     """Appends the accepted tokens to ids and cache and re-right-aligns both; nothing is read back.
 
     With unpacker=None the cache must already be unpacked (Cache.unpack); with the unpacker given
     the accepted rows are taken straight from the packed slots and the unpack step is not needed.
-    left_pads: (B,) int32 leading pad counts of input_ids, if the caller has them already."""
+    left_pads: (B,) int32 leading pad counts of input_ids, if the caller has them already.
+    step_out: two int32 on the device that receive the new length and the accepted tokens summed
+    over the rows (for a caller that reads them together with something else)."""
     assert input_ids.dtype == torch.long, f"prev_input_ids.dtype {input_ids.dtype} is not long"
     B, W, L = beams.shape
     prev = input_ids.shape[1]
     assert left_pads is None or (left_pads.shape == (B,) and left_pads.dtype == torch.int32 and left_pads.is_contiguous())
+    assert step_out is None or (step_out.shape == (2,) and step_out.dtype == torch.int32 and step_out.is_contiguous())
     if prev > 0 and input_ids.stride(1) != 1:
         input_ids = input_ids.contiguous()
     beams = beams.contiguous()
@@ -187,7 +201,8 @@ def realign_enqueue(
             _hip.ptr(input_ids) if prev > 0 else None, input_ids.stride(0), prev,
             _hip.ptr(n_tokens_in_seq), _hip.ptr(seq_in_beam), _hip.ptr(beams), _hip.ptr(unpacker),
             B, W, L, pad_token_id, _hip.ptr(plan), _hip.ptr(ids_buf),
-            _hip.ptr(cache.shift) if cache.rows_in_place else None, _hip.ptr(left_pads), _hip.stream(),
+            _hip.ptr(cache.shift) if cache.rows_in_place else None, _hip.ptr(left_pads), _hip.ptr(step_out),
+            _hip.stream(),
         )
     )
     if cache.rows_in_place:

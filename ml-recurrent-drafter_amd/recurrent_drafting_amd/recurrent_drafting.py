@@ -175,7 +175,7 @@ class RecurrentDrafting(torch.nn.Module):
     # sequence length, accepted tokens, packed tree length, tree slots) and fetches them in ONE
     # read, after the next step's draft has been queued: the drafter's many small launches run
     # behind the model forward instead of in front of an idle GPU.
-    def _draft(self, step_record, context, init_tokens, beam_shape, greedy) -> "_Drafted":
+    def _draft(self, step_record, context, init_tokens, beam_shape, greedy, counts=None) -> "_Drafted":
         # every step times one draft, the one it queues for its successor; the very first draft
         # (step_record None) is not timed, so that each timer key keeps one entry per step
         timer = step_record.time("generate_candidates") if step_record is not None else contextlib.nullcontext()
@@ -184,9 +184,9 @@ class RecurrentDrafting(torch.nn.Module):
                 context, init_tokens, self.llm.base_model.get_input_embeddings(), beam_shape,
                 return_log_probs=not greedy,
             )
-            return _Drafted(beams, log_q, tree_attention.build_tree_enqueue(beams))
+            return _Drafted(beams, log_q, tree_attention.build_tree_enqueue(beams, counts))
 
-    def _verify_and_accept(self, step_record, drafted, tree, input_ids, cache, pad, sampling_args):
+    def _verify_and_accept(self, step_record, drafted, tree, input_ids, cache, pad, sampling_args, step_out=None):
         """-> (context, next_tokens, n_tokens, realignment still to be finished)."""
         llm, beams = self.llm, drafted.beams
         greedy = sampling_args.greedy
@@ -210,7 +210,7 @@ class RecurrentDrafting(torch.nn.Module):
                     logits = llm.lm_head(hidden)
         with step_record.time("accept_candidate_tokens"):
             if greedy:
-                llm_tokens = rows.scatter(acceptance.argmax_rows(logits))  # per packed slot
+                llm_tokens = acceptance.argmax_rows(logits, rows)  # (B, n): per packed slot, written in place
                 with step_record.time("choose_from_candidates"):
                     n_tokens, seq_in_beam, next_tokens, last_slot = acceptance.greedy_accept(
                         beams, llm_tokens, tree.unpacker
@@ -227,11 +227,11 @@ class RecurrentDrafting(torch.nn.Module):
             with step_record.time("update_kv_cache_and_input_ids"):
                 realignment = acceptance.realign_enqueue(
                     input_ids, n_tokens, seq_in_beam, beams, cache, pad, unpacker=tree.unpacker,
-                    left_pads=left_pads,
+                    left_pads=left_pads, step_out=step_out,
                 )
             if greedy:
                 with step_record.time("greedy_prepare_next_input"):
-                    context = hidden.index_select(0, rows.row_of(last_slot))
+                    context = tree_attention.gather_rows(hidden, last_slot.unsqueeze(-1), rows=rows)[:, 0, :]
             else:
                 with step_record.time("prepare_next_input"):
                     probs = acceptance.residual_probs(drafted.log_q, log_p, seq_in_beam, n_tokens)
@@ -269,13 +269,17 @@ class RecurrentDrafting(torch.nn.Module):
                 if drafted is None:  # first step: nothing was drafted ahead
                     drafted = self._draft(None, context, init_tokens, beam_shape, sampling_args.greedy)
                     tree = drafted.tree.finish(*drafted.tree.sizes.tolist())
+                # what the host needs between two steps lands in one small buffer: the coming tree's
+                # counts, sizes and row starts (2B+3 ints), then the new length and the accepted tokens
+                step_ints = torch.empty(2 * batch_size + 5, dtype=torch.int32, device=input_ids.device)
                 context, init_tokens, n_tokens, realignment = self._verify_and_accept(
-                    step_record, drafted, tree, input_ids, cache, special_tokens.pad, sampling_args)
-                drafted = self._draft(step_record, context, init_tokens, beam_shape, sampling_args.greedy)
+                    step_record, drafted, tree, input_ids, cache, special_tokens.pad, sampling_args,
+                    step_out=step_ints[2 * batch_size + 3:])
+                drafted = self._draft(step_record, context, init_tokens, beam_shape, sampling_args.greedy,
+                                      counts=step_ints)
                 # the one host read of the step
-                new_len, n_accepted, tree_n, tree_total = torch.cat(
-                    (realignment.new_len, n_tokens.sum(dtype=torch.int32).view(1), drafted.tree.sizes)
-                ).tolist()
+                read = step_ints[batch_size:].tolist()
+                tree_n, tree_total, new_len, n_accepted = read[0], read[1], read[-2], read[-1]
                 input_ids = realignment.finish(new_len)
                 tree = drafted.tree.finish(tree_n, tree_total)
                 output_tokens = torch.cat((input_ids, init_tokens.unsqueeze(-1)), dim=-1)

@@ -51,7 +51,7 @@ class PendingTree:
     `sizes`, on the device) still have to reach the host before the outputs can be shaped."""
 
     slab: torch.Tensor  # (7, B*W*L) int64
-    counts: torch.Tensor  # (2B+3,) int32: counts (B), max, total, row_start (B+1)
+    counts: torch.Tensor  # (2B+3 or more,) int32: counts (B), max, total, row_start (B+1)
     shape: Tuple[int, int, int]
 
     def __post_init__(self):
@@ -62,7 +62,7 @@ class PendingTree:
         self._unpacker = self._rows[1].view(B, W, L)
         self._prefix_tree = self._rows[0].view(B, W, L)
         self._counts = self.counts[: B + 2]
-        self._row_start = self.counts[B + 2 :]
+        self._row_start = self.counts[B + 2 : 2 * B + 3]
         self._sizes = self.counts[B : B + 2]
 
     @property
@@ -88,15 +88,18 @@ class PendingTree:
         )
 
 
-def build_tree_enqueue(beams: torch.Tensor) -> PendingTree:
+def build_tree_enqueue(beams: torch.Tensor, counts: Optional[torch.Tensor] = None) -> PendingTree:
     """Dedup + unpacker + pack + position offsets in two launches (tree_attention.py:331-335);
-    nothing is read back."""
+    nothing is read back.  counts: an int32 device buffer of at least 2B+3 elements to write the
+    counts into (a caller that reads the sizes together with other numbers owns a longer one)."""
     B, W, L = _check_beams(beams)
     beams = beams.contiguous()
     dev = beams.device
     n_tok = B * W * L
     slab = torch.empty((7, n_tok), dtype=torch.long, device=dev)
-    counts = torch.empty(2 * B + 3, dtype=torch.int32, device=dev)  # counts (B+2), then row_start (B+1)
+    if counts is None:
+        counts = torch.empty(2 * B + 3, dtype=torch.int32, device=dev)  # counts (B+2), then row_start (B+1)
+    assert counts.dtype == torch.int32 and counts.numel() >= 2 * B + 3 and counts.is_contiguous()
     lib = _hip.lib()
     ws_bytes = lib.rd_tree_workspace_bytes(B, W, L)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
@@ -204,14 +207,22 @@ def _pack_beams(
 
 
 def gather_rows(
-    packed: torch.Tensor, index: torch.Tensor, out: Optional[torch.Tensor] = None
+    packed: torch.Tensor, index: torch.Tensor, out: Optional[torch.Tensor] = None,
+    rows: Optional[PackedRows] = None,
 ) -> torch.Tensor:
     """out[b, t, :] = packed[b, index[b, t], :] for packed (B, n, F) and index (B, T) int64.
 
     `out`, if given, is a (B, T, F) view whose last dimension is contiguous (any row/batch stride),
-    e.g. one time slice of a (B, T, steps, F) history."""
-    assert packed.dim() == 3 and index.dim() == 2 and index.dtype == torch.long
-    B, n_src, F = packed.shape
+    e.g. one time slice of a (B, T, steps, F) history.  With `rows`, packed is (rows.rows, F), the
+    slots that exist batch row after batch row, and index[b, t] is a slot of batch row b."""
+    assert index.dim() == 2 and index.dtype == torch.long
+    if rows is not None:
+        assert packed.dim() == 2 and packed.shape[0] == rows.rows and index.shape[0] == rows.batch
+        packed = packed.unsqueeze(0)  # (1, rows, F): the batch stride is not used
+        B, n_src, F = rows.batch, rows.n, packed.shape[2]
+    else:
+        assert packed.dim() == 3
+        B, n_src, F = packed.shape
     T = index.shape[1]
     assert index.shape[0] == B
     if packed.stride(2) != 1 or packed.stride(1) != F:
@@ -224,7 +235,8 @@ def gather_rows(
     _hip.check(
         _hip.lib().rd_unpack_rows(
             _hip.ptr(packed), packed.stride(0) * es, F * es, _hip.ptr(index), T, B, T, n_src,
-            _hip.ptr(out), out.stride(0) * es, out.stride(1) * es, _hip.stream(),
+            _hip.ptr(out), out.stride(0) * es, out.stride(1) * es,
+            _hip.ptr(rows.row_start) if rows is not None else None, _hip.stream(),
         )
     )
     return out

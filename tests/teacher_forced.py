@@ -163,10 +163,12 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
         seen.update(tree=tree, ids=padding_mask, bits=prepared.bits, position_ids=position_ids, left_pads=left_pads)
         return out
 
-    def w_argmax(logits):
-        out = real_argmax(logits)
+    def w_argmax(logits, rows=None):
+        out = real_argmax(logits, rows)
         if "tree" in seen:  # (the prefill calls it too, before any tree exists)
-            seen.update(logits=logits, argmax=out)
+            # (with `rows` the result sits at the (batch, slot) places: back to packed-row order)
+            packed = out if rows is None else out.flatten().index_select(0, rows.index[: rows.total])
+            seen.update(logits=logits, argmax=packed)
         return out
 
     def w_accept(beams, llm_tokens, unpacker=None):
@@ -178,10 +180,10 @@ def run(llm, drafter, ids, max_length: int, W: int, L: int, steps: int, pad: int
                     next_tokens=nxt, last_slot=last)
         return n, s, nxt, last
 
-    def w_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker=None, left_pads=None):
+    def w_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker=None, left_pads=None, step_out=None):
         seen.update(cache=cache, shift=cache.shift.clone(),
                     snap=_snapshot(cache, cache.sliced[0][0].length))
-        return real_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker, left_pads)
+        return real_realign(input_ids, n, s, beams, cache, pad_token_id, unpacker, left_pads, step_out)
 
     drafts = []  # draft k feeds step k; it is queued while step k-1 is being finished
 

@@ -140,3 +140,66 @@ def test_tree_build_lists_the_slots_that_exist():
         assert got.tokens is not None and got.tokens.shape == taken.shape
         assert torch.equal(got.tokens[: got.total], taken[: got.total]) and not got.tokens[got.total :].any()
         assert got.take_tokens(tree.packed_beams) is got.tokens
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_argmax_of_packed_rows_lands_at_the_slots(dtype):
+    """rd_argmax_rows with an output index: the argmax of every packed row at its (batch, slot) place,
+    equal to the plain argmax scattered by torch; the stand-in rows behind the last packed row are
+    not run."""
+    from recurrent_drafting_amd import acceptance
+
+    counts, n, V = [9, 1, 14, 6], 14, 777
+    rows = _rows(counts, n)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    logits = torch.randn(rows.rows, V, generator=g, device="cuda").to(dtype)
+    plain = acceptance.argmax_rows(logits)
+    assert torch.equal(plain, logits.float().argmax(dim=-1))
+    placed = acceptance.argmax_rows(logits, rows)
+    assert placed.shape == (len(counts), n)
+    want = rows.scatter(plain, fill=-1)
+    exists = want >= 0
+    assert int(exists.sum()) == rows.total
+    assert torch.equal(placed[exists], want[exists])
+
+
+def test_gather_of_packed_rows_by_slot():
+    """rd_unpack_rows with row_start: row (b, slot) of a (rows, F) tensor of packed rows; a slot a batch
+    row does not have leaves its output row as it was."""
+    from recurrent_drafting_amd import tree_attention
+
+    counts, n, F = [9, 1, 14, 6], 14, 96
+    rows = _rows(counts, n)
+    g = torch.Generator(device="cuda").manual_seed(4)
+    packed = torch.randn(rows.rows, F, generator=g, device="cuda").to(torch.bfloat16)
+    slots = torch.tensor([[8, 0], [0, 0], [13, 5], [2, 5]], device="cuda")
+    got = tree_attention.gather_rows(packed, slots, rows=rows)
+    want = packed.index_select(0, (rows.row_start[:-1].long()[:, None] + slots).flatten()).view(4, 2, F)
+    assert torch.equal(got, want)
+    out = torch.full((4, 1, F), 7.0, dtype=torch.bfloat16, device="cuda")
+    tree_attention.gather_rows(packed, torch.tensor([[9], [1], [14], [5]], device="cuda"), out=out, rows=rows)
+    assert bool((out[:3] == 7.0).all())  # slots 9, 1 and 14 do not exist in rows 0, 1 and 2
+    assert torch.equal(out[3, 0], packed[int(rows.row_start[3]) + 5])
+
+
+def test_realign_reports_the_new_length_and_the_accepted_tokens():
+    """rd_realign_plan's step_out: the new length M and the accepted tokens summed over the rows."""
+    from recurrent_drafting_amd import acceptance, kv_cache, tree_attention
+
+    torch.manual_seed(5)
+    B, W, L, prev = 4, 5, 4, 9
+    ids = torch.randint(1, 50, (B, prev), device="cuda")
+    ids[1, :3] = 0
+    ids[3, :1] = 0
+    beams = torch.randint(1, 50, (B, W, L), device="cuda")
+    beams[:, :, 0] = beams[:, :1, 0]
+    tree = tree_attention.build_tree(beams)
+    cache = kv_cache.Cache(B, prev + W * L + 4, 1, 2, 8, torch.float32, torch.device("cuda"))
+    cache.set_length(prev + tree.n)
+    n_tokens = torch.tensor([3, 0, 2, 1], device="cuda")
+    seq = torch.tensor([1, 0, 4, 2], device="cuda")
+    out = torch.full((2,), -1, dtype=torch.int32, device="cuda")
+    pending = acceptance.realign_enqueue(ids, n_tokens, seq, beams, cache, 0, unpacker=tree.unpacker, step_out=out)
+    new_len = int(pending.new_len.item())
+    assert out.tolist() == [new_len, 6]
+    assert new_len == max(prev - p + n + 1 for p, n in zip([0, 3, 0, 1], [3, 0, 2, 1]))

@@ -109,7 +109,7 @@ def test_verification_and_acceptance_limits(lib):
     assert sample(width=65536) == ELIMIT
 
     def argmax(rows=1448, vocab=32000, stride=32000):
-        return lib.rd_argmax_rows(None, 0, rows, vocab, stride, None, None)
+        return lib.rd_argmax_rows(None, 0, rows, vocab, stride, None, None, None)
 
     assert argmax() == EINVAL and b"null" in lib.rd_last_error()
     assert argmax(stride=31999) == EINVAL and b"null" not in lib.rd_last_error()
@@ -134,7 +134,7 @@ def test_mask_and_row_movement_limits(lib):
 
     def unpack(batch=8, n_out=225, n_src=168, row_bytes=8192):
         return lib.rd_unpack_rows(None, n_src * row_bytes, row_bytes, None, n_out, batch, n_out, n_src, None,
-                                  n_out * row_bytes, row_bytes, None)
+                                  n_out * row_bytes, row_bytes, None, None)
 
     assert unpack() == EINVAL and b"null" in lib.rd_last_error()
     assert unpack(batch=65536) == ELIMIT
