@@ -44,7 +44,7 @@ typedef enum { RD_BF16 = 0, RD_F16 = 1, RD_F32 = 2 } rd_dtype;
  * that crosses it (the attention plan, the realignment plan) or a workspace size changes.  A caller
  * compiled against this header compares rd_version() with RD_ABI_VERSION before its first call, so
  * that a stale build of the library is refused instead of being called with other arguments. */
-#define RD_ABI_VERSION 104
+#define RD_ABI_VERSION 105
 RD_API int rd_version(void);
 /* Message of the last failed call on this thread ("" if none). */
 RD_API const char* rd_last_error(void);
@@ -316,9 +316,12 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
  * views View.cat returns (kv_cache.py:24-31).  bf16 with head_dim 128 runs on the MFMA kernel
  * (needs 16-byte aligned q/k/v, strides that are multiples of 8 elements, and the workspace);
  * everything else (more than 128 heads included), or force_generic != 0, runs on the generic
- * kernel (head_dim <= 256).  The plan is READ AND WRITTEN: its arrival counters (its tail) are
- * counted up and left at zero by every call, so calls that share a plan must run one after the
- * other on one stream (the layers of a forward do); a plan per stream otherwise.
+ * kernel (head_dim <= 256).  The plan and the bits are only read, so any number of calls, on any
+ * streams, may share them.  Rows whose keys are split over several work items are merged by the
+ * item that finishes last; the arrival counters for that are the library's (a ring of 2^18 per
+ * GPU, of which every call takes batch * n_heads * ceil(n_q / rows per work group) for itself,
+ * RD_ELIMIT beyond the ring) and leaves at zero, so calls that are in flight together do not meet
+ * on a counter; each call needs a workspace of its own while it runs.
  * row_start (batch + 1 int32 on the device, or NULL): packed query rows, as in rd_rope_append:
  * query t of batch row b is row row_start[b] + t of q and of out (sequence stride; their batch
  * strides are unused), queries t >= row_start[b+1] - row_start[b] are neither read nor written.
@@ -358,7 +361,7 @@ RD_API int rd_verify_attention(const void* q, const int64_t* q_strides, const vo
                                const int64_t* k_strides, const void* v, const int64_t* v_strides,
                                void* out, const int64_t* o_strides, int dtype, int batch,
                                int n_heads, int n_kv_heads, int n_q, int kv_len, int head_dim,
-                               float scale, const uint64_t* bits, int32_t* plan,
+                               float scale, const uint64_t* bits, const int32_t* plan,
                                void* workspace, size_t workspace_bytes, int force_generic,
                                const int32_t* row_start, void* stream);
 /* rd_rope_verify_attention: rd_rope_append followed by rd_verify_attention for the new tokens of one
@@ -386,7 +389,7 @@ RD_API int rd_rope_verify_attention(const void* q, const int64_t* q_strides, con
                                     const int64_t* cache_strides, int64_t max_len, void* out,
                                     const int64_t* o_strides, int dtype, int batch, int n_heads,
                                     int n_kv_heads, int n_q, int kv_len, int head_dim, float scale,
-                                    const uint64_t* bits, int32_t* plan, void* workspace,
+                                    const uint64_t* bits, const int32_t* plan, void* workspace,
                                     size_t workspace_bytes, const int32_t* row_start, void* stream);
 
 /* ------------------------------------------------------------------------------------------

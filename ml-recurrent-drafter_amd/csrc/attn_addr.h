@@ -165,8 +165,8 @@ RD_HD int64_t mask_word_index(int b, int n_q, int q_row, int words, int key0) {
 RD_HD int64_t partial_row(int b, int H, int h, int max_splits, int split, int n_q, int q_row) {
   return ((((int64_t)b * H + h) * max_splits) + split) * n_q + q_row;
 }
-RD_HD int64_t counter_index(int b, int max_heads, int h, int q_tiles, int q_tile) {
-  return ((int64_t)b * max_heads + h) * q_tiles + q_tile;
+RD_HD int64_t counter_index(int b, int n_heads, int h, int q_tiles, int q_tile) {
+  return ((int64_t)b * n_heads + h) * q_tiles + q_tile;
 }
 
 

@@ -12,8 +12,8 @@
 //     boundary, key_end), and the keys of the first and last tile outside the span (left padding,
 //     tree slots that do not exist: masked for every query) are never read from memory
 //   scratch: first and last attended key of every (b, q) row (two arrays of batch * n_q)
-//   arrival counters, one per (b, head, query tile), zero between launches: the work items of a
-//   split row count themselves in, and the last one to arrive merges the partials of all
+// The plan is read-only for the attention kernels: the arrival counters of split rows live in a
+// device array of the library (verify_attention.hip), a fresh slab of it for every launch.
 //
 // Nothing here needs the HIP runtime: the sizes and the arithmetic that decides how a row's keys
 // are cut into work items compile for the device and for the host alike, so that a host program
@@ -33,16 +33,17 @@ namespace rd {
 constexpr int kAttnChunk = 512;       // target keys per work item
 constexpr int kAttnSortLimit = 2048;  // more items than this are dispatched unsorted
 
-constexpr int kAttnMaxHeads = 128;    // heads the arrival counters are laid out for
+constexpr int kAttnMaxHeads = 128;    // heads the MFMA kernel takes
 constexpr int kAttnRowsPerTile = 256; // query rows of the largest workgroup layout
 
 inline int attn_max_splits(int kv_len) { return (kv_len + kAttnChunk - 1) / kAttnChunk; }
 inline int attn_max_q_tiles(int n_q) { return (n_q + kAttnRowsPerTile - 1) / kAttnRowsPerTile; }
-inline size_t attn_counter_offset(int batch, int n_q, int kv_len) {
+inline size_t attn_plan_ints(int batch, int n_q, int kv_len) {
   return RD_PLAN_HDR + 4 * (size_t)batch + RD_ITEM_INTS * (size_t)batch * attn_max_splits(kv_len) + 2 * (size_t)batch * n_q;
 }
-inline size_t attn_counter_ints(int batch, int n_q) {
-  return (size_t)batch * kAttnMaxHeads * attn_max_q_tiles(n_q);
+// arrival counters of one launch: one per (batch row, head, query tile)
+inline size_t attn_counter_ints(int batch, int n_heads, int n_q) {
+  return (size_t)batch * n_heads * attn_max_q_tiles(n_q);
 }
 
 // ---- how a row's keys become work items ------------------------------------------------------

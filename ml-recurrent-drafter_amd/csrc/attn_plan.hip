@@ -61,12 +61,10 @@ __global__ __launch_bounds__(kThreads) void mask_bits_kernel(
 // written here, never read back: a serial loop over rows would pay a trip to memory per row).
 __device__ __forceinline__ void build_plan(const int* s_key_min, const int* s_key_end, int* s_rows, int B, int n_q, int kv_len,
                            int words, int min_chunk, int max_splits, int n_heads, int n_cu,
-                           const int32_t* __restrict__ kv_shift, int32_t* __restrict__ plan,
-                           int32_t* __restrict__ counters, int n_counters) {
+                           const int32_t* __restrict__ kv_shift, int32_t* __restrict__ plan) {
   __shared__ int s_n_items;
   __shared__ int s_chunk;
   __shared__ int s_len[rd::kAttnSortLimit];
-  for (int i = threadIdx.x; i < n_counters; i += kThreads) counters[i] = 0;
   int32_t* per_row = plan + RD_PLAN_HDR;
   int* s_splits = s_rows;
   int* s_first_item = s_rows + B;
@@ -247,9 +245,7 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
                                                              int min_chunk, int max_splits,
                                                              int n_heads, int n_cu,
                                                              const int32_t* __restrict__ kv_shift,
-                                                             int32_t* __restrict__ plan,
-                                                             int32_t* __restrict__ counters,
-                                                             int n_counters) {
+                                                             int32_t* __restrict__ plan) {
   extern __shared__ int s_span[];  // [4][B]: first key any query of the row attends to, last such key + 1, build_plan's rows
   int* s_key_min = s_span;
   int* s_key_end = s_span + B;
@@ -273,8 +269,7 @@ __global__ __launch_bounds__(kThreads) void attn_plan_kernel(const int32_t* __re
       s_key_end[b] = last + 1;
     }
   }
-  build_plan(s_key_min, s_key_end, s_span + 2 * B, B, n_q, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan,
-             counters, n_counters);
+  build_plan(s_key_min, s_key_end, s_span + 2 * B, B, n_q, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -318,7 +313,7 @@ __global__ __launch_bounds__(kThreads) void tree_prepare_kernel(
     const int32_t* __restrict__ counts, const PM* __restrict__ padding_mask, int64_t pm_row_stride,
     int64_t pm_pad_value, int64_t prev, int B, int WL, int L, int n, int words, int n_heads, int n_cu,
     int min_chunk, int max_splits, const int32_t* __restrict__ kv_shift, uint64_t* __restrict__ bits,
-    int32_t* __restrict__ plan, int32_t* __restrict__ counters, int n_counters,
+    int32_t* __restrict__ plan,
     int64_t* __restrict__ position_ids, int32_t* __restrict__ left_pads) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kv_len = (int)prev + n;
@@ -342,8 +337,7 @@ __global__ __launch_bounds__(kThreads) void tree_prepare_kernel(
         if (left_pads) left_pads[b] = first;
       }
     }
-    build_plan(s_key_min, s_key_end, s_span + 2 * B, B, n, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan,
-               counters, n_counters);
+    build_plan(s_key_min, s_key_end, s_span + 2 * B, B, n, kv_len, words, min_chunk, max_splits, n_heads, n_cu, kv_shift, plan);
     return;
   }
   // ---- mask bits and position ids of kTreeSlots slots of one batch row -------------------------
@@ -384,7 +378,7 @@ __global__ __launch_bounds__(kThreads) void tree_prepare_kernel(
 
 extern "C" size_t rd_attn_plan_ints(int batch, int n_q, int kv_len) {
   if (batch <= 0 || n_q <= 0 || kv_len <= 0) return 0;
-  return rd::attn_counter_offset(batch, n_q, kv_len) + rd::attn_counter_ints(batch, n_q);
+  return rd::attn_plan_ints(batch, n_q, kv_len);
 }
 
 extern "C" size_t rd_attn_bits_words(int batch, int n_q, int kv_len) {
@@ -428,8 +422,7 @@ extern "C" int rd_attn_prepare(const uint8_t* mask, int64_t mask_stride_b, int64
                      mask_stride_q, n_q, kv_len, words, fix_empty_rows, bits, row_first, row_last); }
   if (int e = rd::check_launch("rd_attn_prepare(bits)")) return e;
   { rd::ScopedTiming rd_t("attn_plan_kernel", s); hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(kThreads), 4 * batch * sizeof(int), s, row_first, row_last, batch, n_q, kv_len,
-                     words, rd::kAttnChunk, max_splits, n_heads, compute_units(), kv_row_shift, plan,
-                     plan + rd::attn_counter_offset(batch, n_q, kv_len), (int)rd::attn_counter_ints(batch, n_q)); }
+                     words, rd::kAttnChunk, max_splits, n_heads, compute_units(), kv_row_shift, plan); }
   return rd::check_launch("rd_attn_prepare(plan)");
 }
 
@@ -459,14 +452,12 @@ extern "C" int rd_tree_attn_prepare(const int64_t* unpacker, const int64_t* pack
   const int max_splits = rd::attn_max_splits(kv_len);
   hipStream_t s = rd::as_stream(stream);
   const dim3 grid((n + kTreeSlots - 1) / kTreeSlots, batch + 1);
-  int32_t* counters = plan + rd::attn_counter_offset(batch, n, kv_len);
-  const int n_counters = (int)rd::attn_counter_ints(batch, n);
 #define RD_LAUNCH_TP(T)                                                                               \
   do { rd::ScopedTiming rd_t("tree_prepare_kernel", s);                                               \
     hipLaunchKernelGGL(tree_prepare_kernel<T>, grid, dim3(kThreads), 4 * batch * sizeof(int), s, unpacker, \
                        packed_token_indices, counts, reinterpret_cast<const T*>(padding_mask), pm_row_stride,  \
                        pm_pad_value, prev, batch, width * length, length, n, words, n_heads, compute_units(),  \
-                       rd::kAttnChunk, max_splits, kv_row_shift, bits, plan, counters, n_counters, position_ids, \
+                       rd::kAttnChunk, max_splits, kv_row_shift, bits, plan, position_ids, \
                        left_pads); } while (0)
   if (pm_elem_bytes == 1) RD_LAUNCH_TP(uint8_t);
   else if (pm_elem_bytes == 4) RD_LAUNCH_TP(int32_t);

@@ -24,11 +24,13 @@
 //                         correctness path for shapes the MFMA kernel does not cover.
 // Work items come from the plan (attn_plan.h): (batch row, key range) chunks, longest first; rows
 // whose keys are split over several items write fp32 partials, and the item that finishes last
-// merges them (an arrival counter per (row, head, query tile) in the plan).
+// merges them (an arrival counter per (row, head, query tile); every launch counts on a slab of its
+// own, taken from a ring of counters that is part of the library).
 #include <hip/hip_bf16.h>
 #include <hip/hip_ext.h>
 #include <hip/hip_fp16.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "attn_addr.h"
@@ -58,7 +60,7 @@ struct AttnArgs {
   // batch strides are unused) and exists only for t < row_start[b + 1] - row_start[b].  The mask
   // rows and the partials keep the padded (batch, n_q) layout.
   const int32_t* row_start;
-  int32_t* counters;  // arrival counters of the plan: [batch][kAttnMaxHeads][query tiles], zero between launches
+  unsigned int* counters;  // arrival counters of this launch, [batch][heads][query tiles]; zero before and after
   int B, H, Hkv, n_q, kv_len, words, max_splits, D;
   float scale;  // softmax scale; the MFMA kernel works in log2 units (scale * log2 e)
   // Rotary embedding and cache append fused in (the ROPE instantiation of the MFMA kernel): q arrives
@@ -779,10 +781,10 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   int* s_last = reinterpret_cast<int*>(smem);  // (the tile buffers are free by now)
-  int32_t* counter = a.counters + counter_index(b, rd::kAttnMaxHeads, h, q_tiles, q_tile);
+  unsigned int* counter = a.counters + counter_index(b, a.H, h, q_tiles, q_tile);
   if (wave == 0) {
     int last = 0;
-    if (lane == 0) last = atomicAdd(counter, 1) == n_splits - 1;
+    if (lane == 0) last = atomicAdd(counter, 1u) == (unsigned int)(n_splits - 1);
     last = __builtin_amdgcn_readfirstlane(last);
     if (lane == 0) *s_last = last;
   }
@@ -842,7 +844,8 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       }
     }
   }
-  if (tid == 0) *counter = 0;  // ready for the next launch on this plan
+  // zero again: for the launch that gets this part of the ring next, and for this one's replay by a graph
+  if (tid == 0) *counter = 0u;
 #undef RD_FOR_KEPT_BLOCKS
 }
 
@@ -928,6 +931,49 @@ __global__ __launch_bounds__(kGenThreads) void attn_generic_kernel(AttnArgs a) {
   }
 }
 
+}  // namespace
+
+// Arrival counters of split rows.  Zero when the library is loaded; the item that merges a row puts
+// the row's counter back to zero.  Every launch takes the next slab of the ring, so two launches
+// that are in flight together (on two streams, on one plan or not) count on different counters
+// unless a whole ring's worth of launches (2^18 counters) was enqueued between them.
+constexpr int kArrivalRing = 1 << 18;
+static __device__ unsigned int attn_arrivals[kArrivalRing];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+// `n` counters of the current device's ring; nullptr with a message on failure
+unsigned int* arrival_slab(const char* who, size_t n, int* error) {
+  static std::mutex mu;
+  static unsigned int* base[kMaxDevices] = {nullptr};
+  static size_t next[kMaxDevices] = {0};
+  if (n > (size_t)kArrivalRing) {
+    *error = rd::fail(RD_ELIMIT, "%s: batch x heads x query tiles = %zu arrival counters (at most %d)", who, n, kArrivalRing);
+    return nullptr;
+  }
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    *error = rd::fail(RD_ELAUNCH, "%s: no current device (or an ordinal above %d)", who, kMaxDevices - 1);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (base[dev] == nullptr) {
+    // (the array's name is a host-side stand-in: its address on this GPU is asked for once)
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(attn_arrivals));
+    if (e != hipSuccess || p == nullptr) {
+      *error = rd::fail(RD_ELAUNCH, "%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
+      return nullptr;
+    }
+    base[dev] = reinterpret_cast<unsigned int*>(p);
+  }
+  if (next[dev] + n > (size_t)kArrivalRing) next[dev] = 0;
+  unsigned int* slab = base[dev] + next[dev];
+  next[dev] += n;
+  return slab;
+}
+
 bool mfma_eligible(const AttnArgs& a, int dtype) {
   auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
   auto m8 = [](int64_t s) { return (s % 8) == 0; };
@@ -961,7 +1007,7 @@ struct RopeInputs {
 int verify_attention(const char* who, const void* q, const int64_t* q_strides, const void* k,
                      const int64_t* k_strides, const void* v, const int64_t* v_strides, void* out,
                      const int64_t* o_strides, int dtype, int batch, int n_heads, int n_kv_heads, int n_q,
-                     int kv_len, int head_dim, float scale, const uint64_t* bits, int32_t* plan,
+                     int kv_len, int head_dim, float scale, const uint64_t* bits, const int32_t* plan,
                      void* workspace, size_t workspace_bytes, int force_generic, const int32_t* row_start,
                      const RopeInputs* rope, void* stream) {
   RD_REQUIRE(batch > 0 && n_heads > 0 && n_kv_heads > 0 && n_q > 0 && kv_len > 0 && head_dim > 0,
@@ -971,6 +1017,12 @@ int verify_attention(const char* who, const void* q, const int64_t* q_strides, c
              n_heads, n_kv_heads);
   RD_REQUIRE(head_dim <= 256, RD_ELIMIT, "%s: head_dim %d > 256", who, head_dim);
   RD_REQUIRE(batch <= 65535 && n_heads <= 65535, RD_ELIMIT, "%s: batch/heads > 65535", who);
+  // what the MFMA kernel's launch would need of the ring of arrival counters (asked of every bf16
+  // call of its head size, before any pointer is looked at)
+  RD_REQUIRE(dtype != RD_BF16 || head_dim != kD || n_heads > rd::kAttnMaxHeads || force_generic ||
+                 rd::attn_counter_ints(batch, n_heads, n_q) <= (size_t)kArrivalRing,
+             RD_ELIMIT, "%s: batch x heads x query tiles = %zu arrival counters (at most %d)", who,
+             rd::attn_counter_ints(batch, n_heads, n_q), kArrivalRing);
   RD_REQUIRE(q && k && v && out && bits && plan && q_strides && k_strides && v_strides && o_strides,
              RD_EINVAL, "%s: null pointer", who);
   RD_REQUIRE(dtype == RD_BF16 || dtype == RD_F16 || dtype == RD_F32, RD_EINVAL, "%s: unknown dtype %d", who, dtype);
@@ -985,7 +1037,7 @@ int verify_attention(const char* who, const void* q, const int64_t* q_strides, c
   a.scale = scale;
   a.part_o = nullptr; a.part_ml = nullptr;
   a.row_start = row_start;
-  a.counters = plan + rd::attn_counter_offset(batch, n_q, kv_len);
+  a.counters = nullptr;
   a.k_new = a.v_new = a.cos = a.sin = nullptr;
   a.kn_sb = a.kn_st = a.vn_sb = a.vn_st = a.table_rows = a.pos_sb = a.max_len = 0;
   a.position_ids = nullptr; a.new_col0 = kv_len;
@@ -1028,6 +1080,9 @@ int verify_attention(const char* who, const void* q, const int64_t* q_strides, c
     const int layout = layout_for(n_q);
     const int q_tiles = (n_q + rows_per_wg(layout) - 1) / rows_per_wg(layout);
     RD_REQUIRE(max_items <= 65535 && (int64_t)q_tiles * n_heads <= 2147483647LL, RD_ELIMIT, "%s: grid too large", who);
+    int slab_error = RD_OK;
+    a.counters = arrival_slab(who, rd::attn_counter_ints(batch, n_heads, n_q), &slab_error);
+    if (a.counters == nullptr) return slab_error;
     {
       // when timed, the events carry the kernel's own begin and end (what a kernel trace reports)
       hipEvent_t t0, t1;
@@ -1063,7 +1118,7 @@ extern "C" int rd_verify_attention(const void* q, const int64_t* q_strides, cons
                                    const int64_t* v_strides, void* out, const int64_t* o_strides,
                                    int dtype, int batch, int n_heads, int n_kv_heads, int n_q,
                                    int kv_len, int head_dim, float scale, const uint64_t* bits,
-                                   int32_t* plan, void* workspace, size_t workspace_bytes,
+                                   const int32_t* plan, void* workspace, size_t workspace_bytes,
                                    int force_generic, const int32_t* row_start, void* stream) {
   return verify_attention("rd_verify_attention", q, q_strides, k, k_strides, v, v_strides, out, o_strides, dtype,
                           batch, n_heads, n_kv_heads, n_q, kv_len, head_dim, scale, bits, plan, workspace,
@@ -1082,7 +1137,7 @@ extern "C" int rd_rope_verify_attention(const void* q, const int64_t* q_strides,
                                         const int64_t* cache_strides, int64_t max_len, void* out,
                                         const int64_t* o_strides, int dtype, int batch, int n_heads,
                                         int n_kv_heads, int n_q, int kv_len, int head_dim, float scale,
-                                        const uint64_t* bits, int32_t* plan, void* workspace,
+                                        const uint64_t* bits, const int32_t* plan, void* workspace,
                                         size_t workspace_bytes, const int32_t* row_start, void* stream) {
   const RopeInputs rope{k_new, k_new_strides, v_new, v_new_strides, cos, sin, table_rows, position_ids,
                         pos_batch_stride, max_len};

@@ -188,7 +188,7 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
   const long long slots = (long long)L.B * L.H * max_splits;
   const size_t part_o_bytes = align_up((size_t)slots * L.n_q * kD * sizeof(float), 256);
   const size_t part_ml_bytes = align_up((size_t)slots * L.n_q * 2 * sizeof(float), 256);
-  const size_t plan_ints = rd::attn_counter_offset(L.B, L.n_q, L.kv_len) + rd::attn_counter_ints(L.B, L.n_q);
+  const size_t plan_ints = rd::attn_plan_ints(L.B, L.n_q, L.kv_len);
   CHECK((int)items.size() <= L.B * max_splits, "chunk %d: %zu items, the plan holds %d", chunk, items.size(), L.B * max_splits);
   CHECK(RD_PLAN_HDR + 4 * (size_t)L.B + RD_ITEM_INTS * (size_t)L.B * max_splits <= plan_ints, "item slots beyond the plan");
   CHECK(q_tiles <= rd::attn_max_q_tiles(L.n_q) || L.n_q <= 256, "query tiles %d beyond the counters' %d", q_tiles, rd::attn_max_q_tiles(L.n_q));
@@ -217,8 +217,8 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
       for (int q_tile = 0; q_tile < q_tiles; ++q_tile) {
         if (q_tile * rows_wg >= rows_n) continue;  // the workgroup returns
         ++st.workgroups;
-        const int64_t cidx = counter_index(b, rd::kAttnMaxHeads, h, q_tiles, q_tile);
-        CHECK(cidx >= 0 && (size_t)cidx < rd::attn_counter_ints(L.B, L.n_q), "counter index %lld of %zu", (long long)cidx, rd::attn_counter_ints(L.B, L.n_q));
+        const int64_t cidx = counter_index(b, L.H, h, q_tiles, q_tile);
+        CHECK(cidx >= 0 && (size_t)cidx < rd::attn_counter_ints(L.B, L.H, L.n_q), "counter index %lld of %zu", (long long)cidx, rd::attn_counter_ints(L.B, L.H, L.n_q));
         for (int tid = 0; tid < kThreads; ++tid) {
           const int wave = tid >> 6, lane = tid & 63, g = lane >> 5, r = lane & 31;
           const WaveRole role = wave_role(layout, wave);

@@ -240,10 +240,10 @@ def test_mfma_kernel_split_rows_in_every_layout_against_the_oracle(nq, kv_prev):
 
 
 def test_split_rows_merge_is_repeatable_on_one_plan():
-    """Every row split into many work items (a plan made for one head: minimum-size items): the item that arrives last
-    merges the partials and leaves the plan's arrival counters at zero, so launch after launch on
-    the same plan (one per layer in the model) must give the same bits, equal to the unsplit result
-    up to the rounding of the merge."""
+    """Every row split into many work items (a plan made for one head: minimum-size items): the item
+    that arrives last merges the partials.  Launch after launch on the same plan (one per layer in
+    the model) must give the same bits, equal to the unsplit result up to the rounding of the
+    merge, and the plan itself is only read."""
     from recurrent_drafting_amd import attention
 
     torch.manual_seed(3)
@@ -257,13 +257,66 @@ def test_split_rows_merge_is_repeatable_on_one_plan():
     whole = attention.masked_attention(q, k, v, whole_plan)
     prep = attention.prepare(mask, n_heads=1)
     assert int(prep.plan[0]) >= 3 * B  # really split
+    plan_before = prep.plan.clone()
     first = attention.masked_attention(q, k, v, prep).clone()
     for _ in range(40):
         again = attention.masked_attention(q, k, v, prep)
         assert torch.equal(again, first)
-    counters = prep.plan[-(B * 128 * 1):]
-    assert not counters.any()
+    assert torch.equal(prep.plan, plan_before)
     assert (first.float() - whole.float()).abs().max() <= 2e-2 * whole.float().abs().max()
+
+
+def test_split_rows_merge_when_the_arrival_counters_come_round_again():
+    """The arrival counters are a ring of 2^18 that launches take slabs of in turn: enough launches
+    to go round it more than once (every launch of the second lap counts on counters that another
+    launch used before it), one result throughout."""
+    from recurrent_drafting_amd import attention
+
+    torch.manual_seed(5)
+    B, H, D, nq, kv = 3, 128, 128, 8, 1900
+    q = torch.randn(B, nq, H, D, device="cuda", dtype=torch.bfloat16).permute(0, 2, 1, 3)
+    k = torch.randn(B, 1, kv, D, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(B, 1, kv, D, device="cuda", dtype=torch.bfloat16)
+    mask = torch.rand(B, nq, kv, device="cuda") > 0.3
+    prep = attention.prepare(mask, n_heads=1)
+    assert int(prep.plan[0]) >= 3 * B
+    first = attention.masked_attention(q, k, v, prep).clone()
+    per_launch = B * H
+    laps = 2 * (1 << 18) // per_launch + 3
+    for i in range(laps):
+        again = attention.masked_attention(q, k, v, prep)
+        if i % 16 == 0 or i >= laps - 3:
+            assert torch.equal(again, first), i
+
+
+def test_two_streams_share_one_plan():
+    """Bits and plan are only read and every launch counts arrivals on counters of its own, so two
+    streams may run split rows on one plan at the same time (each with its own workspace)."""
+    import dataclasses
+
+    from recurrent_drafting_amd import attention
+
+    torch.manual_seed(9)
+    B, H, D, nq, kv = 4, 16, 128, 60, 2300
+    q = torch.randn(B, nq, H, D, device="cuda", dtype=torch.bfloat16).permute(0, 2, 1, 3)
+    k = torch.randn(B, 2, kv, D, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(B, 2, kv, D, device="cuda", dtype=torch.bfloat16)
+    mask = torch.rand(B, nq, kv, device="cuda") > 0.5
+    prep_a = attention.prepare(mask, n_heads=1)
+    prep_b = dataclasses.replace(prep_a, workspace=None)
+    assert int(prep_a.plan[0]) >= 3 * B
+    want = attention.masked_attention(q, k, v, prep_a).clone()
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    for _ in range(30):
+        for i, (st, prep) in enumerate(zip(streams, (prep_a, prep_b))):
+            with torch.cuda.stream(st):
+                outs[i].append(attention.masked_attention(q, k, v, prep))
+    torch.cuda.synchronize()
+    for side in outs:
+        for got in side:
+            assert torch.equal(got, want)
 
 
 def test_mfma_kernel_pad_tokens_inside_the_prefix_and_empty_rows():

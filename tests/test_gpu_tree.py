@@ -63,8 +63,6 @@ def _check_prepare_attention(tree, padding_mask, want_mask, want_offsets, pad_va
     n_items = int(b[0])
     used = 8 + 4 * B + 8 * n_items  # header, per-row records, work items (what the attention reads)
     assert np.array_equal(a[:used], b[:used])
-    counters = int(B * 128 * ((n + 255) // 256))
-    assert not a[-counters:].any()
 
 
 def test_reference_literals(literals):

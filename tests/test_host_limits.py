@@ -50,6 +50,22 @@ def test_attention_plan_limits(lib):
     assert tree_prepare(prev=-1) == EINVAL
 
 
+def test_attention_arrival_counter_limit(lib):
+    """The MFMA attention takes batch x heads x query tiles arrival counters of a ring of 2^18."""
+    def attend(batch, heads, n_q, dtype, generic=0):
+        return lib.rd_verify_attention(None, None, None, None, None, None, None, None, dtype, batch, heads, heads,
+                                       n_q, 64, 128, 1.0, None, None, None, 0, generic, None, None)
+
+    import torch
+
+    from recurrent_drafting_amd import _hip
+
+    bf16 = _hip.dtype_code(torch.bfloat16)
+    assert attend(2048, 128, 256, bf16) == EINVAL and b"null" in lib.rd_last_error()   # exactly the ring
+    assert attend(2048, 128, 257, bf16) == ELIMIT and b"arrival counters" in lib.rd_last_error()
+    assert attend(2048, 128, 257, bf16, generic=1) == EINVAL                             # the generic kernel has none
+
+
 def test_tree_limits(lib):
     def build(batch, width, length):
         return lib.rd_tree_build(None, batch, width, length, None, None, None, None, None, None, None, None, None,
