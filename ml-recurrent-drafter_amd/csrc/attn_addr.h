@@ -147,6 +147,27 @@ RD_HD int lds_merge_ml(int pair, int part, int which, int lane) {
 RD_HD int first_block_kept(int part) { return part == 1 ? 2 : 0; }
 RD_HD int blocks_kept(int part) { return part == 2 ? 4 : 2; }
 
+// ---- results on their way out: a wave's rows through LDS --------------------------------------
+// In the accumulators a lane holds four neighbouring dims of ONE query row, so a store instruction
+// of the wave would touch 32 rows with 16 bytes each.  The wave therefore puts its normalised rows
+// (32 rows x the dims it keeps, bf16) into a region of its own and reads them back along the rows:
+// a store instruction then covers whole rows (256 bytes of a full wave's row, 128 of a half wave's).
+// Rows lie 264 bytes apart: the 32 lanes of a half wave, writing 8 bytes each at that stride, hit
+// 64 different banks.
+constexpr int kOutRowBytes = kD * 2 + 8;
+constexpr int kOutWaveBytes = 32 * kOutRowBytes;
+// where lane (r, g) puts the four outputs (block db, group i4): dims 32*db + 8*i4 + 4*g ..
+RD_HD int lds_out_stage(int wave, int r, int g, int db, int i4) {
+  return wave * kOutWaveBytes + r * kOutRowBytes + (32 * db + 8 * i4 + 4 * g) * 2;
+}
+// The way back: piece = 8 bytes = four dims.  A wave that keeps `blocks` accumulator blocks from
+// block `first` on has 8 * blocks pieces per row and takes 64 of them per pass, lane by lane along
+// the rows: 32 * 8 * blocks / 64 passes.
+RD_HD int out_passes(int blocks) { return 32 * 8 * blocks / 64; }
+RD_HD int out_piece_row(int blocks, int pass, int lane) { return (pass * 64 + lane) / (8 * blocks); }
+RD_HD int out_piece_dim(int first, int blocks, int pass, int lane) { return 32 * first + 4 * ((pass * 64 + lane) % (8 * blocks)); }
+RD_HD int lds_out_piece(int wave, int row, int dim) { return wave * kOutWaveBytes + row * kOutRowBytes + dim * 2; }
+
 // ---- query rows, outputs, mask words ---------------------------------------------------------
 RD_HD int q_row_of(int q_tile, int rows_per_workgroup, int row_block, int r) { return q_tile * rows_per_workgroup + row_block * 32 + r; }
 // element offset of Q fragment ks of lane (r, g) from the first row of the batch row
@@ -156,6 +177,10 @@ RD_HD int64_t q_frag_offset(int h, int64_t q_sh, int q_row, int64_t q_ss, int g,
 // element offset of the four outputs (block db, group i4) of lane (r, g): d = 32*db + 8*i4 + 4*g ..
 RD_HD int64_t out_offset(int h, int64_t o_sh, int q_row, int64_t o_ss, int g, int db, int i4) {
   return (int64_t)h * o_sh + (int64_t)q_row * o_ss + 4 * g + 32 * db + 8 * i4;
+}
+// element offset of dim `dim` of a query row
+RD_HD int64_t out_row_offset(int h, int64_t o_sh, int q_row, int64_t o_ss, int dim) {
+  return (int64_t)h * o_sh + (int64_t)q_row * o_ss + dim;
 }
 RD_HD int64_t mask_word_index(int b, int n_q, int q_row, int words, int key0) {
   return ((int64_t)b * n_q + q_row) * words + (key0 >> 6);

@@ -86,6 +86,15 @@ __device__ inline RowSpan row_span(const AttnArgs& a, int b) {
   return {n < a.n_q ? n : a.n_q, (int64_t)r0 * a.q_ss, (int64_t)r0 * a.o_ss, r0};
 }
 
+// the same from `wide`, which holds entry min(lane, batch) of row_start in every lane (batch < 64:
+// every entry is in some lane; otherwise the two entries are loaded)
+__device__ inline RowSpan row_span(const AttnArgs& a, int b, int wide) {
+  if (a.row_start == nullptr || a.B >= 64) return row_span(a, b);
+  const int r0 = __builtin_amdgcn_readlane(wide, b), r1 = __builtin_amdgcn_readlane(wide, b + 1);
+  const int n = r1 - r0;
+  return {n < a.n_q ? n : a.n_q, (int64_t)r0 * a.q_ss, (int64_t)r0 * a.o_ss, r0};
+}
+
 // round to bf16 and back; products and sums of the rotation are rounded one by one, as the separate
 // elementwise kernels of the reference's op chain round them (no fused multiply-add)
 __device__ inline float bf16_round(float v) { return static_cast<float>(static_cast<__bf16>(v)); }
@@ -139,6 +148,13 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const int item = blockIdx.y;
   const int32_t* it = a.plan + RD_PLAN_HDR + 4 * a.B + RD_ITEM_INTS * item;
   const int n_items = a.plan[0];
+  // Packed query rows: which rows belong to the item's batch row is an entry of row_start that could
+  // only be asked for once the item is here -- one more trip to memory on the way to everything
+  // else.  The lanes ask for all entries now (entry min(lane, batch); of the plan, which is at least
+  // as long, where the rows are not packed: a load that always happens), and the item's two are
+  // picked from them once it is known.
+  const int wide_i = (int)(threadIdx.x & 63) < a.B ? (int)(threadIdx.x & 63) : a.B;
+  const int wide = (a.row_start != nullptr ? a.row_start : a.plan)[wide_i];
   int b = it[0], lo = it[1], hi = it[2], split = it[3];
   int kv_shift = it[4];   // key column c of this row is cache row c - kv_shift
   int key_min = it[5];    // the keys some query of the row attends to lie in [key_min, key_end):
@@ -218,16 +234,46 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   };
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1 % kRing>;
-  // The first tiles are requested as soon as the work item is known: they need nothing but the
-  // item (everything else on the way to the first product -- the row's query rows, Q, the mask
-  // words -- hangs on one more trip to memory, which these loads no longer wait for).
-  if constexpr (!ROPE) {
-    fetch_tile(S0{}, 0);
-    if (k_loader) fetch_tile(S1{}, 1);
-  }
-  const RowSpan rows = row_span(a, b);
-  if (q_tile * kRowsPerWG >= rows.n) return;  // (every thread of the workgroup: no barrier is skipped)
+  // What can be asked for with nothing but the work item is asked for now: a trip to memory takes
+  // more than a microsecond at the start of a launch, and everything on the way to the first product
+  // would otherwise queue up behind the item, the row's query rows and, with the rotation, the
+  // positions and the table rows they select, one trip each.  First the positions (of the lane's
+  // query row and of the new tokens whose keys this thread will rotate: eight bytes each, their
+  // index clamped to the array instead of to the row's query count, which is not here yet), then
+  // the first tiles.  Loads return in the order of their issue: the positions are back after one
+  // trip, and the loads that depend on them go out while the tiles are still coming in.
   const int q_row = q_row_of(q_tile, kRowsPerWG, row_wave, r);
+  // (ROPE) K tile j is requested in step j - 2 - kRing (the prologue for j < 2 + kRing), V tiles
+  // later: t_first is the step whose barrier the new rows must have reached the cache by.  Where
+  // that is the prologue itself (a short cache: its own tiles hold new rows), the rows are written
+  // first, at the price of the trips saved here.
+  const int first_new_tile = a.new_col0 > lo ? (a.new_col0 - lo) / kTile : 0;
+  const int t_first = first_new_tile - 3 - kRing;
+  const bool rows_first = ROPE && t_first < 0;  // (uniform over the workgroup)
+  const int t_lo = new_rows_of_item(lo, hi, key_end, a.new_col0, 0).t_lo;  // (does not depend on the row's query count)
+  int64_t q_pos = 0, pos_a[2] = {0, 0}, pos_b[2] = {0, 0};
+  auto ask_positions = [&](int64_t (&pos)[2], int round) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int t = rope_k_token(t_lo + kNewRowsPerRound * round, tid, i);
+      pos[i] = a.position_ids[(int64_t)b * a.pos_sb + (t < a.n_q ? t : a.n_q - 1)];
+    }
+  };
+  if constexpr (ROPE) {
+    q_pos = a.position_ids[(int64_t)b * a.pos_sb + (q_row < a.n_q ? q_row : a.n_q - 1)];
+    ask_positions(pos_a, 0);
+    ask_positions(pos_b, 1);  // (at most 256 new tokens: two rounds)
+  }
+  // Every thread issues the same eight loads here, on every path: the K loaders tiles 0 and 1, the V
+  // loaders tile 0 twice (the second request rides on the first one's cache lines; the ring refills
+  // that slot before anything reads it), and a workgroup that has to write new rows first asks too
+  // and asks again later.  With a different number of loads on some path, every wait for an older
+  // load below (the row's query rows, the positions) would have to be a wait for the path with the
+  // fewest -- that is, for some or all of these tiles.
+  fetch_tile(S0{}, 0);
+  fetch_tile(S1{}, k_loader ? 1 : 0);
+  const RowSpan rows = row_span(a, b, wide);
+  if (q_tile * kRowsPerWG >= rows.n) return;  // (every thread of the workgroup: no barrier is skipped)
   const bool wave_active = q_tile * kRowsPerWG + row_wave * 32 < rows.n;
   const bool row_valid = q_row < rows.n;
 
@@ -242,21 +288,19 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // A round covers 128 tokens: 1024 rotation tasks (a 16-byte chunk of the first half of a key and
   // its partner in the second half), two per thread, and 2048 copy tasks, four per thread.
   //
-  // Order.  Loads return in the order of their issue, and the tile loads of the prologue keep the
-  // memory system busy for microseconds: whatever this code reads is therefore requested BEFORE
-  // the first tile (`issue`: positions, then the table rows and the new keys and values), and used
-  // (`finish`) after the last tile load of the prologue has been issued.  The stores are not waited
-  // for there either: the first tile that holds new rows is requested many steps into the loop,
-  // and the step before that request waits for them (t_sync), ahead of its barrier.
+  // Order.  The first round's operands (the new keys and values, the table rows of their positions)
+  // are requested once the row's query rows are known, behind the first tiles, and used after those
+  // have been staged; a second round's (more than 128 tokens) go out then and are used under cover of
+  // the ring's first loads.  The stores are not waited for in the prologue: the first tile that holds
+  // new rows is requested many steps into the loop, and the step before that request waits for them
+  // (t_sync), ahead of its barrier.
   const NewRows mine = new_rows_of_item(lo, hi, key_end, a.new_col0, rows.n);  // (uniform over the workgroup)
-  const int t_lo = mine.t_lo, t_hi = ROPE ? mine.t_hi : 0;
+  const int t_hi = ROPE ? mine.t_hi : 0;
   const bool has_new = t_lo < t_hi;
-  // K tile j is requested in step j - 2 - kRing (the prologue for j < 2 + kRing), V tiles later
-  const int first_new_tile = a.new_col0 > lo ? (a.new_col0 - lo) / kTile : 0;
-  const int t_sync = has_new ? first_new_tile - 3 - kRing : -1;  // the step whose barrier the rows need
-  const bool early = has_new && t_sync < 0;  // the prologue's own tiles hold new rows: write first
+  const bool second_round = t_lo + kNewRowsPerRound < t_hi;
+  const int t_sync = has_new && !rows_first ? t_first : -1;  // the step whose barrier the rows need
   struct NewRows {
-    int64_t pos[2]; bf16x8 x1[2], x2[2], vv[4], c1[2], c2[2], s1[2], s2[2];
+    bf16x8 x1[2], x2[2], vv[4], c1[2], c2[2], s1[2], s2[2];
     int kt[2], kc[2], vt[4], vc[4];  // token and chunk of every task; token -1: no task
   } nr;
   const __bf16* kn = nullptr; const __bf16* vn = nullptr;
@@ -270,7 +314,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     pos = pos < 0 ? 0 : (pos >= a.table_rows ? a.table_rows - 1 : pos);  // never read outside the table
     return reinterpret_cast<const __bf16*>(table) + pos * kD;
   };
-  auto new_rows_issue = [&](int round) __attribute__((always_inline)) {
+  auto new_rows_issue = [&](int round, const int64_t (&pos)[2]) __attribute__((always_inline)) {
     // every load reads a token that exists (the round's first one stands in where a thread has no
     // task): the loads are then unconditional and the compiler keeps them together
     const int t0 = t_lo + kNewRowsPerRound * round;
@@ -281,7 +325,6 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       nr.kt[i] = on ? t : -1;
       nr.kc[i] = rope_k_chunk(tid, i);
       const int tl = on ? t : t0;
-      nr.pos[i] = a.position_ids[(int64_t)b * a.pos_sb + tl];
       nr.x1[i] = *reinterpret_cast<const bf16x8*>(kn + (int64_t)tl * a.kn_st + 8 * nr.kc[i]);
       nr.x2[i] = *reinterpret_cast<const bf16x8*>(kn + (int64_t)tl * a.kn_st + kD / 2 + 8 * nr.kc[i]);
     }
@@ -295,8 +338,9 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const __bf16* cos_row = table_row(a.cos, nr.pos[i]) + 8 * nr.kc[i];
-      const __bf16* sin_row = table_row(a.sin, nr.pos[i]) + 8 * nr.kc[i];
+      // (the position of the thread's own token, or of the array's last one where it has no task)
+      const __bf16* cos_row = table_row(a.cos, pos[i]) + 8 * nr.kc[i];
+      const __bf16* sin_row = table_row(a.sin, pos[i]) + 8 * nr.kc[i];
       nr.c1[i] = *reinterpret_cast<const bf16x8*>(cos_row); nr.c2[i] = *reinterpret_cast<const bf16x8*>(cos_row + kD / 2);
       nr.s1[i] = *reinterpret_cast<const bf16x8*>(sin_row); nr.s2[i] = *reinterpret_cast<const bf16x8*>(sin_row + kD / 2);
     }
@@ -323,15 +367,6 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
       }
     }
   };
-  // the rest of the work after the first round's loads: its second half and further rounds (more
-  // than 128 tokens, rare); the rows are in memory after new_rows_wait
-  auto new_rows_complete = [&]() __attribute__((always_inline)) {
-    new_rows_finish();
-    for (int round = 1; t_lo + kNewRowsPerRound * round < t_hi; ++round) {
-      new_rows_issue(round);
-      new_rows_finish();
-    }
-  };
   auto new_rows_wait = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
   // Q fragments: B operand of S^T = K Q^T; lane (r,g) holds Q[q_row][16*ks + 8*g .. +8)
@@ -339,29 +374,38 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // (ROPE) the table rows of the query's position: the lane holds dims 16*ks + 8*g + e, so the
   // partner of a first-half dim (ks < 4) sits in fragment ks + 4 of the same lane
   bf16x8 qc[8], qs[8];
+  if constexpr (ROPE) {
+    if (rows_first) {
+      // a short cache: the new rows first, all of them, and a barrier before anybody's tile load
+      if (has_new) {
+        new_rows_issue(0, pos_a);
+        new_rows_finish();
+        if (second_round) {
+          new_rows_issue(1, pos_b);
+          new_rows_finish();
+        }
+      }
+      new_rows_wait();
+      __syncthreads();
+      fetch_tile(S0{}, 0);
+      fetch_tile(S1{}, k_loader ? 1 : 0);
+    }
+  }
   {
     const __bf16* qp = reinterpret_cast<const __bf16*>(a.q) + rows.q_off +
                        q_frag_offset(h, a.q_sh, row_valid ? q_row : 0, a.q_ss, g, 0);
-    int64_t q_pos = 0;
-    if constexpr (ROPE) q_pos = a.position_ids[(int64_t)b * a.pos_sb + (row_valid ? q_row : 0)];
+    // (a lane whose row does not exist takes the batch row's first one: its results are never used,
+    // and a load that always happens is one the compiler can keep in flight)
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-      qf[ks] = row_valid ? *reinterpret_cast<const bf16x8*>(qp + 16 * ks) : z;
-    }
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
     if constexpr (ROPE) {
-      if (has_new) new_rows_issue(0);
+      if (has_new && !rows_first) new_rows_issue(0, pos_a);
       const __bf16* cos_row = table_row(a.cos, q_pos) + 8 * g;
       const __bf16* sin_row = table_row(a.sin, q_pos) + 8 * g;
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
         qc[ks] = *reinterpret_cast<const bf16x8*>(cos_row + 16 * ks);
         qs[ks] = *reinterpret_cast<const bf16x8*>(sin_row + 16 * ks);
-      }
-      if (early) {
-        new_rows_complete();
-        new_rows_wait();
-        __syncthreads();
       }
     }
   }
@@ -429,25 +473,16 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // the tile that step t stages in ring slot (t + 1) % kRing, so that one piece of code, with
   // the same registers, serves both.
   const int ahead = k_loader ? 2 : 1;
-  if constexpr (!ROPE) {
-    if (k_loader) {  // (requested at the kernel's entry)
-      stage_k(S0{}, 0);
-      stage_k(S1{}, 1);
-    } else {
-      stage_v(S0{}, 0);
-    }
+  if (k_loader) {  // (requested at the kernel's entry)
+    stage_k(S0{}, 0);
+    stage_k(S1{}, 1);
   } else {
-    // the first tiles are requested, and while they are on their way the vector ALU rotates the
-    // queries and the new keys (whose operands were requested before the tiles and arrive first)
-    fetch_tile(S0{}, 0);
-    if (k_loader) fetch_tile(S1{}, 1);
-    if (has_new && !early) new_rows_complete();
-    rotate_q();
-    if (k_loader) {
-      stage_k(S0{}, 0);
-      stage_k(S1{}, 1);
-    } else {
-      stage_v(S0{}, 0);
+    stage_v(S0{}, 0);
+  }
+  if constexpr (ROPE) {
+    if (has_new && !rows_first) {
+      new_rows_finish();
+      if (second_round) new_rows_issue(1, pos_b);
     }
   }
   // The ring is filled in the order in which the steps refill it (mask word, then tile, slot by
@@ -460,6 +495,11 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     fetch_word(std::integral_constant<int, J>{}, J);
     fetch_tile(std::integral_constant<int, (J + 1) % kRing>{}, ahead + J);
   });
+  if constexpr (ROPE) {
+    // under cover of the ring's first loads: the queries are rotated, a second round of new rows finished
+    rotate_q();
+    if (has_new && !rows_first && second_round) new_rows_finish();
+  }
   __syncthreads();
   // The scores of a unit are masked, and their row maximum taken, as soon as they exist: in the
   // step before the one that turns them into probabilities, under that step's second product
@@ -730,21 +770,48 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
     else { body(B2{}); body(B3{}); }                                     \
   } while (0)
   if (n_splits == 1) {
-    if (!writer) return;
+    // The rows leave through LDS (attn_addr.h: lds_out_stage): in the accumulators a lane holds
+    // four dims of one row, and stored from there an instruction would touch 32 rows with 16 bytes
+    // each -- 32 requests to the L2 where, read back along the rows, two or four whole rows go out.
+    // Each wave uses a region of its own and needs no barrier for it (the tile buffers are free:
+    // every wave has passed the loop's last barrier; where accumulators were merged through LDS, the
+    // merge buffers must have been read first).
+    if constexpr (kHasHalf) __syncthreads();
+    if (!wave_active) return;  // (wave-uniform)
     const bool live = l > 0.f;
     const float inv = live ? 1.f / l : 0.f;
-    __bf16* op = reinterpret_cast<__bf16*>(a.out) + rows.o_off + out_offset(h, a.o_sh, q_row, a.o_ss, g, 0, 0);
-    auto store_block = [&](auto db_c) __attribute__((always_inline)) {
+    char* const mine = smem + lds_out_stage(wave, r, g, 0, 0);
+    auto stage_block = [&](auto db_c) __attribute__((always_inline)) {
       constexpr int db = decltype(db_c)::value;
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         // (a row without any attended key gets zeros, whatever its accumulators picked up)
         bf16x4 w = {static_cast<__bf16>(live ? o[db][4 * i4 + 0] * inv : 0.f), static_cast<__bf16>(live ? o[db][4 * i4 + 1] * inv : 0.f),
                     static_cast<__bf16>(live ? o[db][4 * i4 + 2] * inv : 0.f), static_cast<__bf16>(live ? o[db][4 * i4 + 3] * inv : 0.f)};
-        *reinterpret_cast<bf16x4*>(op + (out_offset(0, 0, 0, 0, 0, db, i4))) = w;
+        *reinterpret_cast<bf16x4*>(mine + lds_out_stage(0, 0, 0, db, i4)) = w;
       }
     };
-    RD_FOR_KEPT_BLOCKS(store_block);
+    RD_FOR_KEPT_BLOCKS(stage_block);
+    // (the wave reads what its own lanes wrote: its LDS instructions execute in program order)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __bf16* const orow = reinterpret_cast<__bf16*>(a.out) + rows.o_off;
+    auto store_rows = [&](auto first_c, auto blocks_c) __attribute__((always_inline)) {
+      constexpr int kFirst = decltype(first_c)::value, kBlocks = decltype(blocks_c)::value;
+#pragma unroll
+      for (int pass = 0; pass < out_passes(kBlocks); ++pass) {
+        const int row = out_piece_row(kBlocks, pass, lane), dim = out_piece_dim(kFirst, kBlocks, pass, lane);
+        const bf16x4 w = *reinterpret_cast<const bf16x4*>(smem + lds_out_piece(wave, row, dim));
+        const int q = q_row_of(q_tile, kRowsPerWG, row_wave, row);
+        if (q < rows.n) *reinterpret_cast<bf16x4*>(orow + out_row_offset(h, a.o_sh, q, a.o_ss, dim)) = w;
+      }
+    };
+    using Two = std::integral_constant<int, 2>;
+    using Four = std::integral_constant<int, 4>;
+    if (full || !kHasHalf) store_rows(B0{}, Four{});
+    else if (kp == 0) store_rows(B0{}, Two{});
+    else store_rows(B2{}, Two{});
     return;
   }
   // The keys of this batch row are split over n_splits work items: each leaves (m, l, O) of its

@@ -144,6 +144,49 @@ void check_lds(Failure& f) {
           CHECK(off >= lds_merge_o(kWaves / 2 - 1, 63, 63) + 4 && off + 4 <= kLdsBytes && off + 4 <= kMergeFloats * 4, "merge (m, l) offset %d", off);
         }
     }
+  // Results through LDS: every wave puts the accumulator blocks it keeps into its own region (tagged
+  // here row * 128 + dim) and reads them back along the rows; every piece it reads must hold the
+  // four dims the store then writes, and no two waves may share a byte.
+  for (int layout = kSplit; layout <= kFull; ++layout) {
+    std::vector<int> tag(kLdsBytes / 2, -1), owner(kLdsBytes / 2, -1);
+    for (int w = 0; w < kWaves; ++w) {
+      const WaveRole role = wave_role(layout, w);
+      const int first = first_block_kept(role.part), blocks = blocks_kept(role.part);
+      for (int lane = 0; lane < 64; ++lane) {
+        const int r = lane & 31, g = lane >> 5;
+        for (int db = first; db < first + blocks; ++db)
+          for (int i4 = 0; i4 < 4; ++i4) {
+            const int off = lds_out_stage(w, r, g, db, i4);
+            CHECK(off >= 0 && off + 8 <= kLdsBytes && off % 8 == 0, "output stage offset %d (layout %d wave %d lane %d)", off, layout, w, lane);
+            for (int x = 0; x < 4; ++x) {
+              CHECK(tag[off / 2 + x] == -1, "output stage writes overlap at byte %d (layout %d wave %d)", off + 2 * x, layout, w);
+              tag[off / 2 + x] = r * kD + 32 * db + 8 * i4 + 4 * g + x;  // accumulator 4*i4 + x of block db
+              owner[off / 2 + x] = w;
+            }
+          }
+      }
+    }
+    for (int w = 0; w < kWaves; ++w) {
+      const WaveRole role = wave_role(layout, w);
+      const int first = first_block_kept(role.part), blocks = blocks_kept(role.part);
+      std::vector<int> seen(32 * kD, 0);
+      CHECK(out_passes(blocks) * 64 == 32 * 8 * blocks, "output passes of a wave that keeps %d blocks", blocks);
+      for (int pass = 0; pass < out_passes(blocks); ++pass)
+        for (int lane = 0; lane < 64; ++lane) {
+          const int row = out_piece_row(blocks, pass, lane), dim = out_piece_dim(first, blocks, pass, lane);
+          CHECK(row >= 0 && row < 32 && dim >= 32 * first && dim + 4 <= 32 * (first + blocks) && dim % 4 == 0, "output piece (row %d, dim %d) of pass %d lane %d", row, dim, pass, lane);
+          const int off = lds_out_piece(w, row, dim);
+          CHECK(off >= 0 && off + 8 <= kLdsBytes && off % 8 == 0, "output piece offset %d", off);
+          for (int x = 0; x < 4; ++x) {
+            CHECK(owner[off / 2 + x] == w && tag[off / 2 + x] == row * kD + dim + x, "layout %d wave %d reads (row %d, dim %d) and finds %d of wave %d", layout, w, row, dim + x, tag[off / 2 + x], owner[off / 2 + x]);
+            seen[row * kD + dim + x]++;
+          }
+        }
+      for (int row = 0; row < 32; ++row)
+        for (int d = 0; d < kD; ++d)
+          CHECK(seen[row * kD + d] == (d >= 32 * first && d < 32 * (first + blocks) ? 1 : 0), "layout %d wave %d: (row %d, dim %d) goes out %d times", layout, w, row, d, seen[row * kD + d]);
+    }
+  }
   // the two waves of a pair hand over disjoint accumulator blocks and keep the other two: every
   // block of the head dimension is kept by exactly one of them
   for (int part = 0; part < 2; ++part) {
@@ -189,6 +232,8 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
   const size_t part_o_bytes = align_up((size_t)slots * L.n_q * kD * sizeof(float), 256);
   const size_t part_ml_bytes = align_up((size_t)slots * L.n_q * 2 * sizeof(float), 256);
   const size_t plan_ints = rd::attn_plan_ints(L.B, L.n_q, L.kv_len);
+  // every lane reads entry min(lane, B) of row_start, or of the plan where the rows are not packed
+  CHECK(plan_ints >= (size_t)(L.B < 63 ? L.B : 63) + 1, "the plan is shorter than the %d entries read in place of row_start", (L.B < 63 ? L.B : 63) + 1);
   CHECK((int)items.size() <= L.B * max_splits, "chunk %d: %zu items, the plan holds %d", chunk, items.size(), L.B * max_splits);
   CHECK(RD_PLAN_HDR + 4 * (size_t)L.B + RD_ITEM_INTS * (size_t)L.B * max_splits <= plan_ints, "item slots beyond the plan");
   CHECK(q_tiles <= rd::attn_max_q_tiles(L.n_q) || L.n_q <= 256, "query tiles %d beyond the counters' %d", q_tiles, rd::attn_max_q_tiles(L.n_q));
@@ -219,6 +264,7 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
         ++st.workgroups;
         const int64_t cidx = counter_index(b, L.H, h, q_tiles, q_tile);
         CHECK(cidx >= 0 && (size_t)cidx < rd::attn_counter_ints(L.B, L.H, L.n_q), "counter index %lld of %zu", (long long)cidx, rd::attn_counter_ints(L.B, L.H, L.n_q));
+        std::vector<int> covered((size_t)rows_wg * (kD / 4), 0);  // pieces of four dims of the tile's rows
         for (int tid = 0; tid < kThreads; ++tid) {
           const int wave = tid >> 6, lane = tid & 63, g = lane >> 5, r = lane & 31;
           const WaveRole role = wave_role(layout, wave);
@@ -227,8 +273,7 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
           const bool wave_active = q_tile * rows_wg + role.block * 32 < rows_n;
           // Q fragments and mask words (rows past the count read row 0 of the batch row)
           const int q_use = row_valid ? q_row : 0;
-          if (row_valid)
-            for (int ks = 0; ks < 8; ++ks) {
+          for (int ks = 0; ks < 8; ++ks) {
               const int64_t off = q_off + q_frag_offset(h, L.q_sh, q_use, L.q_ss, g, ks);
               CHECK(off >= 0 && off + 8 <= L.q_elems, "Q element %lld of %lld (row %d head %d query %d)", (long long)off, (long long)L.q_elems, b, h, q_row);
               ++st.q_loads;
@@ -250,15 +295,23 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
               ++st.tile_loads;
             }
           }
-          // results
-          const bool writer = wave_active && row_valid;  // every wave stores the accumulator blocks it keeps
+          // results.  A row with all its keys in one item: every active wave sends out the rows of its
+          // block along the rows, whatever rows its lanes computed
+          if (it.n_splits == 1 && wave_active) {
+            const int first = first_block_kept(role.part), blocks = blocks_kept(role.part);
+            for (int pass = 0; pass < out_passes(blocks); ++pass) {
+              const int row = out_piece_row(blocks, pass, lane), dim = out_piece_dim(first, blocks, pass, lane);
+              const int q = q_row_of(q_tile, rows_wg, role.block, row);
+              if (q >= rows_n) continue;
+              const int64_t off = o_off + out_row_offset(h, L.o_sh, q, L.o_ss, dim);
+              CHECK(off >= 0 && off + 4 <= L.o_elems, "output element %lld of %lld (row %d head %d query %d)", (long long)off, (long long)L.o_elems, b, h, q);
+              CHECK(q >= q_tile * rows_wg && q < (q_tile + 1) * rows_wg, "query %d outside tile %d", q, q_tile);
+              covered[(size_t)(q - q_tile * rows_wg) * (kD / 4) + dim / 4]++;
+              ++st.stores;
+            }
+          }
+          const bool writer = wave_active && row_valid;  // split rows: every wave leaves the accumulator blocks it keeps as partials
           if (writer) {
-            for (int db = first_block_kept(role.part); db < first_block_kept(role.part) + blocks_kept(role.part); ++db)
-              for (int i4 = 0; i4 < 4; ++i4) {
-                const int64_t off = o_off + out_offset(h, L.o_sh, q_row, L.o_ss, g, db, i4);
-                CHECK(off >= 0 && off + 4 <= L.o_elems, "output element %lld of %lld (row %d head %d query %d)", (long long)off, (long long)L.o_elems, b, h, q_row);
-                ++st.stores;
-              }
             if (it.n_splits > 1) {
               const int64_t row = partial_row(b, L.H, h, max_splits, it.split, L.n_q, q_row);
               CHECK(row >= 0 && row < slots * L.n_q, "partial row %lld of %lld", (long long)row, slots * L.n_q);
@@ -284,6 +337,20 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
                   }
                 }
           }
+          // the positions are asked for before the row's query count is known, by every thread: of
+          // its query row and of the tokens of two rounds of new rows, clamped to the array
+          if (L.rope) {
+            CHECK(nr.t_lo == new_rows_of_item(lo, hi, key_end, L.kv_len - L.n_q, 0).t_lo, "the first new token depends on the row count");
+            CHECK(nr.t_hi - nr.t_lo <= 2 * kNewRowsPerRound, "%d new tokens in one item: more than two rounds", nr.t_hi - nr.t_lo);
+            const int64_t qp = (int64_t)b * L.pos_sb + (q_row < L.n_q ? q_row : L.n_q - 1);
+            CHECK(qp >= 0 && qp < L.pos_elems, "position id %lld of %lld (query row %d)", (long long)qp, (long long)L.pos_elems, q_row);
+            for (int round = 0; round < 2; ++round)
+              for (int i = 0; i < 2; ++i) {
+                const int t = rope_k_token(nr.t_lo + kNewRowsPerRound * round, tid, i);
+                const int64_t pos = (int64_t)b * L.pos_sb + (t < L.n_q ? t : L.n_q - 1);
+                CHECK(t >= 0 && pos >= 0 && pos < L.pos_elems, "position id %lld of %lld (token %d)", (long long)pos, (long long)L.pos_elems, t);
+              }
+          }
           // new cache rows of the fused rotation
           if (L.rope && nr.t_lo < nr.t_hi) {
             const int new_col0 = L.kv_len - L.n_q;
@@ -297,8 +364,6 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
                 const bool on = t < nr.t_hi && new_row_in_slab(new_col0, t, kv_shift, L.max_len);
                 const int tl = on ? t : t0;  // (a thread without a task reads the round's first token)
                 CHECK(tl >= 0 && tl < rows_n, "new token %d of %d (row %d)", tl, rows_n, b);
-                const int64_t pos = (int64_t)b * L.pos_sb + tl;
-                CHECK(pos >= 0 && pos < L.pos_elems, "position id %lld of %lld", (long long)pos, (long long)L.pos_elems);
                 const int64_t src = new_off + (int64_t)hk * kD + (int64_t)tl * L.kn_st + 8 * c + (is_k ? kD / 2 : 0);
                 CHECK(src >= 0 && src + 8 <= L.kn_elems, "new key/value element %lld of %lld", (long long)src, (long long)L.kn_elems);
                 if (on) {
@@ -312,6 +377,13 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
             }
           }
         }
+        // a row that is not split goes out whole, every piece once, and no row past the count
+        if (it.n_splits == 1)
+          for (int row = 0; row < rows_wg; ++row)
+            for (int piece = 0; piece < kD / 4; ++piece) {
+              const int want = q_tile * rows_wg + row < rows_n ? 1 : 0;
+              CHECK(covered[(size_t)row * (kD / 4) + piece] == want, "row %d head %d query %d dims %d..: stored %d times", b, h, q_tile * rows_wg + row, 4 * piece, covered[(size_t)row * (kD / 4) + piece]);
+            }
       }
     }
   }
