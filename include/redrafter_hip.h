@@ -44,7 +44,7 @@ typedef enum { RD_BF16 = 0, RD_F16 = 1, RD_F32 = 2 } rd_dtype;
  * that crosses it (the attention plan, the realignment plan) or a workspace size changes.  A caller
  * compiled against this header compares rd_version() with RD_ABI_VERSION before its first call, so
  * that a stale build of the library is refused instead of being called with other arguments. */
-#define RD_ABI_VERSION 105
+#define RD_ABI_VERSION 106
 RD_API int rd_version(void);
 /* Message of the last failed call on this thread ("" if none). */
 RD_API const char* rd_last_error(void);
@@ -427,6 +427,19 @@ RD_API int rd_beam_topk(const void* logits, int dtype, int64_t row_stride, int64
                         int64_t* parents, int64_t* beams_out, float* logp_out,
                         int64_t logp_row_stride, void* workspace, size_t workspace_bytes,
                         int force_fallback, void* stream);
+
+/* rd_beam_init: the state a beam search starts from (modeling_drafter.py:170-189), in one launch
+ * where the reference runs a fill, a slice assignment, two broadcasts and a zeros: log_p_beam
+ * (batch, width) float32 = 0 for beam 0 and mask_value for the others; beams (batch, width) int64 =
+ * the row's init token; head_in[b, w, 0 : hidden_bytes) = prompt_state[b] (the context half of the
+ * [context, state] input of the head, modeling_drafter.py:199; rows head_in_row_bytes apart, the
+ * state half is left alone); state (batch, state_rows, hidden_bytes), state_rows <= width: zeros.
+ * Bytes are copied as they are, whatever the dtype; rows and strides are multiples of 16 bytes and
+ * 16-byte aligned. */
+RD_API int rd_beam_init(const void* prompt_state, int64_t ps_row_bytes, const int64_t* init_token,
+                        int batch, int width, int64_t hidden_bytes, float mask_value,
+                        float* log_p_beam, int64_t* beams, void* head_in, int64_t head_in_row_bytes,
+                        void* state, int state_rows, void* stream);
 
 /* rd_beam_topk_static: rd_beam_topk without the workspace argument, for callers that cannot
  * allocate device memory -- code under HIP graph capture, serving loops and harnesses that forbid

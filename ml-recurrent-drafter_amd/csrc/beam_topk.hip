@@ -357,6 +357,57 @@ void* static_scratch(int* error) {
 }
 }  // namespace
 
+namespace {
+
+// One workgroup per (batch row, beam): the row's prompt state into the context half of the head's
+// input, zeros into the recurrent state, the beam's first token and score.
+constexpr int kInitThreads = 256;
+__global__ __launch_bounds__(kInitThreads) void beam_init_kernel(const char* prompt_state, int64_t ps_row_bytes,
+                                                                 const int64_t* init_token, int width, int64_t hidden_bytes,
+                                                                 float mask_value, float* log_p_beam, int64_t* beams,
+                                                                 char* head_in, int64_t head_in_row_bytes, char* state,
+                                                                 int state_rows) {
+  const int w = blockIdx.x, b = blockIdx.y;
+  const int64_t row = (int64_t)b * width + w;
+  const uint4* src = reinterpret_cast<const uint4*>(prompt_state + (int64_t)b * ps_row_bytes);
+  uint4* dst = reinterpret_cast<uint4*>(head_in + row * head_in_row_bytes);
+  const int64_t chunks = hidden_bytes / 16;
+  for (int64_t i = threadIdx.x; i < chunks; i += kInitThreads) dst[i] = src[i];
+  if (w < state_rows) {
+    uint4* z = reinterpret_cast<uint4*>(state + ((int64_t)b * state_rows + w) * hidden_bytes);
+    for (int64_t i = threadIdx.x; i < chunks; i += kInitThreads) z[i] = make_uint4(0u, 0u, 0u, 0u);
+  }
+  if (threadIdx.x == 0) {
+    log_p_beam[row] = w == 0 ? 0.f : mask_value;
+    beams[row] = init_token[b];
+  }
+}
+
+}  // namespace
+
+extern "C" int rd_beam_init(const void* prompt_state, int64_t ps_row_bytes, const int64_t* init_token, int batch,
+                            int width, int64_t hidden_bytes, float mask_value, float* log_p_beam, int64_t* beams,
+                            void* head_in, int64_t head_in_row_bytes, void* state, int state_rows, void* stream) {
+  RD_REQUIRE(batch > 0 && width > 0 && hidden_bytes > 0 && state_rows > 0 && state_rows <= width, RD_EINVAL,
+             "rd_beam_init: bad sizes (batch %d width %d hidden bytes %lld state rows %d)", batch, width,
+             (long long)hidden_bytes, state_rows);
+  RD_REQUIRE(batch <= 65535, RD_ELIMIT, "rd_beam_init: batch %d > 65535", batch);
+  RD_REQUIRE(prompt_state && init_token && log_p_beam && beams && head_in && state, RD_EINVAL, "rd_beam_init: null pointer");
+  auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  RD_REQUIRE(hidden_bytes % 16 == 0 && ps_row_bytes % 16 == 0 && head_in_row_bytes % 16 == 0 && al(prompt_state) &&
+                 al(head_in) && al(state) && ps_row_bytes >= hidden_bytes && head_in_row_bytes >= hidden_bytes,
+             RD_EINVAL, "rd_beam_init: rows must be 16-byte aligned multiples of 16 bytes, strides at least a row");
+  hipStream_t s = rd::as_stream(stream);
+  {
+    rd::ScopedTiming rd_t("beam_init_kernel", s);
+    hipLaunchKernelGGL(beam_init_kernel, dim3(width, batch), dim3(kInitThreads), 0, s,
+                       reinterpret_cast<const char*>(prompt_state), ps_row_bytes, init_token, width, hidden_bytes,
+                       mask_value, log_p_beam, beams, reinterpret_cast<char*>(head_in), head_in_row_bytes,
+                       reinterpret_cast<char*>(state), state_rows);
+  }
+  return rd::check_launch("rd_beam_init");
+}
+
 extern "C" size_t rd_beam_topk_workspace_bytes(int batch, int width) {
   if (batch <= 0 || width <= 0) return 0;
   const size_t n = (size_t)batch * width * width;

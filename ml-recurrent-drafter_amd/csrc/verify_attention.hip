@@ -270,8 +270,12 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // and asks again later.  With a different number of loads on some path, every wait for an older
   // load below (the row's query rows, the positions) would have to be a wait for the path with the
   // fewest -- that is, for some or all of these tiles.
+  // (Without the rotation the only older load is the one for the row's query rows: there the V
+  // loaders skip the second request, and the K loaders' wait for those rows becomes a wait for their
+  // first tile as well -- measured 0.35 us shorter per launch than with the extra requests.)
   fetch_tile(S0{}, 0);
-  fetch_tile(S1{}, k_loader ? 1 : 0);
+  if constexpr (ROPE) fetch_tile(S1{}, k_loader ? 1 : 0);
+  else if (k_loader) fetch_tile(S1{}, 1);
   const RowSpan rows = row_span(a, b, wide);
   if (q_tile * kRowsPerWG >= rows.n) return;  // (every thread of the workgroup: no barrier is skipped)
   const bool wave_active = q_tile * kRowsPerWG + row_wave * 32 < rows.n;

@@ -20,7 +20,7 @@ import sys
 _DEFAULT_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libredrafter_hip.so")
 _LIB_PATH = os.environ.get("RD_HIP_LIBRARY") or _DEFAULT_LIB_PATH
 _lib = None
-ABI_VERSION = 105  # RD_ABI_VERSION of include/redrafter_hip.h that _PROTOTYPES below was written against
+ABI_VERSION = 106  # RD_ABI_VERSION of include/redrafter_hip.h that _PROTOTYPES below was written against
 
 RD_BF16, RD_F16, RD_F32 = 0, 1, 2
 _DTYPES = {torch.bfloat16: RD_BF16, torch.float16: RD_F16, torch.float32: RD_F32}
@@ -87,6 +87,7 @@ _PROTOTYPES = {
         _I,
         [_P, _I, _L, _L, _I, _I, _I, _P, _I, _F, _P, _I, _P, _P, _P, _P, _P, _L, _P, _Z, _I, _P],
     ),
+    "rd_beam_init": (_I, [_P, _L, _P, _I, _I, _L, _F, _P, _P, _P, _L, _P, _I, _P]),
     "rd_beam_topk_static": (
         _I,
         [_P, _I, _L, _L, _I, _I, _I, _P, _I, _F, _P, _I, _P, _P, _P, _P, _P, _L, _I, _P],

@@ -133,6 +133,30 @@ def beam_topk_step(
     return new_lpb, tok_par[0], tok_par[1], new_beams, logp
 
 
+def beam_init(prompt_state: torch.Tensor, init_token: torch.Tensor, width: int, state_rows: int):
+    """The state the beam search starts from (modeling_drafter.py:170-189): log_p_beam (B, W) float32
+    with only beam 0 alive, beams (B, W, 1) holding the init token, the (B, W, 2*hidden) input of the
+    head with its context half filled in, and the zero state of the first `state_rows` beams."""
+    B, hidden = prompt_state.shape
+    dev, dt = prompt_state.device, prompt_state.dtype
+    if prompt_state.stride(1) != 1:
+        prompt_state = prompt_state.contiguous()
+    init_token = init_token.contiguous()
+    log_p_beam = torch.empty((B, width), dtype=torch.float32, device=dev)
+    beams = torch.empty((B, width, 1), dtype=torch.long, device=dev)
+    head_in = torch.empty((B, width, 2 * hidden), dtype=dt, device=dev)
+    state = torch.empty((B, state_rows, hidden), dtype=dt, device=dev)
+    esize = prompt_state.element_size()
+    _hip.check(
+        _hip.lib().rd_beam_init(
+            _hip.ptr(prompt_state), prompt_state.stride(0) * esize, _hip.ptr(init_token), B, width, hidden * esize,
+            LOG_0, _hip.ptr(log_p_beam), _hip.ptr(beams), _hip.ptr(head_in), 2 * hidden * esize, _hip.ptr(state),
+            state_rows, _hip.stream(),
+        )
+    )
+    return log_p_beam, beams, head_in, state
+
+
 class Drafter(transformers.PreTrainedModel):
     config_class = configuration_drafter.DrafterConfig
     # False computes the first beam-search iteration for all W (identical) beams, as upstream does
@@ -192,16 +216,13 @@ class Drafter(transformers.PreTrainedModel):
         V = embeddings.num_embeddings
         dev = prompt_state.device
 
-        # only beam 0 is alive at the start, so the first iteration fans out from it alone
-        log_p_beam = torch.full((B, W), LOG_0, dtype=torch.float32, device=dev)
-        log_p_beam[:, 0] = LOG_1
-        context = prompt_state.unsqueeze(1).expand(B, W, hidden)
-        beams = init_token.view(B, 1, 1).expand(B, W, 1).contiguous()
-        state = torch.zeros(B, W, hidden, device=dev, dtype=prompt_state.dtype)
-        # [context, state], the input of the head (modeling_drafter.py:199): the context half is
-        # written once, the state half by the kernel that forms the state
-        head_in = torch.empty(B, W, 2 * hidden, device=dev, dtype=prompt_state.dtype)
-        head_in[..., :hidden] = context
+        # only beam 0 is alive at the start, so the first iteration fans out from it alone.
+        # [context, state] is the input of the head (modeling_drafter.py:199): the context half is
+        # written once, here, the state half by the kernel that forms the state.  Scores, first
+        # tokens, context halves and the zero state come from one launch.
+        first_rows = 1 if self.first_iteration_once else W  # beams whose state the first iteration reads
+        log_p_beam, beams, head_in, state = beam_init(prompt_state, init_token, W, first_rows)
+        newest = init_token.view(B, 1) if first_rows == 1 else beams[:, :, 0]  # (B, rows of the first iteration)
         step_log_probs: List[torch.Tensor] = []
         step_parents: List[torch.Tensor] = []
 
@@ -210,7 +231,9 @@ class Drafter(transformers.PreTrainedModel):
             # (modeling_drafter.py:170-189), so the W rows of logits are W copies of one row:
             # that row is computed once per batch row and shown W times.
             rows = 1 if it == 0 and self.first_iteration_once else W
-            last = embeddings(beams[:, :rows, -1])
+            # (the newest token of every beam, from a contiguous tensor: beams[:, :rows, -1] is a
+            # strided view, which the lookup would copy first)
+            last = embeddings(newest[:, :rows])
             if self.config.rnn:
                 state = silu_add(self.rnn_w(last), self.rnn_u(state[:, :rows]), mode=1,
                                  also=head_in[:, :rows, hidden:])
@@ -221,7 +244,7 @@ class Drafter(transformers.PreTrainedModel):
             if rows != W:
                 logits = logits.expand(B, W, V)
                 state = state.expand(B, W, hidden)
-            log_p_beam, _, parents, beams, logp = beam_topk_step(
+            log_p_beam, newest, parents, beams, logp = beam_topk_step(
                 logits, log_p_beam, beams, want_log_probs=return_log_probs
             )
             state = _gather_beams(state, parents)

@@ -184,6 +184,38 @@ def _models(seed, dtype):
     return llm.to(dtype).eval(), drafter.to(dtype).eval()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,W,hidden,state_rows", [(1, 1, 8, 1), (3, 7, 40, 1), (8, 45, 4096, 1), (2, 64, 256, 64), (5, 6, 24, 6)])
+def test_beam_init_is_the_reference_initial_state(dtype, B, W, hidden, state_rows):
+    """modeling_drafter.py:170-189 op by op, against the one launch; a strided prompt state and the
+    state half of the head's input untouched."""
+    from recurrent_drafting_amd import modeling_drafter as md
+
+    if hidden * torch.empty((), dtype=dtype).element_size() % 16:
+        pytest.skip("rows must be multiples of 16 bytes")
+    g = torch.Generator().manual_seed(B * 1000 + W)
+    wide = torch.randn(B, 2 * hidden, generator=g).to(dtype).cuda()
+    prompt_state = wide[:, :hidden]  # row stride 2 * hidden
+    init_token = torch.randint(0, 32000, (B,), generator=g).cuda()
+    log_p_beam, beams, head_in, state = md.beam_init(prompt_state, init_token, W, state_rows)
+    want_lpb = torch.full((B, W), md.LOG_0, dtype=torch.float32)
+    want_lpb[:, 0] = md.LOG_1
+    assert torch.equal(log_p_beam.cpu(), want_lpb) and log_p_beam.dtype == torch.float32
+    assert torch.equal(beams.cpu(), init_token.cpu().view(B, 1, 1).expand(B, W, 1)) and beams.dtype == torch.long
+    assert head_in.shape == (B, W, 2 * hidden) and head_in.dtype == dtype
+    assert torch.equal(head_in[..., :hidden].cpu(), prompt_state.cpu().unsqueeze(1).expand(B, W, hidden))
+    assert state.shape == (B, state_rows, hidden) and state.dtype == dtype and not state.cpu().float().abs().any()
+    # what the launch must not touch: the state half of the head's input
+    head_in2 = torch.full((B, W, 2 * hidden), 3.0, dtype=dtype, device="cuda")
+    from recurrent_drafting_amd import _hip
+    e = prompt_state.element_size()
+    _hip.check(_hip.lib().rd_beam_init(_hip.ptr(prompt_state), prompt_state.stride(0) * e, _hip.ptr(init_token), B, W,
+                                       hidden * e, md.LOG_0, _hip.ptr(log_p_beam), _hip.ptr(beams), _hip.ptr(head_in2),
+                                       2 * hidden * e, _hip.ptr(state), state_rows, _hip.stream()))
+    assert torch.equal(head_in2[..., hidden:].cpu(), torch.full((B, W, hidden), 3.0, dtype=dtype))
+    assert torch.equal(head_in2[..., :hidden], head_in[..., :hidden])
+
+
 def test_beam_search_candidates_matches_reference_vectors(ref_vectors):
     """The reference's own beams on tie-free float32 drafters (weights are multiples of 1/64)."""
     import recurrent_drafting_amd as rd

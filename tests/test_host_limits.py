@@ -27,6 +27,18 @@ def test_beam_search_limits(lib):
     assert _beam_topk(lib, batch=0) == EINVAL and b"bad sizes" in lib.rd_last_error()
 
 
+def test_beam_init_limits(lib):
+    def init(batch=8, width=45, hidden_bytes=8192, state_rows=1, stride=None):
+        stride = hidden_bytes if stride is None else stride
+        return lib.rd_beam_init(None, stride, None, batch, width, hidden_bytes, -50000.0, None, None, None, 2 * stride,
+                                None, state_rows, None)
+
+    assert init() == EINVAL and b"null" in lib.rd_last_error()
+    assert init(state_rows=46) == EINVAL and init(state_rows=0) == EINVAL and b"bad sizes" in lib.rd_last_error()
+    assert init(batch=65536) == ELIMIT
+    # (the alignment rules are checked behind the null pointers: covered on the GPU)
+
+
 def test_attention_plan_limits(lib):
     def prepare(batch, n_q=168, kv_len=2716, heads=32):
         return lib.rd_attn_prepare(None, 0, 0, batch, n_q, kv_len, heads, 0, None, None, None, None)
