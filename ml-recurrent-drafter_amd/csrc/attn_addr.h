@@ -86,24 +86,25 @@ RD_HD int n_tiles_of(int lo, int hi) { return (hi - lo + kTile - 1) / kTile; }
 // first key of tile j of an item; tile indices past the end repeat the last tile (the loads of the
 // pipeline's tail are issued like all the others and never used)
 RD_HD int tile_key0(int lo, int j, int n_tiles) { return lo + (j < n_tiles ? j : n_tiles - 1) * kTile; }
-// a tile that leaves the span [key_min, key_end) of the keys somebody attends to
-RD_HD bool tile_leaves_span(int key0, int key_min, int key_end) { return key0 + kTile > key_end || key0 < key_min; }
-// the key whose cache row stands in for `key`: keys in front of the row's first attended key (left
-// padding) re-read that key, keys behind its last attended key (tree slots that do not exist, the
-// end of the cache) re-read that one
-RD_HD int key_in_span(int key, int key_min, int key_end) { return key < key_end ? (key > key_min ? key : key_min) : key_end - 1; }
+// K and V are read through a buffer descriptor that covers exactly the cache rows of the span
+// [key_min, key_end) of keys that some query of the batch row attends to: it begins at the row of
+// key_min and holds span_bytes.  A tile may begin up to 63 keys below the span or end behind it; a
+// lane whose key lies outside gets zeros from the hardware's range check and asks nothing of the
+// memory (the probabilities of those keys are zero, and zero times zero is zero, where zero times
+// whatever lay in the cache could be NaN).
 // key column read by chunk i (0..3) of a loader thread for the tile at key0
-RD_HD int tile_chunk_key(const Loader& ld, int key0, int i, int key_min, int key_end) {
-  const int key = key0 + ld.first_key + i * ld.key_step;
-  return tile_leaves_span(key0, key_min, key_end) ? key_in_span(key, key_min, key_end) : key;
+RD_HD int tile_chunk_key(const Loader& ld, int key0, int i) { return key0 + ld.first_key + i * ld.key_step; }
+RD_HD uint32_t span_bytes(int key_min, int key_end, int64_t row_bytes) { return (uint32_t)((int64_t)(key_end - key_min) * row_bytes); }
+// byte offset of that chunk from the descriptor's base, as the 32-bit number the load instruction
+// takes: below the span it wraps around to the top of the range
+RD_HD uint32_t tile_chunk_offset(const Loader& ld, int key0, int i, int key_min, int64_t row_bytes) {
+  return (uint32_t)((int64_t)(tile_chunk_key(ld, key0, i) - key_min) * row_bytes + 16 * ld.chunk);
 }
-
-// L2 touch: beyond the tiles that travel in the register ring, every loader thread reads four bytes
-// of a tile further ahead, so that the line is on its way into the L2 long before the ring asks for
-// it (256 threads, the 128 lines of a tile's 64 rows of 256 bytes: two threads per line).
-RD_HD int touch_row(int tid) { return (tid & 255) >> 2; }
-RD_HD int touch_byte(int tid) { return ((tid >> 1) & 1) * 128; }
-RD_HD int touch_key(int tid, int key0, int key_min, int key_end) { return key_in_span(key0 + touch_row(tid), key_min, key_end); }
+// the range check of a 16-byte load (no swizzle, no stride in the descriptor)
+RD_HD bool chunk_in_range(uint32_t offset, uint32_t records) { return (uint64_t)offset + 16 <= records; }
+// what the host checks before a launch: every span fits the 32-bit offsets with room for the
+// wrap-around of the 63 rows below it
+RD_HD bool span_fits(int64_t kv_len, int64_t row_bytes) { return (kv_len + 2 * kTile) * row_bytes < ((int64_t)1 << 31); }
 
 // ---- LDS -------------------------------------------------------------------------------------
 // byte offsets from the start of the workgroup's LDS; K buffers first, then the V buffers

@@ -201,33 +201,31 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   const char* base = reinterpret_cast<const char*>(k_loader ? kbase : vbase);
   const int64_t row_bytes = (k_loader ? a.k_ss : a.v_ss) * 2;
   const int key_step = ld.key_step, first_key = ld.first_key;  // this thread's keys within a tile: first_key + i * key_step
-  const uint32_t lane_off = (uint32_t)(first_key * row_bytes + 16 * chunk);
+  // K and V come through a buffer descriptor over the cache rows of the keys that some query of the
+  // row attends to (attn_addr.h: tile_chunk_offset): every step issues the same four loads whatever
+  // the tile, and the lanes whose key lies outside that span -- left padding in front of it, tree
+  // slots that do not exist and the end of the cache behind it -- get zeros without touching memory.
+  // Non-temporal: every K and V row is read once per launch (twice when two query tiles or grouped
+  // heads share it, back to back), so it should not push the L2's other lines out on its way
+  // through.  In the decode step this alone takes the launch from 28.8 to 27.3 us at 600 keys per
+  // row and from 85 to 70 us at 2500.
+  const __amdgpu_buffer_rsrc_t tiles = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(base) + (int64_t)key_min * row_bytes, 0, (int)span_bytes(key_min, key_end, row_bytes), 0x00020000);
+  const uint32_t lane_off = tile_chunk_offset(ld, 0, 0, 0, row_bytes);  // the thread's place in a tile
+  const uint32_t step_bytes = (uint32_t)(key_step * row_bytes);
+  constexpr int kNonTemporal = 2;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   auto fetch_into = [&](bf16x8& c0, bf16x8& c1, bf16x8& c2, bf16x8& c3, int j) __attribute__((always_inline)) {
     const int key0 = tile_key0(lo, j, n_tiles);
-    const char* tile = base + (int64_t)key0 * row_bytes;
-    const int64_t step_bytes = key_step * row_bytes;
-    // chunk i reads key column tile_chunk_key(ld, key0, i, key_min, key_end): inside the span that
-    // is key0 + first_key + i * key_step ...
-    int64_t o0 = lane_off, o1 = step_bytes + lane_off, o2 = 2 * step_bytes + lane_off, o3 = 3 * step_bytes + lane_off;
-    if (tile_leaves_span(key0, key_min, key_end)) {
-      // the first and the last tile of a row: keys in front of the row's first attended key (left
-      // padding) re-read that key, keys behind its last attended key (tree slots that do not exist,
-      // the end of the cache) re-read that one.  Nothing outside the row's live cache rows is ever
-      // touched: the probabilities of those keys are zero, but zero times whatever lay there
-      // could be NaN
-      auto clamped = [&](int i) __attribute__((always_inline)) {
-        return (int64_t)(tile_chunk_key(ld, key0, i, key_min, key_end) - key0) * row_bytes + 16 * chunk;
-      };
-      o0 = clamped(0); o1 = clamped(1); o2 = clamped(2); o3 = clamped(3);
-    }
-    // Non-temporal loads: every K and V row is read once per launch (twice when two query tiles or
-    // grouped heads share it, back to back), so it should not push the L2's other lines out on its
-    // way through.  In the decode step this alone takes the launch from 28.8 to 27.3 us at 600 keys
-    // per row and from 85 to 70 us at 2500.
-    c0 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(tile + o0));
-    c1 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(tile + o1));
-    c2 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(tile + o2));
-    c3 = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(tile + o3));
+    const uint32_t at = (uint32_t)((int64_t)(key0 - key_min) * row_bytes) + lane_off;  // (wraps below the span)
+    const u32x4 w0 = __builtin_amdgcn_raw_buffer_load_b128(tiles, at, 0, kNonTemporal);
+    const u32x4 w1 = __builtin_amdgcn_raw_buffer_load_b128(tiles, at + step_bytes, 0, kNonTemporal);
+    const u32x4 w2 = __builtin_amdgcn_raw_buffer_load_b128(tiles, at + 2 * step_bytes, 0, kNonTemporal);
+    const u32x4 w3 = __builtin_amdgcn_raw_buffer_load_b128(tiles, at + 3 * step_bytes, 0, kNonTemporal);
+    c0 = __builtin_bit_cast(bf16x8, w0);
+    c1 = __builtin_bit_cast(bf16x8, w1);
+    c2 = __builtin_bit_cast(bf16x8, w2);
+    c3 = __builtin_bit_cast(bf16x8, w3);
   };
   auto fetch_tile = [&](auto slot_c, int j) __attribute__((always_inline)) {
     if constexpr (decltype(slot_c)::value == 0) fetch_into(a0, a1, a2, a3, j); else fetch_into(b0, b1, b2, b3, j);
@@ -1048,6 +1046,8 @@ unsigned int* arrival_slab(const char* who, size_t n, int* error) {
 bool mfma_eligible(const AttnArgs& a, int dtype) {
   auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
   auto m8 = [](int64_t s) { return (s % 8) == 0; };
+  // (the tile loads address a row's keys with 32-bit byte offsets)
+  if (a.k_ss <= 0 || a.v_ss <= 0 || !span_fits(a.kv_len, a.k_ss * 2) || !span_fits(a.kv_len, a.v_ss * 2)) return false;
   return dtype == RD_BF16 && a.D == kD && a.H <= rd::kAttnMaxHeads && al(a.q) && al(a.k) && al(a.v) && ((uintptr_t)a.out & 7) == 0 &&
          m8(a.q_sb) && m8(a.q_sh) && m8(a.q_ss) && m8(a.k_sb) && m8(a.k_sh) && m8(a.k_ss) &&
          m8(a.v_sb) && m8(a.v_sh) && m8(a.v_ss) && (a.o_sb % 4) == 0 && (a.o_sh % 4) == 0 &&

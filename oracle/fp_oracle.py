@@ -33,8 +33,11 @@ Pin status
                      attention; fully masked row == mean of V (finite-min bias)
   warp/maintain      pinned: max becomes 0, <= k survivors without ties, shift invariance
   beam_search_step   pinned on tie-free inputs: W=1 is an argmax chain; one iteration from the
-                     initial state == argsort of row 0; sets-not-order check.  With ties: parity
-                     unpinned against torch.topk's order (documented rule above instead)
+                     initial state == argsort of row 0; sets-not-order check; the reference's own
+                     beams (tests/golden/reference_vectors.json), two cases at width 64, where
+                     ties are certain after the first iteration but cannot reach the final beams.
+                     The order of tied candidates inside an iteration: parity unpinned against
+                     torch.topk's order (documented rule above instead)
 """
 
 from __future__ import annotations

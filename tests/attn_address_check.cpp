@@ -238,6 +238,7 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
   CHECK(RD_PLAN_HDR + 4 * (size_t)L.B + RD_ITEM_INTS * (size_t)L.B * max_splits <= plan_ints, "item slots beyond the plan");
   CHECK(q_tiles <= rd::attn_max_q_tiles(L.n_q) || L.n_q <= 256, "query tiles %d beyond the counters' %d", q_tiles, rd::attn_max_q_tiles(L.n_q));
   CHECK(L.H <= rd::kAttnMaxHeads, "heads %d", L.H);
+  CHECK(span_fits(L.kv_len, L.k_ss * 2), "keys %d x %lld bytes per cache row do not fit the 32-bit offsets of the tile loads", L.kv_len, (long long)L.k_ss * 2);
   for (const Item& it : items) {
     ++st.items;
     const int b = it.b, lo = it.lo, hi = it.hi;
@@ -285,9 +286,17 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
             const int key0 = tile_key0(lo, j, n_tiles);
             const int64_t w = mask_word_index(b, L.n_q, q_use, words, key0);
             CHECK(w >= 0 && w < (int64_t)L.B * L.n_q * words && (key0 >> 6) < words, "mask word %lld (row %d query %d key0 %d)", (long long)w, b, q_use, key0);
+            // K and V through the descriptor over the span's cache rows: a lane is served exactly if
+            // its key lies in the span, and then reads inside the slab
+            const int64_t row_bytes = L.k_ss * 2;
+            const uint32_t records = span_bytes(key_min, key_end, row_bytes);
             for (int i = 0; i < 4; ++i) {
-              const int key = tile_chunk_key(ld, key0, i, key_min, key_end);
-              CHECK(key >= key_min && key < key_end, "tile load of key %d outside the span [%d, %d) of row %d (item [%d, %d) tile %d thread %d)", key, key_min, key_end, b, lo, hi, j, tid);
+              const int key = tile_chunk_key(ld, key0, i);
+              const uint32_t at = tile_chunk_offset(ld, key0, i, key_min, row_bytes);
+              const bool served = chunk_in_range(at, records);
+              CHECK(served == (key >= key_min && key < key_end), "tile load of key %d (span [%d, %d) of row %d, item [%d, %d) tile %d thread %d): offset %u of %u bytes is %s", key, key_min, key_end, b, lo, hi, j, tid, at, records, served ? "served" : "refused");
+              if (!served) continue;
+              CHECK((int64_t)at == (int64_t)(key - key_min) * row_bytes + 16 * ld.chunk, "tile load offset %u of key %d", at, key);
               const int64_t row = (int64_t)key - kv_shift;
               CHECK(row >= 0 && row < L.slab_rows, "cache row %lld of %lld (row %d key %d shift %d)", (long long)row, (long long)L.slab_rows, b, key, kv_shift);
               const int64_t off = (int64_t)b * L.k_sb + (int64_t)hk * L.k_sh + row * L.k_ss + 8 * ld.chunk;
