@@ -321,7 +321,10 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
  * item that finishes last; the arrival counters for that are the library's (a ring of 2^18 per
  * GPU, of which every call takes batch * n_heads * ceil(n_q / rows per work group) for itself,
  * RD_ELIMIT beyond the ring) and leaves at zero, so calls that are in flight together do not meet
- * on a counter; each call needs a workspace of its own while it runs.
+ * on a counter; each call needs a workspace of its own while it runs.  The first MFMA-path call on
+ * a device looks the ring's address up (hipGetSymbolAddress): make it before a graph capture
+ * begins.  K and V are addressed with 32-bit byte offsets inside a batch row's slab: shapes with
+ * (kv_len + 128) * row stride in bytes >= 2^31 run on the generic kernel.
  * row_start (batch + 1 int32 on the device, or NULL): packed query rows, as in rd_rope_append:
  * query t of batch row b is row row_start[b] + t of q and of out (sequence stride; their batch
  * strides are unused), queries t >= row_start[b+1] - row_start[b] are neither read nor written.
