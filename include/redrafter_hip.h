@@ -332,8 +332,8 @@ RD_API int rd_rope_append(const void* q, const int64_t* q_strides, const void* k
  * kv_row_shift (rd_attn_prepare; batch int32 on the device, or NULL): recorded in the plan; the
  * attention then reads key column c of row b from cache row c - kv_row_shift[b] of k and v (see
  * rd_realign_plan).  Only cache rows of keys that some query of the row attends to are read (the
- * first and last 64-key tile of a row re-read its first / last such key in place of the others),
- * so nothing is asked of the memory around a row's live cache rows.
+ * other keys of the first and last 64-key tile of a row count as zeros, which their zero
+ * probabilities multiply), so nothing is asked of the memory around a row's live cache rows.
  * ------------------------------------------------------------------------------------------ */
 RD_API size_t rd_attn_plan_ints(int batch, int n_q, int kv_len);
 RD_API size_t rd_attn_bits_words(int batch, int n_q, int kv_len);

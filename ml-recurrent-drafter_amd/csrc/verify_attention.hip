@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kMfmaThreads) void attn_mfma_kernel(AttnArgs a) {
   // Tiles in flight: a ring of kRing register stages between global memory and LDS; tile j
   // passes through slot j % kRing.  The mask words travel in a ring of their own.
   // Every step issues the same loads on every path (tile indices past the end are clamped to the
-  // last tile, keys past kv_len to the last key): with loads under divergent or data-dependent
+  // last tile, keys outside the row's span read as zeros): with loads under divergent or data-dependent
   // branches the compiler can no longer count which loads are still in flight and waits for all
   // of them at every use, which would cap the ring at one tile.
   static_assert(kRing == 2, "two named register stages");
