@@ -179,9 +179,9 @@ def _rope_theta(config: LlamaConfig) -> float:
 class LlamaAttention(nn.Module):
     # False: rotation + cache append, then attention (two kernels).  None: one kernel wherever the
     # fused one applies (bf16, head_dim 128, at most 256 new tokens).  Same bits either way.  Measured
-    # on the 7B-shaped decode step the fused kernel is 6 us longer than the attention alone and saves
-    # the 12 us rotation kernel, but the step gains only 0.5 % (14.54 -> 14.46 ms), so the default
-    # keeps the two kernels, whose timings can be read one by one.
+    # on the 7B-shaped decode step the fused kernel is 10 us longer than the attention alone and saves
+    # the 10-12 us rotation kernel; the step gains between nothing and 2 % from box to box, so the
+    # default keeps the two kernels, whose timings can be read one by one.
     fused_rope_attention: Optional[bool] = False
 
     def __init__(self, config: LlamaConfig):
