@@ -293,6 +293,11 @@ void check_items(const Launch& L, const std::vector<Item>& items, int chunk, int
             for (int i = 0; i < 4; ++i) {
               const int key = tile_chunk_key(ld, key0, i);
               const uint32_t at = tile_chunk_offset(ld, key0, i, key_min, row_bytes);
+              // (the kernel forms the same number from three 32-bit parts: the tile's place relative to
+              // the span, which wraps around below it, the thread's place in a tile, the chunk's step)
+              const uint32_t in_parts = (uint32_t)((int64_t)(key0 - key_min) * row_bytes) + tile_chunk_offset(ld, 0, 0, 0, row_bytes) +
+                                        (uint32_t)i * (uint32_t)(ld.key_step * row_bytes);
+              CHECK(in_parts == at, "tile load offset of key %d: %u in parts, %u whole", key, in_parts, at);
               const bool served = chunk_in_range(at, records);
               CHECK(served == (key >= key_min && key < key_end), "tile load of key %d (span [%d, %d) of row %d, item [%d, %d) tile %d thread %d): offset %u of %u bytes is %s", key, key_min, key_end, b, lo, hi, j, tid, at, records, served ? "served" : "refused");
               if (!served) continue;
