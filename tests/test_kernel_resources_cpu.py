@@ -105,3 +105,11 @@ def test_plain_attention_kernels_load_tiles_without_per_load_loops(assembly):
         # the loop's waits are counted ones: some wait with loads still in flight exists behind the loop header
         header = next(i for i, ln in enumerate(lines) if "Loop Header" in ln)
         assert any(re.search(r"s_waitcnt vmcnt\([1-9]", ln) for ln in lines[header:header + 1200]), name
+
+
+def test_no_scalar_sign_extension_on_the_way_to_an_address(assembly):
+    """A 32-bit half of an address that is widened as a signed number (an `int` OR-ed or added into a
+    64-bit value) turns every address with bit 31 set into a wild one; in the scalar code of these
+    kernels such a widening shows as s_bfe_i64, which their address arithmetic has no other use for."""
+    for name, lines in assembly.items():
+        assert not any("s_bfe_i64" in ln for ln in lines), name
